@@ -1,0 +1,717 @@
+/*
+ * glades_oracle.c -- CPU restatement of the Glades dense feed-forward hot path.
+ * TEST INFRASTRUCTURE ONLY (see glades_oracle.h).  Plain C, fp32 arithmetic written
+ * so that the compiler can neither fuse multiply-add nor re-associate: build with
+ * -ffp-contract=off and without -ffast-math.
+ *
+ * "ML/" = "Backend/Machine Learning/" in the reference tree.
+ */
+#include "glades_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define OUTLIER 0.046f /* ML/GMath/gmath.h:35 */
+
+/* ------------------------------------------------------------------ element-wise */
+
+/* ML/GMath/gmath.cpp:22-101.  tanh/exp on a float argument resolve to the float
+ * overloads in the reference's C++ (tanhf/expf). */
+float go_squash(float z, int act, float p)
+{
+    switch (act) {
+    case GO_TANH: return tanhf(z);
+    case GO_TANHP:
+        if (z > 1.0f - p) return 1.0f;
+        if (z < p - 1.0f) return -1.0f;
+        return tanhf(z);
+    case GO_SIGMOID: return 1.0f / (1.0f + expf(-z));
+    case GO_SIGMOIDP:
+        if (z < p) return 0.01f;
+        if (z > 1.0f - p) return 0.99f;
+        return 1.0f / (1.0f + expf(-z));
+    case GO_RELU: return (z < OUTLIER) ? 0.0f : z;
+    case GO_LEAKY: return (z < OUTLIER) ? p * z : z;
+    case GO_LINEAR: return p * z;
+    case GO_STEP: return (z < p) ? 0.0f : 1.0f;
+    }
+    return 0.0f;
+}
+
+/* ML/GMath/gmath.cpp:182-245: derivative expressed in the activation's OUTPUT. */
+float go_act_der(float a, int act, float p)
+{
+    switch (act) {
+    case GO_TANH:
+    case GO_TANHP: return 1.0f - (a * a);
+    case GO_SIGMOID:
+    case GO_SIGMOIDP: return a * (1.0f - a);
+    case GO_RELU: return (a > 0.0f) ? 1.0f : 0.0f;
+    case GO_LEAKY:
+        if (a > 0.0f) return 1.0f;
+        return (p < 0) ? p : -p;
+    case GO_LINEAR: return p;
+    case GO_STEP: return 0.0f;
+    }
+    return 1.0f;
+}
+
+/* ML/GMath/gmath.cpp:272-321 */
+float go_cost(float e, float p, float data_size, int cost)
+{
+    float c = 0.0f;
+    switch (cost) {
+    case GO_REGRESSION: {
+        float d = e - p;
+        c = d * d;
+        c /= data_size;
+        break;
+    }
+    case GO_CLASSIFICATION:
+        c = -((e * logf(p)) + ((1 - e) * logf(1 - p)));
+        c /= data_size;
+        break;
+    case GO_KL:
+        c = logf(e / p);
+        c /= data_size;
+        break;
+    }
+    return c;
+}
+
+/* ML/GMath/gmath.cpp:323-353 */
+float go_cost_der(float e, float p, int cost)
+{
+    switch (cost) {
+    case GO_REGRESSION: return 2.0f * (p - e);
+    case GO_CLASSIFICATION: return (p - e) / ((1 - p) * p);
+    case GO_KL: return -(e / p);
+    }
+    return 1.0f;
+}
+
+/* ML/GMath/gmath.cpp:252-270 */
+float go_percent_error(float pred, float expect)
+{
+    float pe = pred - expect;
+    if (pe < 0.0f) pe = -pe;
+    if (pe > 1.0f) pe = 1.0f;
+    return pe;
+}
+
+/* ML/GMath/gmath.cpp:412-455: strictly-greater scan starting from max = 0 */
+int go_argmax_ref(const float* v, int n)
+{
+    float mx = 0.0f;
+    int idx = -1;
+    for (int i = 0; i < n; ++i)
+        if (v[i] > mx) { mx = v[i]; idx = i; }
+    return idx;
+}
+
+/* ------------------------------------------------------------------ init sampler */
+
+/* ML/GMath/gmath.cpp:355-405 (Acklam).  log/sqrt on float arguments are the float
+ * overloads in the reference; the rational part is evaluated in double. */
+static float norm_inv_cdf(float x)
+{
+    const double a1 = -39.69683028665376, a2 = 220.9460984245205, a3 = -275.9285104469687,
+                 a4 = 138.3577518672690, a5 = -30.66479806614716, a6 = 2.506628277459239;
+    const double b1 = -54.47609879822406, b2 = 161.5858368580409, b3 = -155.6989798598866,
+                 b4 = 66.80131188771972, b5 = -13.280681552885721;
+    const double c1 = -0.007784894002430293, c2 = -0.3223964580411365, c3 = -2.400758277161838,
+                 c4 = -2.549732539343734, c5 = 4.374664141464968, c6 = 2.938163982698783;
+    const double d1 = 0.007784695709041462, d2 = 0.3224671290700398, d3 = 2.445134137142996,
+                 d4 = 3.754408661907416;
+    float p_low = 0.02452;
+    float p_high = 1 - p_low;
+    if (x < p_low) {
+        double q = sqrtf(-2 * logf(x));
+        return (float)((((((c1 * q + c2) * q + c3) * q + c4) * q + c5) * q + c6) /
+                       ((((d1 * q + d2) * q + d3) * q + d4) * q + 1));
+    } else if (x < p_high) {
+        double q = x - 0.5;
+        double r = q * q;
+        return (float)(((((((a1 * r + a2) * r + a3) * r + a4) * r + a5) * r + a6) * q) /
+                       (((((b1 * r + b2) * r + b3) * r + b4) * r + b5) * r + 1));
+    } else {
+        double q = sqrtf(-2 * logf(1 - x));
+        return (float)(-(((((c1 * q + c2) * q + c3) * q + c4) * q + c5) * q + c6) /
+                       ((((d1 * q + d2) * q + d3) * q + d4) * q + 1));
+    }
+}
+
+/* ML/GMath/gmath.cpp:407-410 */
+static float normal_pdf(float z)
+{
+    return (float)((1 / sqrt(6.2831853)) * expf(-(z * z) / 2));
+}
+
+/* ML/State/layer.cpp:196-217 (table) + ML/State/node.cpp:241-276 (rejection loop).
+ * Both INIT_XAVIER and INIT_POSXAVIER take this path, so every weight is >= 0. */
+void go_ref_xavier_layer(int fan_in, int n_out, int act_type, float* W)
+{
+    enum { NL = 2048 };
+    static float zigg[NL + 1];
+    float cdf = 1.0;
+    for (unsigned i = 1; i < NL; i++) {
+        cdf = cdf - (1 / ((float)NL * 2));
+        zigg[i] = norm_inv_cdf(cdf);
+    }
+    zigg[0] = zigg[1];
+    zigg[NL] = 0;
+
+    float std_dev;
+    if (act_type != GO_RELU) std_dev = sqrtf(1 / (float)fan_in);
+    else std_dev = sqrtf(2 / (float)fan_in);
+
+    for (int o = 0; o < n_out; ++o)
+        for (int i = 0; i < fan_in; ++i) {
+            int accepted = 0;
+            float x = 0.0f;
+            while (!accepted) {
+                int layer = rand() % 2048;
+                x = rand() / (RAND_MAX / zigg[layer]);
+                if (layer == 0) continue;
+                else if (x < zigg[layer + 1]) accepted = 1;
+                else if (x > zigg[layer + 1]) {
+                    float randU = rand() / RAND_MAX; /* integer division, as written */
+                    float y = normal_pdf(zigg[layer]) +
+                              randU * (normal_pdf(zigg[layer - 1] - normal_pdf(zigg[layer])));
+                    if (y < normal_pdf(x)) accepted = 1;
+                }
+            }
+            W[(size_t)o * fan_in + i] = x * std_dev;
+        }
+}
+
+/* ------------------------------------------------------------------ exact mode */
+
+struct go_exact {
+    go_spec s;
+    float* W[GO_MAX_LAYERS];     /* [n_out][n_in] row-major: the incoming edges of node o */
+    float* wsum[GO_MAX_LAYERS];  /* running sum of the edge's pending deltas (edge.cpp window) */
+    float* wlast[GO_MAX_LAYERS]; /* last pending delta, 0 when the window is empty */
+    float  bias[GO_MAX_LAYERS];  /* scalar bias of layer l, added to layer l+1 (l >= 1) */
+    float* a[GO_MAX_LAYERS + 1]; /* node values */
+    float* e[GO_MAX_LAYERS + 1]; /* node error accumulators */
+};
+
+go_exact* go_exact_create(const go_spec* spec)
+{
+    go_exact* n = (go_exact*)calloc(1, sizeof(go_exact));
+    n->s = *spec;
+    for (int l = 0; l < spec->n_layers; ++l) {
+        size_t cnt = (size_t)spec->sizes[l] * spec->sizes[l + 1];
+        n->W[l] = (float*)calloc(cnt, sizeof(float));
+        n->wsum[l] = (float*)calloc(cnt, sizeof(float));
+        n->wlast[l] = (float*)calloc(cnt, sizeof(float));
+    }
+    for (int l = 0; l <= spec->n_layers; ++l) {
+        n->a[l] = (float*)calloc(spec->sizes[l], sizeof(float));
+        n->e[l] = (float*)calloc(spec->sizes[l], sizeof(float));
+    }
+    return n;
+}
+
+void go_exact_destroy(go_exact* n)
+{
+    if (!n) return;
+    for (int l = 0; l < n->s.n_layers; ++l) { free(n->W[l]); free(n->wsum[l]); free(n->wlast[l]); }
+    for (int l = 0; l <= n->s.n_layers; ++l) { free(n->a[l]); free(n->e[l]); }
+    free(n);
+}
+
+void go_exact_set_weights(go_exact* n, int l, const float* W)
+{ memcpy(n->W[l], W, sizeof(float) * n->s.sizes[l] * n->s.sizes[l + 1]); }
+void go_exact_get_weights(const go_exact* n, int l, float* W)
+{ memcpy(W, n->W[l], sizeof(float) * n->s.sizes[l] * n->s.sizes[l + 1]); }
+void go_exact_set_bias(go_exact* n, int l, float b) { n->bias[l] = b; }
+float go_exact_get_bias(const go_exact* n, int l) { return n->bias[l]; }
+void go_exact_get_window(const go_exact* n, int l, float* sum, float* last)
+{
+    size_t cnt = (size_t)n->s.sizes[l] * n->s.sizes[l + 1];
+    memcpy(sum, n->wsum[l], cnt * sizeof(float));
+    memcpy(last, n->wlast[l], cnt * sizeof(float));
+}
+
+/* network.cpp:457-575 for one row (no dropout). */
+static void exact_forward(go_exact* n, const float* x, const float* y, int64_t N,
+                          float* tot_err, float* tot_acc)
+{
+    const go_spec* s = &n->s;
+    const int H1 = s->n_layers;
+    memcpy(n->a[0], x, sizeof(float) * s->sizes[0]);
+    for (int l = 0; l < H1; ++l) {
+        const int ni = s->sizes[l], no = s->sizes[l + 1];
+        const float* W = n->W[l];
+        for (int o = 0; o < no; ++o) {
+            float z = 0.0f; /* node.cpp:82-93: sum of edge activations, i ascending */
+            for (int i = 0; i < ni; ++i) {
+                float ea = W[(size_t)o * ni + i] * n->a[l][i]; /* network.cpp:485-487 */
+                z += ea;
+            }
+            if (l != 0) z += n->bias[l]; /* network.cpp:501-502 */
+            n->a[l + 1][o] = go_squash(z, s->act[l], s->act_param[l]);
+            if (l == H1 - 1) { /* network.cpp:519-559 */
+                float pred = n->a[l + 1][o], expect = y[o];
+                float data_size = (float)((unsigned)N * (unsigned)no);
+                float c = go_cost(expect, pred, data_size, s->cost);
+                *tot_err += c;
+                float acc = (1.0f - go_percent_error(pred, expect)) * 100.0f;
+                if (acc < 0.0f) acc = 0.0f;
+                *tot_acc += acc;
+            }
+        }
+    }
+}
+
+/* network.cpp:577-668 for one row `r` (no dropout); node.cpp:278-307 inlined. */
+static void exact_backward(go_exact* n, const float* y, int64_t r)
+{
+    const go_spec* s = &n->s;
+    const int H1 = s->n_layers;
+    const int mb = s->batch;
+    for (int L = H1; L > 0; --L) {
+        const int l = L - 1; /* weight layer; hyper-parameter row of the in-layer */
+        const int ni = s->sizes[l], no = s->sizes[L];
+        float* W = n->W[l];
+        float* ws = n->wsum[l];
+        float* wl = n->wlast[l];
+        const float lr = s->lr[l], mom = s->mom[l], wd1 = s->wd1[l], wd2 = s->wd2[l];
+        for (int i = 0; i < ni; ++i) {
+            const float ain = n->a[l][i];
+            for (int o = 0; o < no; ++o) {
+                float der = 1.0f;
+                if (L == H1) { /* output layer: clearErrDer + adjustErrDer(costErrDer) */
+                    n->e[L][o] = 0;
+                    n->e[L][o] += go_cost_der(y[o], n->a[L][o], s->cost);
+                } else {
+                    der = go_act_der(n->a[L][o], s->act[l], 0.01f); /* network.cpp:616-618 */
+                }
+                float d = n->e[L][o];
+                d *= der;
+                if (i == ni - 1) n->e[L][o] = 0;
+                float base = lr * d;
+                size_t k = (size_t)o * ni + i;
+                /* node.cpp:285-288 */
+                float dW = ((base * ain) + (mom * wl[k]) + (wd1 * lr * fabsf(ain)) +
+                            (wd2 * lr * ain));
+                ws[k] += dW; /* same order as node.cpp:299-301 summing the window from 0 */
+                wl[k] = dW;
+                if ((r % mb) == 0) { /* network.cpp:647-651 */
+                    float dsum = ws[k];
+                    dsum /= mb;
+                    W[k] = W[k] - dsum;
+                    ws[k] = 0.0f;
+                    wl[k] = 0.0f;
+                }
+                if (l != 0) n->bias[l] = n->bias[l] - base; /* network.cpp:654-656 */
+                /* network.cpp:660-662 + node.cpp:173-176 */
+                float cin = n->e[l][i] + (d * W[k]);
+                n->e[l][i] += cin;
+            }
+        }
+    }
+    /* the accumulators of the row's own input nodes are never read again */
+    memset(n->e[0], 0, sizeof(float) * s->sizes[0]);
+}
+
+void go_exact_epoch(go_exact* n, const float* X, const float* Y, int64_t N, int train,
+                    go_metrics* m, float* preds)
+{
+    const go_spec* s = &n->s;
+    const int nf = s->sizes[0], no = s->sizes[s->n_layers];
+    float tot_err = 0.0f, tot_acc = 0.0f;
+    int64_t correct = 0;
+    for (int64_t r = 0; r < N; ++r) {
+        const float* x = X + r * nf;
+        const float* y = Y + r * no;
+        exact_forward(n, x, y, N, &tot_err, &tot_acc);
+        const float* p = n->a[s->n_layers];
+        if (preds) memcpy(preds + r * no, p, sizeof(float) * no);
+        if (go_argmax_ref(p, no) == go_argmax_ref(y, no)) ++correct;
+        if (train) exact_backward(n, y, r);
+    }
+    tot_acc /= ((float)(unsigned)N) * ((float)(unsigned)no); /* network.cpp:194-195 */
+    if (m) { m->loss = tot_err; m->accuracy = tot_acc; m->correct = correct; }
+}
+
+/* ------------------------------------------------------------------ canonical mode */
+
+static int g_threads = 1;
+void go_set_threads(int t) { g_threads = t > 0 ? t : 1; }
+
+struct go_canon {
+    go_spec s;
+    float* W[GO_MAX_LAYERS];  float* b[GO_MAX_LAYERS];
+    float* vW[GO_MAX_LAYERS]; float* vb[GO_MAX_LAYERS]; /* previous step's applied delta */
+    float* gW[GO_MAX_LAYERS]; float* gb[GO_MAX_LAYERS];
+    float* a[GO_MAX_LAYERS + 1]; /* [B][n] activations */
+    float* d[GO_MAX_LAYERS + 1]; /* [B][n] deltas (dL/dz) */
+    int64_t cap;
+};
+
+go_canon* go_canon_create(const go_spec* spec)
+{
+    go_canon* n = (go_canon*)calloc(1, sizeof(go_canon));
+    n->s = *spec;
+    for (int l = 0; l < spec->n_layers; ++l) {
+        size_t cnt = (size_t)spec->sizes[l] * spec->sizes[l + 1];
+        n->W[l] = (float*)calloc(cnt, 4); n->vW[l] = (float*)calloc(cnt, 4);
+        n->gW[l] = (float*)calloc(cnt, 4);
+        n->b[l] = (float*)calloc(spec->sizes[l + 1], 4);
+        n->vb[l] = (float*)calloc(spec->sizes[l + 1], 4);
+        n->gb[l] = (float*)calloc(spec->sizes[l + 1], 4);
+    }
+    return n;
+}
+
+static void canon_free_acts(go_canon* n)
+{
+    for (int l = 0; l <= n->s.n_layers; ++l) { free(n->a[l]); free(n->d[l]); n->a[l] = n->d[l] = 0; }
+    n->cap = 0;
+}
+
+void go_canon_destroy(go_canon* n)
+{
+    if (!n) return;
+    canon_free_acts(n);
+    for (int l = 0; l < n->s.n_layers; ++l) {
+        free(n->W[l]); free(n->vW[l]); free(n->gW[l]); free(n->b[l]); free(n->vb[l]); free(n->gb[l]);
+    }
+    free(n);
+}
+
+static void canon_reserve(go_canon* n, int64_t B)
+{
+    if (B <= n->cap) return;
+    canon_free_acts(n);
+    for (int l = 0; l <= n->s.n_layers; ++l) {
+        n->a[l] = (float*)malloc(sizeof(float) * B * n->s.sizes[l]);
+        n->d[l] = (float*)malloc(sizeof(float) * B * n->s.sizes[l]);
+    }
+    n->cap = B;
+}
+
+void go_canon_set_params(go_canon* n, int l, const float* W, const float* bias)
+{
+    size_t cnt = (size_t)n->s.sizes[l] * n->s.sizes[l + 1];
+    memcpy(n->W[l], W, cnt * 4);
+    if (bias) memcpy(n->b[l], bias, 4 * n->s.sizes[l + 1]);
+    else memset(n->b[l], 0, 4 * n->s.sizes[l + 1]);
+}
+void go_canon_get_params(const go_canon* n, int l, float* W, float* bias)
+{
+    if (W) memcpy(W, n->W[l], 4 * (size_t)n->s.sizes[l] * n->s.sizes[l + 1]);
+    if (bias) memcpy(bias, n->b[l], 4 * n->s.sizes[l + 1]);
+}
+void go_canon_get_momentum(const go_canon* n, int l, float* vW, float* vb)
+{
+    if (vW) memcpy(vW, n->vW[l], 4 * (size_t)n->s.sizes[l] * n->s.sizes[l + 1]);
+    if (vb) memcpy(vb, n->vb[l], 4 * n->s.sizes[l + 1]);
+}
+void go_canon_get_grads(const go_canon* n, int l, float* gW, float* gb)
+{
+    if (gW) memcpy(gW, n->gW[l], 4 * (size_t)n->s.sizes[l] * n->s.sizes[l + 1]);
+    if (gb) memcpy(gb, n->gb[l], 4 * n->s.sizes[l + 1]);
+}
+
+#define TB 16 /* batch rows handled together so the inner loop vectorises without re-association */
+
+/* z[b][o] = sum_i W[o][i]*a[b][i] (i ascending, product rounded before the add) + bias[o] */
+__attribute__((target_clones("avx2", "default")))
+static void canon_layer_forward(const float* W, const float* bias, const float* A, float* Z,
+                                int64_t B, int ni, int no)
+{
+    int64_t nblk = (B + TB - 1) / TB;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t blk = 0; blk < nblk; ++blk) {
+        int64_t b0 = blk * TB;
+        int nb = (int)((B - b0) < TB ? (B - b0) : TB);
+        float* At = (float*)malloc(sizeof(float) * (size_t)ni * TB);
+        for (int i = 0; i < ni; ++i)
+            for (int t = 0; t < TB; ++t) At[(size_t)i * TB + t] = (t < nb) ? A[(b0 + t) * ni + i] : 0.0f;
+        for (int o = 0; o < no; ++o) {
+            float acc[TB];
+            for (int t = 0; t < TB; ++t) acc[t] = 0.0f;
+            const float* w = W + (size_t)o * ni;
+            for (int i = 0; i < ni; ++i) {
+                const float wi = w[i];
+                const float* at = At + (size_t)i * TB;
+                for (int t = 0; t < TB; ++t) { float pr = wi * at[t]; acc[t] += pr; }
+            }
+            const float bo = bias[o];
+            for (int t = 0; t < nb; ++t) Z[(b0 + t) * no + o] = acc[t] + bo;
+        }
+        free(At);
+    }
+}
+
+static void canon_activate(const go_spec* s, int l, float* Z, int64_t B)
+{
+    const int no = s->sizes[l + 1];
+    const int act = s->act[l];
+    const float p = s->act_param[l];
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t b = 0; b < B; ++b) {
+        float* z = Z + b * no;
+        if (act == GO_SOFTMAX) {
+            float mx = z[0];
+            for (int o = 1; o < no; ++o) if (z[o] > mx) mx = z[o];
+            float sum = 0.0f;
+            for (int o = 0; o < no; ++o) { z[o] = expf(z[o] - mx); sum += z[o]; }
+            for (int o = 0; o < no; ++o) z[o] = z[o] / sum;
+        } else {
+            for (int o = 0; o < no; ++o) z[o] = go_squash(z[o], act, p);
+        }
+    }
+}
+
+static void canon_forward_all(go_canon* n, const float* X, int64_t B)
+{
+    const go_spec* s = &n->s;
+    canon_reserve(n, B);
+    memcpy(n->a[0], X, sizeof(float) * B * s->sizes[0]);
+    for (int l = 0; l < s->n_layers; ++l) {
+        canon_layer_forward(n->W[l], n->b[l], n->a[l], n->a[l + 1], B, s->sizes[l], s->sizes[l + 1]);
+        canon_activate(s, l, n->a[l + 1], B);
+    }
+}
+
+void go_canon_forward(go_canon* n, const float* X, int64_t B, float* out)
+{
+    canon_forward_all(n, X, B);
+    memcpy(out, n->a[n->s.n_layers], sizeof(float) * B * n->s.sizes[n->s.n_layers]);
+}
+
+/* canonical derivative: the reference's output-expressed forms with the layer's own
+ * parameter (LEAKY slope = +param). */
+static inline float canon_act_der(float a, int act, float p)
+{
+    if (act == GO_LEAKY) return (a > 0.0f) ? 1.0f : p;
+    return go_act_der(a, act, p);
+}
+
+/* per-sample loss = sum over outputs (no 1/data_size); delta = dLoss/dz */
+static double canon_output_delta(const go_spec* s, const float* P, const float* Y, float* D,
+                                 int64_t B, go_metrics* m)
+{
+    const int L = s->n_layers, no = s->sizes[L];
+    const int act = s->act[L - 1];
+    const float par = s->act_param[L - 1];
+    double loss = 0.0, acc = 0.0;
+    int64_t correct = 0;
+    for (int64_t b = 0; b < B; ++b) {
+        const float* p = P + b * no;
+        const float* y = Y + b * no;
+        float* d = D ? D + b * no : 0;
+        for (int o = 0; o < no; ++o) {
+            float c;
+            if (act == GO_SOFTMAX) c = -(y[o] * logf(p[o] > 1e-30f ? p[o] : 1e-30f));
+            else c = go_cost(y[o], p[o], 1.0f, s->cost);
+            if (!(act == GO_SOFTMAX && y[o] == 0.0f)) loss += c;
+            if (d) {
+                if (act == GO_SOFTMAX ||
+                    ((act == GO_SIGMOID || act == GO_SIGMOIDP) && s->cost == GO_CLASSIFICATION))
+                    d[o] = p[o] - y[o];
+                else
+                    d[o] = go_cost_der(y[o], p[o], s->cost) * canon_act_der(p[o], act, par);
+            }
+            float a = (1.0f - go_percent_error(p[o], y[o])) * 100.0f;
+            if (a < 0.0f) a = 0.0f;
+            acc += a;
+        }
+        if (go_argmax_ref(p, no) == go_argmax_ref(y, no)) ++correct;
+    }
+    if (m) {
+        m->loss = (float)(loss / (double)B);
+        m->accuracy = (float)(acc / ((double)B * no));
+        m->correct = correct;
+    }
+    return loss / (double)B;
+}
+
+double go_canon_loss(go_canon* n, const float* X, const float* Y, int64_t B)
+{
+    canon_forward_all(n, X, B);
+    return canon_output_delta(&n->s, n->a[n->s.n_layers], Y, 0, B, 0);
+}
+
+/* E[b][i] = sum_o D[b][o]*W[o][i] (o ascending) */
+__attribute__((target_clones("avx2", "default")))
+static void canon_dgrad(const float* W, const float* D, float* E, int64_t B, int ni, int no)
+{
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t b = 0; b < B; ++b) {
+        float* e = E + b * ni;
+        for (int i = 0; i < ni; ++i) e[i] = 0.0f;
+        for (int o = 0; o < no; ++o) {
+            const float dv = D[b * no + o];
+            const float* w = W + (size_t)o * ni;
+            for (int i = 0; i < ni; ++i) { float pr = dv * w[i]; e[i] += pr; }
+        }
+    }
+}
+
+/* G[o][i] = (sum_b D[b][o]*A[b][i]) / B  (b ascending);  gb[o] = (sum_b D[b][o]) / B */
+__attribute__((target_clones("avx2", "default")))
+static void canon_wgrad(const float* D, const float* A, float* G, float* gb, int64_t B, int ni, int no)
+{
+    const float invB = 1.0f / (float)B;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int o = 0; o < no; ++o) {
+        float* g = G + (size_t)o * ni;
+        for (int i = 0; i < ni; ++i) g[i] = 0.0f;
+        float sb = 0.0f;
+        for (int64_t b = 0; b < B; ++b) {
+            const float dv = D[b * no + o];
+            const float* a = A + b * ni;
+            for (int i = 0; i < ni; ++i) { float pr = dv * a[i]; g[i] += pr; }
+            sb += dv;
+        }
+        for (int i = 0; i < ni; ++i) g[i] = g[i] * invB;
+        gb[o] = sb * invB;
+    }
+}
+
+static inline float sgnf(float w) { return (w > 0.0f) ? 1.0f : ((w < 0.0f) ? -1.0f : 0.0f); }
+
+void go_canon_step(go_canon* n, const float* X, const float* Y, int64_t B, go_metrics* m)
+{
+    const go_spec* s = &n->s;
+    const int L = s->n_layers;
+    canon_forward_all(n, X, B);
+    canon_output_delta(s, n->a[L], Y, n->d[L], B, m);
+    for (int l = L - 1; l >= 0; --l) {
+        const int ni = s->sizes[l], no = s->sizes[l + 1];
+        canon_wgrad(n->d[l + 1], n->a[l], n->gW[l], n->gb[l], B, ni, no);
+        if (l > 0) { /* uses the pre-update weights */
+            canon_dgrad(n->W[l], n->d[l + 1], n->d[l], B, ni, no);
+            const int act = s->act[l - 1];
+            const float par = s->act_param[l - 1];
+            float* d = n->d[l];
+            const float* a = n->a[l];
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+            for (int64_t k = 0; k < B * ni; ++k) d[k] = d[k] * canon_act_der(a[k], act, par);
+        }
+        /* delta_t = lr*(g + wd1*sign(W) + wd2*W) + mom*delta_{t-1};  W -= delta_t */
+        const float lr = s->lr[l], mom = s->mom[l], wd1 = s->wd1[l], wd2 = s->wd2[l];
+        float* W = n->W[l]; float* vW = n->vW[l]; const float* gW = n->gW[l];
+        const int64_t cnt = (int64_t)ni * no;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+        for (int64_t k = 0; k < cnt; ++k) {
+            float g = gW[k] + wd1 * sgnf(W[k]) + wd2 * W[k];
+            float dl = lr * g + mom * vW[k];
+            vW[k] = dl;
+            W[k] = W[k] - dl;
+        }
+        for (int o = 0; o < no; ++o) { /* biases: momentum, no decay */
+            float dl = lr * n->gb[l][o] + mom * n->vb[l][o];
+            n->vb[l][o] = dl;
+            n->b[l][o] = n->b[l][o] - dl;
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ low precision */
+
+static inline uint32_t f2u(float x) { uint32_t u; memcpy(&u, &x, 4); return u; }
+static inline float u2f(uint32_t u) { float x; memcpy(&x, &u, 4); return x; }
+
+uint16_t go_bf16_from_f32(float x)
+{
+    uint32_t u = f2u(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40); /* quiet NaN */
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+float go_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* OCP FP8 E4M3 (finite-only variant: bias 7, max 448, 0x7f = NaN) */
+float go_e4m3_to_f32(uint8_t b)
+{
+    int sign = b >> 7, e = (b >> 3) & 0xf, mnt = b & 7;
+    float v;
+    if (e == 0xf && mnt == 7) return NAN;
+    if (e == 0) v = ldexpf((float)mnt, -9);
+    else v = ldexpf(1.0f + (float)mnt / 8.0f, e - 7);
+    return sign ? -v : v;
+}
+
+uint8_t go_e4m3_from_f32(float x)
+{
+    uint8_t sign = (uint8_t)((f2u(x) >> 31) << 7);
+    float a = fabsf(x);
+    if (a != a) return (uint8_t)(sign | 0x7f);
+    if (a >= 448.0f) return (uint8_t)(sign | 0x7e); /* saturate */
+    if (a < 0.015625f) { /* below the smallest normal 2^-6: multiples of 2^-9 */
+        int q = (int)rintf(a * 512.0f);
+        return (uint8_t)(sign | q); /* q == 8 is exactly the smallest normal's code */
+    }
+    int ex;
+    float fr = frexpf(a, &ex); /* a = fr * 2^ex, fr in [0.5,1) */
+    float mant = fr * 2.0f;    /* [1,2) */
+    ex -= 1;
+    int q = (int)rintf((mant - 1.0f) * 8.0f); /* ties to even */
+    if (q == 8) { q = 0; ex += 1; }
+    int code = ((ex + 7) << 3) | q;
+    if (code > 0x7e) code = 0x7e;
+    return (uint8_t)(sign | code);
+}
+
+void go_e4m3_quant_rows(const float* x, int64_t rows, int64_t cols, uint8_t* q, float* scale)
+{
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t r = 0; r < rows; ++r) {
+        const float* xr = x + r * cols;
+        float amax = 0.0f;
+        for (int64_t c = 0; c < cols; ++c) { float a = fabsf(xr[c]); if (a > amax) amax = a; }
+        float sc = (amax > 0.0f) ? amax / 448.0f : 1.0f;
+        scale[r] = sc;
+        for (int64_t c = 0; c < cols; ++c) q[r * cols + c] = go_e4m3_from_f32(xr[c] / sc);
+    }
+}
+
+void go_fp8_forward(const go_spec* s, const uint8_t* const* Wq, const float* const* wscale,
+                    const float* X, int64_t B, float* out)
+{
+    static float lut[256];
+    for (int i = 0; i < 256; ++i) lut[i] = go_e4m3_to_f32((uint8_t)i);
+    int maxw = 0;
+    for (int l = 0; l <= s->n_layers; ++l) if (s->sizes[l] > maxw) maxw = s->sizes[l];
+    float* cur = (float*)malloc(sizeof(float) * B * maxw);
+    float* nxt = (float*)malloc(sizeof(float) * B * maxw);
+    uint8_t* q = (uint8_t*)malloc((size_t)B * maxw);
+    float* xs = (float*)malloc(sizeof(float) * B);
+    memcpy(cur, X, sizeof(float) * B * s->sizes[0]);
+    for (int l = 0; l < s->n_layers; ++l) {
+        const int ni = s->sizes[l], no = s->sizes[l + 1];
+        go_e4m3_quant_rows(cur, B, ni, q, xs);
+        float* wf = (float*)malloc(sizeof(float) * (size_t)ni * no);
+        for (size_t k = 0; k < (size_t)ni * no; ++k) wf[k] = lut[Wq[l][k]];
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+        for (int64_t b = 0; b < B; ++b) {
+            float* xf = (float*)malloc(sizeof(float) * ni);
+            for (int i = 0; i < ni; ++i) xf[i] = lut[q[b * ni + i]];
+            for (int o = 0; o < no; ++o) {
+                const float* w = wf + (size_t)o * ni;
+                float acc = 0.0f;
+                for (int i = 0; i < ni; ++i) { float pr = w[i] * xf[i]; acc += pr; }
+                float v = acc * (xs[b] * wscale[l][o]);
+                v = go_squash(v, s->act[l], s->act_param[l]);
+                if (l + 1 < s->n_layers) v = go_bf16_to_f32(go_bf16_from_f32(v));
+                nxt[b * no + o] = v;
+            }
+            free(xf);
+        }
+        free(wf);
+        float* t = cur; cur = nxt; nxt = t;
+    }
+    memcpy(out, cur, sizeof(float) * B * s->sizes[s->n_layers]);
+    free(cur); free(nxt); free(q); free(xs);
+}

@@ -1,0 +1,313 @@
+"""ctypes view of oracle/libglades_oracle.so (the CPU restatement).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the CPU-baseline
+leg of bench.py -- never by the product package.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libglades_oracle.so")
+REF_HARNESS = os.path.join(HERE, "_ref", "ref_harness")
+MAX_LAYERS = 16
+
+TANH, TANHP, SIGMOID, SIGMOIDP, LINEAR, RELU, LEAKY, STEP, SOFTMAX = range(9)
+REGRESSION, CLASSIFICATION, KL = range(3)
+
+
+class Spec(C.Structure):
+    _fields_ = [
+        ("n_layers", C.c_int),
+        ("sizes", C.c_int * (MAX_LAYERS + 1)),
+        ("lr", C.c_float * MAX_LAYERS),
+        ("mom", C.c_float * MAX_LAYERS),
+        ("wd1", C.c_float * MAX_LAYERS),
+        ("wd2", C.c_float * MAX_LAYERS),
+        ("act", C.c_int * MAX_LAYERS),
+        ("act_param", C.c_float * MAX_LAYERS),
+        ("batch", C.c_int),
+        ("cost", C.c_int),
+    ]
+
+
+class Metrics(C.Structure):
+    _fields_ = [("loss", C.c_float), ("accuracy", C.c_float), ("correct", C.c_int64)]
+
+
+def build(force=False):
+    """Compile the C restatement (and the reference harness when the reference tree exists)."""
+    if force or not os.path.exists(LIB_PATH):
+        subprocess.check_call(["make", "-C", HERE, "-B", "libglades_oracle.so"])
+    if os.path.isdir("/root/reference") and (force or not os.path.exists(REF_HARNESS)):
+        subprocess.check_call(["make", "-C", HERE, "-B", "ref"])
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            build()
+        L = C.CDLL(LIB_PATH)
+        f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+        u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
+        vp = C.c_void_p
+        sig = {
+            "go_squash": (C.c_float, [C.c_float, C.c_int, C.c_float]),
+            "go_act_der": (C.c_float, [C.c_float, C.c_int, C.c_float]),
+            "go_cost": (C.c_float, [C.c_float, C.c_float, C.c_float, C.c_int]),
+            "go_cost_der": (C.c_float, [C.c_float, C.c_float, C.c_int]),
+            "go_percent_error": (C.c_float, [C.c_float, C.c_float]),
+            "go_argmax_ref": (C.c_int, [f32p, C.c_int]),
+            "go_ref_xavier_layer": (None, [C.c_int, C.c_int, C.c_int, f32p]),
+            "go_exact_create": (vp, [C.POINTER(Spec)]),
+            "go_exact_destroy": (None, [vp]),
+            "go_exact_set_weights": (None, [vp, C.c_int, f32p]),
+            "go_exact_get_weights": (None, [vp, C.c_int, f32p]),
+            "go_exact_set_bias": (None, [vp, C.c_int, C.c_float]),
+            "go_exact_get_bias": (C.c_float, [vp, C.c_int]),
+            "go_exact_get_window": (None, [vp, C.c_int, f32p, f32p]),
+            "go_exact_epoch": (None, [vp, f32p, f32p, C.c_int64, C.c_int, C.POINTER(Metrics), vp]),
+            "go_canon_create": (vp, [C.POINTER(Spec)]),
+            "go_canon_destroy": (None, [vp]),
+            "go_canon_set_params": (None, [vp, C.c_int, f32p, vp]),
+            "go_canon_get_params": (None, [vp, C.c_int, vp, vp]),
+            "go_canon_get_momentum": (None, [vp, C.c_int, vp, vp]),
+            "go_canon_get_grads": (None, [vp, C.c_int, vp, vp]),
+            "go_canon_forward": (None, [vp, f32p, C.c_int64, f32p]),
+            "go_canon_step": (None, [vp, f32p, f32p, C.c_int64, C.POINTER(Metrics)]),
+            "go_canon_loss": (C.c_double, [vp, f32p, f32p, C.c_int64]),
+            "go_set_threads": (None, [C.c_int]),
+            "go_bf16_from_f32": (C.c_uint16, [C.c_float]),
+            "go_bf16_to_f32": (C.c_float, [C.c_uint16]),
+            "go_e4m3_from_f32": (C.c_uint8, [C.c_float]),
+            "go_e4m3_to_f32": (C.c_float, [C.c_uint8]),
+            "go_e4m3_quant_rows": (None, [f32p, C.c_int64, C.c_int64, u8p, f32p]),
+            "go_fp8_forward": (None, [C.POINTER(Spec), C.POINTER(vp), C.POINTER(vp), f32p, C.c_int64, f32p]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def make_spec(sizes, acts, lr=0.01, mom=0.0, wd1=0.0, wd2=0.0, act_params=0.0, batch=1,
+              cost=REGRESSION):
+    """sizes: n_layers+1 ints; the per-layer arguments are scalars or lists of n_layers."""
+    nl = len(sizes) - 1
+    assert 1 <= nl <= MAX_LAYERS
+
+    def per(v):
+        return list(v) if isinstance(v, (list, tuple, np.ndarray)) else [v] * nl
+
+    s = Spec()
+    s.n_layers = nl
+    for i, v in enumerate(sizes):
+        s.sizes[i] = int(v)
+    for name, v in (("lr", lr), ("mom", mom), ("wd1", wd1), ("wd2", wd2), ("act_param", act_params)):
+        arr = getattr(s, name)
+        for i, x in enumerate(per(v)):
+            arr[i] = float(x)
+    for i, a in enumerate(per(acts)):
+        s.act[i] = int(a)
+    s.batch = int(batch)
+    s.cost = int(cost)
+    return s
+
+
+def _vp(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+class ExactNet:
+    """Reference semantics: sequential rows, scalar layer bias, delta windows."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.sizes = [spec.sizes[i] for i in range(spec.n_layers + 1)]
+        self.h = lib().go_exact_create(C.byref(spec))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().go_exact_destroy(self.h)
+            self.h = None
+
+    def set_weights(self, l, W):
+        W = np.ascontiguousarray(W, np.float32)
+        assert W.shape == (self.sizes[l + 1], self.sizes[l])
+        lib().go_exact_set_weights(self.h, l, W)
+
+    def get_weights(self, l):
+        W = np.empty((self.sizes[l + 1], self.sizes[l]), np.float32)
+        lib().go_exact_get_weights(self.h, l, W)
+        return W
+
+    def set_bias(self, l, b):
+        lib().go_exact_set_bias(self.h, l, float(b))
+
+    def get_bias(self, l):
+        return np.float32(lib().go_exact_get_bias(self.h, l))
+
+    def get_window(self, l):
+        s = np.empty((self.sizes[l + 1], self.sizes[l]), np.float32)
+        t = np.empty_like(s)
+        lib().go_exact_get_window(self.h, l, s, t)
+        return s, t
+
+    def epoch(self, X, Y, train=True, want_preds=True):
+        X = np.ascontiguousarray(X, np.float32)
+        Y = np.ascontiguousarray(Y, np.float32)
+        N = X.shape[0]
+        assert X.shape == (N, self.sizes[0]) and Y.shape == (N, self.sizes[-1])
+        preds = np.empty((N, self.sizes[-1]), np.float32) if want_preds else None
+        m = Metrics()
+        lib().go_exact_epoch(self.h, X, Y, N, 1 if train else 0, C.byref(m), _vp(preds))
+        return m, preds
+
+
+class CanonNet:
+    """Batched textbook training; forward identical to the reference forward."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.sizes = [spec.sizes[i] for i in range(spec.n_layers + 1)]
+        self.h = lib().go_canon_create(C.byref(spec))
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            lib().go_canon_destroy(self.h)
+            self.h = None
+
+    def set_params(self, l, W, b=None):
+        W = np.ascontiguousarray(W, np.float32)
+        assert W.shape == (self.sizes[l + 1], self.sizes[l])
+        if b is not None:
+            b = np.ascontiguousarray(b, np.float32)
+            assert b.shape == (self.sizes[l + 1],)
+        lib().go_canon_set_params(self.h, l, W, _vp(b))
+
+    def _pair(self, fn, l):
+        W = np.empty((self.sizes[l + 1], self.sizes[l]), np.float32)
+        b = np.empty((self.sizes[l + 1],), np.float32)
+        fn(self.h, l, _vp(W), _vp(b))
+        return W, b
+
+    def get_params(self, l):
+        return self._pair(lib().go_canon_get_params, l)
+
+    def get_momentum(self, l):
+        return self._pair(lib().go_canon_get_momentum, l)
+
+    def get_grads(self, l):
+        return self._pair(lib().go_canon_get_grads, l)
+
+    def forward(self, X):
+        X = np.ascontiguousarray(X, np.float32)
+        out = np.empty((X.shape[0], self.sizes[-1]), np.float32)
+        lib().go_canon_forward(self.h, X, X.shape[0], out)
+        return out
+
+    def step(self, X, Y):
+        X = np.ascontiguousarray(X, np.float32)
+        Y = np.ascontiguousarray(Y, np.float32)
+        m = Metrics()
+        lib().go_canon_step(self.h, X, Y, X.shape[0], C.byref(m))
+        return m
+
+    def loss(self, X, Y):
+        X = np.ascontiguousarray(X, np.float32)
+        Y = np.ascontiguousarray(Y, np.float32)
+        return lib().go_canon_loss(self.h, X, Y, X.shape[0])
+
+
+def bf16_round(x):
+    """fp32 array -> fp32 array holding the bf16-rounded values (RNE)."""
+    x = np.ascontiguousarray(x, np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return r.astype(np.uint32).view(np.float32).reshape(x.shape)
+
+
+def e4m3_quant_rows(x):
+    x = np.ascontiguousarray(x, np.float32)
+    q = np.empty(x.shape, np.uint8)
+    s = np.empty((x.shape[0],), np.float32)
+    lib().go_e4m3_quant_rows(x, x.shape[0], x.shape[1], q, s)
+    return q, s
+
+
+def e4m3_table():
+    return np.array([lib().go_e4m3_to_f32(i) for i in range(256)], np.float32)
+
+
+def fp8_forward(spec, Wq, wscale, X):
+    nl = spec.n_layers
+    X = np.ascontiguousarray(X, np.float32)
+    Wq = [np.ascontiguousarray(w, np.uint8) for w in Wq]
+    wscale = [np.ascontiguousarray(s, np.float32) for s in wscale]
+    wp = (C.c_void_p * nl)(*[w.ctypes.data for w in Wq])
+    sp = (C.c_void_p * nl)(*[s.ctypes.data for s in wscale])
+    out = np.empty((X.shape[0], spec.sizes[nl]), np.float32)
+    lib().go_fp8_forward(C.byref(spec), wp, sp, X, X.shape[0], out)
+    return out
+
+
+# ---------------------------------------------------------------- reference harness
+
+
+def have_ref():
+    return os.path.exists(REF_HARNESS)
+
+
+def ref_train(spec, weights, biases, X, Y, epochs, tmpdir):
+    """Run the harness built from the reference's compiled objects.  Returns a dict with
+    per-epoch (loss, accuracy), final weights, biases, last-epoch predictions and windows."""
+    nl = spec.n_layers
+    sizes = [spec.sizes[i] for i in range(nl + 1)]
+    X = np.ascontiguousarray(X, np.float32)
+    Y = np.ascontiguousarray(Y, np.float32)
+    N = X.shape[0]
+    cin = os.path.join(tmpdir, "case.bin")
+    cout = os.path.join(tmpdir, "out.bin")
+    with open(cin, "wb") as f:
+        f.write(np.array([0x474C4144, nl] + sizes + [spec.batch, spec.cost, N, epochs], np.int32).tobytes())
+        for l in range(nl):
+            f.write(np.array([spec.lr[l], spec.mom[l], spec.wd1[l], spec.wd2[l]], np.float32).tobytes())
+            f.write(np.array([spec.act[l]], np.int32).tobytes())
+            f.write(np.array([spec.act_param[l]], np.float32).tobytes())
+        for l in range(nl):
+            f.write(np.ascontiguousarray(weights[l], np.float32).tobytes())
+        f.write(np.array([biases[l] for l in range(nl)], np.float32).tobytes())
+        f.write(X.tobytes())
+        f.write(Y.tobytes())
+    with open(os.devnull, "w") as dn:
+        subprocess.check_call([REF_HARNESS, "train", cin, cout], stdout=dn)
+    raw = np.fromfile(cout, np.float32)
+    pos = 0
+    out = {"epochs": raw[: 2 * epochs].reshape(epochs, 2).copy()}
+    pos = 2 * epochs
+    out["W"] = []
+    for l in range(nl):
+        cnt = sizes[l] * sizes[l + 1]
+        out["W"].append(raw[pos : pos + cnt].reshape(sizes[l + 1], sizes[l]).copy())
+        pos += cnt
+    out["bias"] = raw[pos : pos + nl].copy()
+    pos += nl
+    out["preds"] = raw[pos : pos + N * sizes[-1]].reshape(N, sizes[-1]).copy()
+    pos += N * sizes[-1]
+    out["wsum"], out["wlast"] = [], []
+    for l in range(nl):
+        cnt = sizes[l] * sizes[l + 1]
+        w = raw[pos : pos + 2 * cnt].reshape(sizes[l + 1], sizes[l], 2)
+        out["wsum"].append(w[..., 0].copy())
+        out["wlast"].append(w[..., 1].copy())
+        pos += 2 * cnt
+    assert pos == raw.size
+    return out

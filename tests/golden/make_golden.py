@@ -1,0 +1,133 @@
+"""Writes the golden fixtures in this directory.
+
+Runs ONLY where oracle/_ref/ref_harness exists (the build container: it is compiled from the
+reference's own node/edge/layer/Terminator/gmath sources by `make -C oracle ref`).  Every
+number stored here was produced by that reference code; the inputs are seeded numpy draws,
+the reference's unit-test data (xor gate table, iris measurements) and its NNInfo fixture
+hyper-parameters (xornet: 2-2-1 TANH lr .003 mb 1 REGRESSION; iris: 4-5-3 SIGMOID lr .01
+mb 1 CLASSIFICATION).
+
+    python tests/golden/make_golden.py
+"""
+import os
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+import pyoracle as po  # noqa: E402
+
+# (name, sizes, acts, cost, N, mb, epochs, lr, mom, wd1, wd2, act_params, seed, kind)
+CASES = [
+    ("one_sample_2_3_2", [2, 3, 2], [po.TANH, po.TANH], po.REGRESSION, 1, 1, 1, 0.1, 0, 0, 0, 0, 1, "rand"),
+    ("window_4_5_3_1", [4, 5, 3, 1], [po.TANH] * 3, po.REGRESSION, 11, 3, 4, 0.05, 0.5, 0, 0, 0, 2, "rand"),
+    ("decay_3_4_2", [3, 4, 2], [po.SIGMOID] * 2, po.CLASSIFICATION, 10, 4, 3, 0.05, 0.9, 0.01, 0.01, 0, 3, "rand"),
+    ("cfg1_shape_4_16_3", [4, 16, 3], [po.SIGMOID] * 2, po.CLASSIFICATION, 150, 150, 25, 0.01, 0.9, 0, 0, 0, 4, "rand"),
+    ("cfg2_shape_32_64_64_1", [32, 64, 64, 1], [po.TANH, po.TANH, po.LINEAR], po.REGRESSION, 300, 256, 2,
+     0.01, 0.9, 0, 0, [0, 0, 1.0], 5, "rand"),
+    ("mixed_5_7_6_4", [5, 7, 6, 4], [po.RELU, po.LEAKY, po.SIGMOIDP], po.CLASSIFICATION, 23, 5, 3, 0.01, 0.3,
+     0.001, 0.002, [0, 0.05, 0.1], 6, "rand"),
+    ("kl_3_5_4_2", [3, 5, 4, 2], [po.TANHP, po.STEP, po.LINEAR], po.KL, 9, 2, 2, 0.01, 0.2, 0, 0,
+     [0.1, 0.2, 0.5], 7, "rand"),
+    ("xornet", [2, 2, 1], [po.TANH, po.TANH], po.REGRESSION, 4, 1, 200, 0.003, 0, 0, 0, 0, 11, "xor"),
+    ("iris", [4, 5, 3], [po.SIGMOID, po.SIGMOID], po.CLASSIFICATION, 150, 1, 30, 0.01, 0, 0, 0, 0, 12, "iris"),
+]
+
+IRIS = os.path.join(HERE, "iris_measurements.csv")
+
+
+def ref_xavier(seed, fan_in, n_out, act, td):
+    out = os.path.join(td, "xav.bin")
+    subprocess.check_call([po.REF_HARNESS, "xavier", str(seed), str(fan_in), str(n_out), str(act), out])
+    return np.fromfile(out, np.float32).reshape(n_out, fan_in)
+
+
+def iris_tables():
+    """Measurements scaled the way NumberInput.cpp:68-212 scales a classification table
+    (min/max start from 0 for every column but the first; x -> (x-min)/range*0.98+0.01) and
+    labels one-hot at 0.99/0.01 in order of first appearance (OHE.cpp:159-198)."""
+    rows = [ln.strip().split(",") for ln in open(IRIS) if ln.strip()]
+    feats = np.array([[np.float32(v) for v in r[:4]] for r in rows], np.float32)
+    names = []
+    for r in rows:
+        if r[4] not in names:
+            names.append(r[4])
+    X = np.empty_like(feats)
+    for c in range(4):
+        col = feats[:, c]
+        fmin = np.float32(min(col.min(), col[0] if c == 0 else np.float32(0)))
+        fmax = np.float32(max(col.max(), col[0] if c == 0 else np.float32(0)))
+        rng = np.float32(fmax - fmin)
+        X[:, c] = ((col - fmin) / rng) * np.float32(0.98) + np.float32(0.01)
+    Y = np.full((len(rows), 3), 0.01, np.float32)
+    for i, r in enumerate(rows):
+        Y[i, names.index(r[4])] = 0.99
+    return X, Y
+
+
+def main():
+    if not po.have_ref():
+        raise SystemExit("oracle/_ref/ref_harness missing: run `make -C oracle ref` where /root/reference exists")
+    with tempfile.TemporaryDirectory() as td:
+        # element-wise grid
+        g = os.path.join(td, "g.bin")
+        subprocess.check_call([po.REF_HARNESS, "gmath", g])
+        raw = open(g, "rb").read()
+        nz, npar = np.frombuffer(raw[:8], np.int32)
+        body = np.frombuffer(raw[8:], np.float32)
+        n_act = 8 * npar * nz * 3
+        np.savez_compressed(os.path.join(HERE, "gmath_grid.npz"), nz=nz, npar=npar,
+                            act=body[:n_act].reshape(8, npar, nz, 3), cost=body[n_act:].reshape(3, 6, -1, 5))
+        # Terminator truth table
+        t = os.path.join(td, "t.bin")
+        subprocess.check_call([po.REF_HARNESS, "term", t])
+        np.savez_compressed(os.path.join(HERE, "terminator_table.npz"),
+                            rec=np.fromfile(t, np.int32).reshape(-1, 7))
+        # sampler
+        xav = {}
+        for seed, fi, no, act in [(1, 4, 5, po.SIGMOID), (7, 2, 2, po.TANH), (42, 16, 3, po.RELU), (3, 64, 8, po.TANH)]:
+            xav[f"s{seed}_{fi}_{no}_{act}"] = ref_xavier(seed, fi, no, act, td)
+        np.savez_compressed(os.path.join(HERE, "xavier_samples.npz"), **xav)
+        # training runs
+        for (name, sizes, acts, cost, N, mb, epochs, lr, mom, wd1, wd2, params, seed, kind) in CASES:
+            rng = np.random.default_rng(seed)
+            nl = len(sizes) - 1
+            spec = po.make_spec(sizes, acts, lr=lr, mom=mom, wd1=wd1, wd2=wd2, act_params=params, batch=mb, cost=cost)
+            if kind == "rand":
+                Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * 0.5).astype(np.float32) for l in range(nl)]
+                bs = [0.0] + [float(np.float32(rng.standard_normal() * 0.1)) for _ in range(nl - 1)]
+                X = rng.random((N, sizes[0])).astype(np.float32)
+                if cost == po.CLASSIFICATION:
+                    Y = (np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], N)] * 0.98 + 0.01).astype(np.float32)
+                else:
+                    Y = rng.random((N, sizes[-1])).astype(np.float32)
+            else:
+                Ws = [ref_xavier(seed + l, sizes[l], sizes[l + 1], acts[max(l - 1, 0)] if l == nl - 1 else acts[l], td)
+                      for l in range(nl)]
+                bs = [0.0] * nl
+                if kind == "xor":
+                    X = np.array([[0, 0], [0, 1], [1, 0], [1, 1]], np.float32)
+                    Y = np.array([[0], [1], [1], [0]], np.float32)
+                else:
+                    X, Y = iris_tables()
+            ref = po.ref_train(spec, Ws, bs, X, Y, epochs, td)
+            d = dict(sizes=np.array(sizes, np.int32), acts=np.array(acts, np.int32),
+                     hyper=np.array([lr, mom, wd1, wd2], np.float32),
+                     act_params=np.array(params if isinstance(params, list) else [params] * nl, np.float32),
+                     ints=np.array([cost, N, mb, epochs], np.int32), X=X, Y=Y,
+                     bias0=np.array(bs, np.float32), epochs=ref["epochs"], bias=ref["bias"], preds=ref["preds"])
+            for l in range(nl):
+                d[f"W0_{l}"] = Ws[l]
+                d[f"W_{l}"] = ref["W"][l]
+                d[f"wsum_{l}"] = ref["wsum"][l]
+                d[f"wlast_{l}"] = ref["wlast"][l]
+            np.savez_compressed(os.path.join(HERE, f"train_{name}.npz"), **d)
+            print(name, "epochs", epochs, "last", ref["epochs"][-1])
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,123 @@
+"""Canonical (batched) mode of the restatement: no counterpart in the reference, so it is
+pinned against torch autograd + torch.optim.SGD and against the exact-mode forward."""
+import numpy as np
+import pytest
+import torch
+
+import pyoracle as po
+from helpers import bits_equal
+
+
+def torch_mlp(sizes, acts, params, Ws, bs):
+    Wt = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in Ws]
+    bt = [torch.tensor(b, dtype=torch.float64, requires_grad=True) for b in bs]
+
+    def fwd(x):
+        a = x
+        for l, (W, b) in enumerate(zip(Wt, bt)):
+            z = a @ W.T + b
+            k = acts[l]
+            if k == po.RELU:
+                a = torch.where(z < 0.046, torch.zeros_like(z), z)
+            elif k == po.TANH:
+                a = torch.tanh(z)
+            elif k == po.SIGMOID:
+                a = torch.sigmoid(z)
+            elif k == po.LINEAR:
+                a = params[l] * z
+            elif k == po.SOFTMAX:
+                a = torch.softmax(z, dim=1)
+        return a
+    return Wt, bt, fwd
+
+
+CASES = [
+    ("relu_softmax", [12, 20, 16, 5], [po.RELU, po.RELU, po.SOFTMAX], [0, 0, 0], po.CLASSIFICATION),
+    ("sigmoid_bce", [6, 9, 4], [po.SIGMOID, po.SIGMOID], [0, 0], po.CLASSIFICATION),
+    ("tanh_linear_mse", [8, 10, 7, 2], [po.TANH, po.TANH, po.LINEAR], [0, 0, 1.0], po.REGRESSION),
+]
+
+
+@pytest.mark.parametrize("name,sizes,acts,params,cost", CASES)
+def test_steps_match_torch_sgd(name, sizes, acts, params, cost):
+    rng = np.random.default_rng(3)
+    nl = len(sizes) - 1
+    lr, mom, wd2 = 0.05, 0.9, 1e-3
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (1.5 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(nl)]
+    bs = [(rng.standard_normal(sizes[l + 1]) * 0.1).astype(np.float32) for l in range(nl)]
+    B = 37
+    steps = 6
+    Xs = rng.standard_normal((steps, B, sizes[0])).astype(np.float32)
+    if cost == po.CLASSIFICATION:
+        Ys = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], (steps, B))]
+    else:
+        Ys = rng.standard_normal((steps, B, sizes[-1])).astype(np.float32)
+    net = po.CanonNet(po.make_spec(sizes, acts, lr=lr, mom=mom, wd2=wd2, act_params=params, batch=B, cost=cost))
+    for l in range(nl):
+        net.set_params(l, Ws[l], bs[l])
+    Wt, bt, fwd = torch_mlp(sizes, acts, params, Ws, bs)
+    opt = torch.optim.SGD([{"params": Wt, "weight_decay": wd2}, {"params": bt, "weight_decay": 0.0}], lr=lr, momentum=mom)
+    for s in range(steps):
+        x = torch.tensor(Xs[s], dtype=torch.float64)
+        y = torch.tensor(Ys[s], dtype=torch.float64)
+        p = fwd(x)
+        if acts[-1] == po.SOFTMAX:
+            loss = -(y * torch.log(p)).sum(1).mean()
+        elif cost == po.CLASSIFICATION:
+            loss = -(y * torch.log(p) + (1 - y) * torch.log(1 - p)).sum(1).mean()
+        else:
+            loss = ((p - y) ** 2).sum(1).mean()
+        opt.zero_grad()
+        loss.backward()
+        m = net.step(Xs[s], Ys[s])
+        if s == 0:
+            for l in range(nl):
+                gW, gb = net.get_grads(l)
+                np.testing.assert_allclose(gW, Wt[l].grad.numpy(), rtol=2e-4, atol=2e-6)
+                np.testing.assert_allclose(gb, bt[l].grad.numpy(), rtol=2e-4, atol=2e-6)
+        opt.step()
+        np.testing.assert_allclose(m.loss, loss.item(), rtol=1e-4)
+        if cost == po.CLASSIFICATION:
+            assert m.correct == int((p.argmax(1) == y.argmax(1)).sum())
+    for l in range(nl):
+        W, b = net.get_params(l)
+        np.testing.assert_allclose(W, Wt[l].detach().numpy(), rtol=5e-4, atol=5e-6)
+        np.testing.assert_allclose(b, bt[l].detach().numpy(), rtol=5e-4, atol=5e-6)
+
+
+def test_l1_term_and_ragged_batch():
+    """wd1 adds wd1*sign(W) to the gradient; a batch of 1 and a batch that is not a multiple
+    of the internal row block give the same per-row forward."""
+    rng = np.random.default_rng(8)
+    sizes, acts = [5, 6, 3], [po.TANH, po.SOFTMAX]
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * 0.5).astype(np.float32) for l in range(2)]
+    X = rng.standard_normal((19, 5)).astype(np.float32)
+    Y = np.eye(3, dtype=np.float32)[rng.integers(0, 3, 19)]
+    a = po.CanonNet(po.make_spec(sizes, acts, lr=0.1, wd1=0.0, cost=po.CLASSIFICATION))
+    b = po.CanonNet(po.make_spec(sizes, acts, lr=0.1, wd1=0.01, cost=po.CLASSIFICATION))
+    for n in (a, b):
+        for l in range(2):
+            n.set_params(l, Ws[l])
+    full = a.forward(X)
+    for r in (0, 7, 18):
+        assert bits_equal(a.forward(X[r:r + 1]), full[r:r + 1])
+    a.step(X, Y); b.step(X, Y)
+    for l in range(2):
+        np.testing.assert_allclose(a.get_params(l)[0] - b.get_params(l)[0], 0.1 * 0.01 * np.sign(Ws[l]), rtol=1e-3, atol=1e-7)
+
+
+def test_forward_equals_exact_mode_forward():
+    """An all-equal bias vector reproduces the reference's scalar layer bias bit for bit."""
+    rng = np.random.default_rng(4)
+    sizes, acts, params = [7, 9, 8, 4], [po.RELU, po.SIGMOIDP, po.LEAKY], [0, 0.1, 0.05]
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * 0.5).astype(np.float32) for l in range(3)]
+    sb = [0.0, 0.25, -0.125]
+    X = rng.standard_normal((21, 7)).astype(np.float32)
+    Y = rng.random((21, 4)).astype(np.float32)
+    ex = po.ExactNet(po.make_spec(sizes, acts, act_params=params, batch=1, cost=po.REGRESSION))
+    ca = po.CanonNet(po.make_spec(sizes, acts, act_params=params, batch=1, cost=po.REGRESSION))
+    for l in range(3):
+        ex.set_weights(l, Ws[l]); ex.set_bias(l, sb[l])
+        ca.set_params(l, Ws[l], np.full(sizes[l + 1], sb[l], np.float32))
+    _, preds = ex.epoch(X, Y, train=False)
+    assert bits_equal(ca.forward(X), preds)
