@@ -1,0 +1,865 @@
+// C ABI of libglades_hip.so (declared in include/glades_hip.h): the device-side network object
+// and the host logic that strings the kernels together.
+
+#include "ghip_internal.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <string>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...)
+{
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                         \
+    do {                                                                                      \
+        hipError_t e__ = (expr);                                                              \
+        if (e__ != hipSuccess)                                                                \
+            return fail(GHIP_EHIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__), __FILE__, __LINE__); \
+    } while (0)
+
+int g_device = -1;
+int g_max_lds = 65536;
+
+struct ProfRec { std::string name; hipEvent_t a, b; };
+struct ProfAgg { std::string name; double ms; int64_t n; };
+
+}  // namespace
+
+struct ghip_net {
+    ghip_net_spec spec;
+    hipStream_t stream = nullptr;
+    int L = 0;
+    // dataset
+    const float* dX = nullptr;
+    const float* dY = nullptr;
+    float* ownX = nullptr;
+    float* ownY = nullptr;
+    int64_t n_rows = 0;
+    uint16_t* Xbf = nullptr;  // bf16 copy of the table (BF16 / FP8_INFER)
+    // exact
+    ExactLaunch ex;
+    int ex_threads = 64;
+    size_t ex_lds = 0;
+    float *exW = nullptr, *exSum = nullptr, *exLast = nullptr, *exBias = nullptr, *exPreds = nullptr;
+    ghip_metrics* exMetrics = nullptr;
+    int exMetricsCap = 0;
+    int64_t exPredsCap = 0;
+    int* exEpochs = nullptr;
+    // canonical fp32 state (also the master copy for BF16 / the source for FP8)
+    float* W[GHIP_MAX_LAYERS] = {};
+    float* b[GHIP_MAX_LAYERS] = {};
+    float* vW[GHIP_MAX_LAYERS] = {};
+    float* vb[GHIP_MAX_LAYERS] = {};
+    float* gW[GHIP_MAX_LAYERS] = {};
+    float* act[GHIP_MAX_LAYERS + 1] = {};
+    float* dlt[GHIP_MAX_LAYERS + 1] = {};
+    float* stageX = nullptr;
+    int cap_batch = 0;
+    double* dAcc = nullptr;
+    int last_batch = 0;
+    // bf16
+    uint16_t* Wh[GHIP_MAX_LAYERS] = {};
+    uint16_t* WhT[GHIP_MAX_LAYERS] = {};
+    uint16_t* H[GHIP_MAX_LAYERS + 1] = {};
+    uint16_t* HT[GHIP_MAX_LAYERS + 1] = {};
+    uint16_t* D[GHIP_MAX_LAYERS + 1] = {};
+    uint16_t* DT[GHIP_MAX_LAYERS + 1] = {};
+    float* logits = nullptr;
+    bool shadow_dirty = true;
+    // fp8
+    uint8_t* Wq[GHIP_MAX_LAYERS] = {};
+    float* wscale[GHIP_MAX_LAYERS] = {};
+    uint8_t* Aq[2] = {};
+    float* ascale[2] = {};
+    unsigned int* amax_bits = nullptr;
+    uint16_t* Hq = nullptr;
+    float* out8 = nullptr;
+    bool quantized = false;
+    // profiling
+    bool prof = false;
+    std::vector<ProfRec> recs;
+    std::vector<ProfAgg> aggs;
+};
+
+namespace {
+
+template <typename T>
+int dalloc(T** p, size_t count)
+{
+    if (count == 0) count = 1;
+    hipError_t e = hipMalloc((void**)p, count * sizeof(T));
+    if (e != hipSuccess) {
+        *p = nullptr;
+        return fail(GHIP_ENOMEM, "hipMalloc of %zu bytes failed: %s", count * sizeof(T), hipGetErrorString(e));
+    }
+    return 0;
+}
+#define TRY(expr) do { int r__ = (expr); if (r__ != 0) return r__; } while (0)
+
+template <typename T>
+void dfree(T*& p) { if (p) { (void)hipFree((void*)p); p = nullptr; } }
+
+struct Scope {
+    ghip_net* n; const char* name; hipEvent_t a = nullptr, b = nullptr;
+    Scope(ghip_net* n_, const char* nm) : n(n_), name(nm)
+    {
+        if (n->prof) {
+            (void)hipEventCreate(&a);
+            (void)hipEventCreate(&b);
+            (void)hipEventRecord(a, n->stream);
+        }
+    }
+    ~Scope()
+    {
+        if (n->prof) {
+            (void)hipEventRecord(b, n->stream);
+            n->recs.push_back(ProfRec{name, a, b});
+        }
+    }
+};
+#define LAUNCH(net, name, expr)                                                                \
+    do {                                                                                       \
+        hipError_t e__;                                                                        \
+        { Scope sc__(net, name); e__ = (expr); }                                               \
+        if (e__ != hipSuccess) return fail(GHIP_EHIP, "%s: %s", name, hipGetErrorString(e__)); \
+    } while (0)
+
+void prof_collect(ghip_net* n)
+{
+    if (n->recs.empty()) return;
+    (void)hipStreamSynchronize(n->stream);
+    for (auto& r : n->recs) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, r.a, r.b) == hipSuccess) {
+            bool found = false;
+            for (auto& g : n->aggs)
+                if (g.name == r.name) { g.ms += ms; g.n += 1; found = true; break; }
+            if (!found) n->aggs.push_back(ProfAgg{r.name, ms, 1});
+        }
+        (void)hipEventDestroy(r.a);
+        (void)hipEventDestroy(r.b);
+    }
+    n->recs.clear();
+}
+
+int pow2ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
+int ilog2(int v) { int l = 0; while ((1 << l) < v) ++l; return l; }
+
+bool is_canon(const ghip_net* n) { return n->spec.mode == GHIP_MODE_CANONICAL; }
+
+int check_spec(const ghip_net_spec* s)
+{
+    if (!s) return fail(GHIP_EINVAL, "spec is NULL");
+    if (s->n_layers < 1 || s->n_layers > GHIP_MAX_LAYERS) return fail(GHIP_EINVAL, "n_layers %d out of range", s->n_layers);
+    for (int l = 0; l <= s->n_layers; ++l)
+        if (s->sizes[l] < 1) return fail(GHIP_EINVAL, "layer %d has size %d", l, s->sizes[l]);
+    if (s->cost < GHIP_REGRESSION || s->cost > GHIP_KL) return fail(GHIP_EINVAL, "unknown cost %d", s->cost);
+    for (int l = 0; l < s->n_layers; ++l) {
+        if (s->act[l] < GHIP_TANH || s->act[l] > GHIP_SOFTMAX) return fail(GHIP_EINVAL, "unknown activation %d", s->act[l]);
+        if (s->act[l] == GHIP_SOFTMAX && (l != s->n_layers - 1 || s->mode != GHIP_MODE_CANONICAL))
+            return fail(GHIP_EINVAL, "softmax is a canonical-mode output activation only");
+    }
+    if (s->mode == GHIP_MODE_EXACT) {
+        // BATCH_FULL = 0 would be "row % 0" in the reference (nninfo.h:63, network.cpp:647)
+        if (s->batch < 1) return fail(GHIP_EINVAL, "exact mode needs batch >= 1 (full batch = number of rows)");
+        if (s->dtype != GHIP_F32) return fail(GHIP_EINVAL, "exact mode is fp32 only");
+    } else if (s->mode == GHIP_MODE_CANONICAL) {
+        if (s->dtype < GHIP_F32 || s->dtype > GHIP_FP8_INFER) return fail(GHIP_EINVAL, "unknown dtype %d", s->dtype);
+        if (s->dtype != GHIP_F32) {
+            for (int l = 0; l <= s->n_layers; ++l)
+                if (s->sizes[l] % 256) return fail(GHIP_EINVAL, "bf16/fp8 paths need layer sizes that are multiples of 256 (layer %d is %d)", l, s->sizes[l]);
+        }
+    } else {
+        return fail(GHIP_EINVAL, "unknown mode %d", s->mode);
+    }
+    return 0;
+}
+
+int setup_exact(ghip_net* n)
+{
+    ExactLaunch& e = n->ex;
+    memset(&e, 0, sizeof(e));
+    const ghip_net_spec& s = n->spec;
+    e.n_layers = s.n_layers;
+    int woff = 0, aoff = 0, max_edges = 0, max_nodes = 0;
+    for (int l = 0; l <= s.n_layers; ++l) {
+        e.sizes[l] = s.sizes[l];
+        e.aoff[l] = aoff;
+        aoff += s.sizes[l];
+        if (s.sizes[l] > max_nodes) max_nodes = s.sizes[l];
+    }
+    for (int l = 0; l < s.n_layers; ++l) {
+        e.ld[l] = s.sizes[l] | 1;
+        e.woff[l] = woff;
+        woff += e.ld[l] * s.sizes[l + 1];
+        int edges = s.sizes[l] * s.sizes[l + 1];
+        if (edges > max_edges) max_edges = edges;
+        e.lr[l] = s.lr[l]; e.mom[l] = s.mom[l]; e.wd1[l] = s.wd1[l]; e.wd2[l] = s.wd2[l];
+        e.act[l] = s.act[l]; e.act_param[l] = s.act_param[l];
+    }
+    e.state_floats = woff;
+    e.node_floats = aoff;
+    e.mb = s.batch; e.cost = s.cost; e.bias_mode = s.bias_mode;
+    int T = pow2ceil((max_edges + 7) / 8);
+    if (T < pow2ceil(max_nodes)) T = pow2ceil(max_nodes);
+    if (T < 64) T = 64;
+    if (T > 1024) T = 1024;
+    if (const char* env = getenv("GHIP_EXACT_THREADS")) {
+        int v = atoi(env);
+        if (v == 64 || v == 128 || v == 256 || v == 512 || v == 1024) T = v;
+    }
+    n->ex_threads = T;
+    for (int l = 0; l < s.n_layers; ++l) {
+        int tw = pow2ceil(s.sizes[l]);
+        if (tw > T) tw = T;
+        e.tw_log2[l] = ilog2(tw);
+    }
+    size_t lds_full = ghip_exact_lds_bytes(e, true);
+    e.state_in_lds = lds_full <= (size_t)g_max_lds ? 1 : 0;
+    n->ex_lds = ghip_exact_lds_bytes(e, e.state_in_lds != 0);
+    if (n->ex_lds > (size_t)g_max_lds)
+        return fail(GHIP_EINVAL, "exact mode: layers too wide (%zu bytes of node state exceed LDS)", n->ex_lds);
+    TRY(dalloc(&n->exW, (size_t)woff));
+    TRY(dalloc(&n->exSum, (size_t)woff));
+    TRY(dalloc(&n->exLast, (size_t)woff));
+    TRY(dalloc(&n->exBias, GHIP_MAX_LAYERS));
+    TRY(dalloc(&n->exEpochs, 1));
+    HIP_TRY(hipMemsetAsync(n->exW, 0, sizeof(float) * woff, n->stream));
+    HIP_TRY(hipMemsetAsync(n->exSum, 0, sizeof(float) * woff, n->stream));
+    HIP_TRY(hipMemsetAsync(n->exLast, 0, sizeof(float) * woff, n->stream));
+    HIP_TRY(hipMemsetAsync(n->exBias, 0, sizeof(float) * GHIP_MAX_LAYERS, n->stream));
+    e.W = n->exW; e.wsum = n->exSum; e.wlast = n->exLast; e.bias = n->exBias; e.epochs_run = n->exEpochs;
+    return 0;
+}
+
+int setup_canon(ghip_net* n)
+{
+    const ghip_net_spec& s = n->spec;
+    for (int l = 0; l < s.n_layers; ++l) {
+        size_t cnt = (size_t)s.sizes[l] * s.sizes[l + 1];
+        TRY(dalloc(&n->W[l], cnt));
+        TRY(dalloc(&n->b[l], (size_t)s.sizes[l + 1]));
+        HIP_TRY(hipMemsetAsync(n->W[l], 0, cnt * 4, n->stream));
+        HIP_TRY(hipMemsetAsync(n->b[l], 0, (size_t)s.sizes[l + 1] * 4, n->stream));
+        if (s.dtype != GHIP_FP8_INFER) {
+            TRY(dalloc(&n->vW[l], cnt));
+            TRY(dalloc(&n->vb[l], (size_t)s.sizes[l + 1]));
+            HIP_TRY(hipMemsetAsync(n->vW[l], 0, cnt * 4, n->stream));
+            HIP_TRY(hipMemsetAsync(n->vb[l], 0, (size_t)s.sizes[l + 1] * 4, n->stream));
+        }
+        if (s.dtype == GHIP_F32) TRY(dalloc(&n->gW[l], cnt));
+        if (s.dtype == GHIP_BF16) {
+            TRY(dalloc(&n->Wh[l], cnt));
+            TRY(dalloc(&n->WhT[l], cnt));
+        }
+        if (s.dtype == GHIP_FP8_INFER) {
+            TRY(dalloc(&n->Wq[l], cnt));
+            TRY(dalloc(&n->wscale[l], (size_t)s.sizes[l + 1]));
+        }
+    }
+    TRY(dalloc(&n->dAcc, 4));
+    HIP_TRY(hipMemsetAsync(n->dAcc, 0, 4 * sizeof(double), n->stream));
+    return 0;
+}
+
+void free_batch_buffers(ghip_net* n)
+{
+    for (int l = 0; l <= GHIP_MAX_LAYERS; ++l) {
+        dfree(n->act[l]); dfree(n->dlt[l]);
+        if (l > 0) dfree(n->H[l]);
+        dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]);
+    }
+    dfree(n->stageX); dfree(n->logits);
+    dfree(n->Aq[0]); dfree(n->Aq[1]); dfree(n->ascale[0]); dfree(n->ascale[1]);
+    dfree(n->amax_bits); dfree(n->Hq); dfree(n->out8);
+    n->cap_batch = 0;
+}
+
+int reserve_batch(ghip_net* n, int B)
+{
+    if (B <= n->cap_batch) return 0;
+    (void)hipStreamSynchronize(n->stream);
+    free_batch_buffers(n);
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    int maxw = 0;
+    for (int l = 0; l <= L; ++l) if (s.sizes[l] > maxw) maxw = s.sizes[l];
+    if (s.dtype == GHIP_F32) {
+        TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
+        for (int l = 1; l <= L; ++l) {
+            TRY(dalloc(&n->act[l], (size_t)B * s.sizes[l]));
+            TRY(dalloc(&n->dlt[l], (size_t)B * s.sizes[l]));
+        }
+    } else if (s.dtype == GHIP_BF16) {
+        TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
+        TRY(dalloc(&n->HT[0], (size_t)B * s.sizes[0]));
+        for (int l = 1; l <= L; ++l) {
+            if (l < L) {
+                TRY(dalloc(&n->H[l], (size_t)B * s.sizes[l]));
+                TRY(dalloc(&n->HT[l], (size_t)B * s.sizes[l]));
+            }
+            TRY(dalloc(&n->D[l], (size_t)B * s.sizes[l]));
+            TRY(dalloc(&n->DT[l], (size_t)B * s.sizes[l]));
+        }
+        TRY(dalloc(&n->logits, (size_t)B * s.sizes[L]));
+    } else {
+        TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
+        TRY(dalloc(&n->Aq[0], (size_t)B * maxw));
+        TRY(dalloc(&n->Aq[1], (size_t)B * maxw));
+        TRY(dalloc(&n->ascale[0], (size_t)B));
+        TRY(dalloc(&n->ascale[1], (size_t)B));
+        TRY(dalloc(&n->amax_bits, (size_t)B));
+        TRY(dalloc(&n->Hq, (size_t)B * maxw));
+        TRY(dalloc(&n->out8, (size_t)B * s.sizes[L]));
+    }
+    n->cap_batch = B;
+    return 0;
+}
+
+// bf16 shadows W, W^T from the fp32 master (after ghip_net_set_params)
+int refresh_shadows(ghip_net* n)
+{
+    if (!n->shadow_dirty) return 0;
+    const ghip_net_spec& s = n->spec;
+    for (int l = 0; l < s.n_layers; ++l)
+        LAUNCH(n, "f32_to_bf16_transpose", ghip_f32_to_bf16_2d(n->W[l], n->Wh[l], n->WhT[l], s.sizes[l + 1], s.sizes[l], n->stream));
+    n->shadow_dirty = false;
+    return 0;
+}
+
+int out_act(const ghip_net_spec& s, int l, float* param)
+{
+    // the GEMM epilogue leaves softmax logits untouched (LINEAR with slope 1)
+    if (s.act[l] == GHIP_SOFTMAX) { *param = 1.0f; return GHIP_LINEAR; }
+    *param = s.act_param[l];
+    return s.act[l];
+}
+
+// ---- canonical fp32 ----
+int forward_f32(ghip_net* n, const float* X, int B)
+{
+    const ghip_net_spec& s = n->spec;
+    const float* in = X;
+    for (int l = 0; l < s.n_layers; ++l) {
+        GemmF32Args g;
+        memset(&g, 0, sizeof(g));
+        g.A = in; g.B = n->W[l]; g.C = n->act[l + 1];
+        g.M = B; g.N = s.sizes[l + 1]; g.K = s.sizes[l];
+        g.lda = s.sizes[l]; g.ldb = s.sizes[l]; g.ldc = s.sizes[l + 1];
+        g.epilogue = EPI_BIAS_ACT; g.bias = n->b[l];
+        g.act = out_act(s, l, &g.act_param);
+        g.alpha = 1.0f;
+        LAUNCH(n, "gemm_f32_forward", ghip_gemm_f32(g, n->stream));
+        in = n->act[l + 1];
+    }
+    return 0;
+}
+
+int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* Dbf, int B)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    LAUNCH(n, "fill_metrics", ghip_fill_f64(n->dAcc, 4, 0.0, n->stream));
+    DeltaArgs a;
+    memset(&a, 0, sizeof(a));
+    a.P = P; a.Y = Y; a.D = D; a.Dbf = Dbf; a.DbfT = nullptr;
+    a.B = B; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
+    a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost; a.acc = n->dAcc;
+    LAUNCH(n, "output_delta", ghip_output_delta(a, n->stream));
+    return 0;
+}
+
+int step_f32(ghip_net* n, int64_t row0, int B)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    const float* X = n->dX + row0 * s.sizes[0];
+    const float* Y = n->dY + row0 * s.sizes[L];
+    TRY(forward_f32(n, X, B));
+    TRY(output_delta_f32(n, n->act[L], Y, n->dlt[L], nullptr, B));
+    for (int l = L - 1; l >= 0; --l) {
+        const int ni = s.sizes[l], no = s.sizes[l + 1];
+        const float* Ain = (l == 0) ? X : n->act[l];
+        GemmF32Args g;
+        memset(&g, 0, sizeof(g));
+        // gradient: G[no][ni] = D^T A / B
+        g.A = n->dlt[l + 1]; g.lda = no; g.a_kmajor = 1;
+        g.B = Ain; g.ldb = ni; g.b_kmajor = 1;
+        g.C = n->gW[l]; g.ldc = ni; g.M = no; g.N = ni; g.K = B;
+        g.epilogue = EPI_STORE; g.alpha = 1.0f / (float)B;
+        LAUNCH(n, "gemm_f32_wgrad", ghip_gemm_f32(g, n->stream));
+        if (l > 0) {  // back-prop with the pre-update weights: E = D W, times f'(a_l)
+            memset(&g, 0, sizeof(g));
+            g.A = n->dlt[l + 1]; g.lda = no; g.a_kmajor = 0;
+            g.B = n->W[l]; g.ldb = ni; g.b_kmajor = 1;
+            g.C = n->dlt[l]; g.ldc = ni; g.M = B; g.N = ni; g.K = no;
+            g.epilogue = EPI_MUL_DER; g.aux = n->act[l];
+            g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1]; g.alpha = 1.0f;
+            LAUNCH(n, "gemm_f32_dgrad", ghip_gemm_f32(g, n->stream));
+        }
+        LAUNCH(n, "bias_update", ghip_bias_update_f32(n->dlt[l + 1], B, no, no, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+        LAUNCH(n, "sgd_update_f32", ghip_sgd_update_f32(n->W[l], n->vW[l], n->gW[l], (long long)ni * no, s.lr[l], s.mom[l],
+                                                       s.wd1[l], s.wd2[l], 1.0f, n->stream));
+    }
+    return 0;
+}
+
+// ---- canonical bf16 ----
+int forward_bf16(ghip_net* n, const uint16_t* X, int B)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    const uint16_t* in = X;
+    for (int l = 0; l < L; ++l) {
+        GemmLpArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = in; g.B = n->Wh[l]; g.M = B; g.N = s.sizes[l + 1]; g.K = s.sizes[l];
+        g.fp8 = 0; g.bias = n->b[l];
+        g.act = out_act(s, l, &g.act_param);
+        if (l < L - 1) {
+            g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = n->HT[l + 1];
+            LAUNCH(n, "gemm_bf16_forward", ghip_gemm_lp(g, n->stream));
+        } else {
+            g.epilogue = LP_FWD_F32; g.out = n->logits;
+            LAUNCH(n, "gemm_bf16_forward_out", ghip_gemm_lp(g, n->stream));
+        }
+        in = n->H[l + 1];
+    }
+    return 0;
+}
+
+int step_bf16(ghip_net* n, int64_t row0, int B)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    TRY(refresh_shadows(n));
+    const uint16_t* X = n->Xbf + row0 * s.sizes[0];
+    const float* Y = n->dY + row0 * s.sizes[L];
+    LAUNCH(n, "bf16_transpose_input", ghip_bf16_transpose(X, n->HT[0], B, s.sizes[0], n->stream));
+    TRY(forward_bf16(n, X, B));
+    TRY(output_delta_f32(n, n->logits, Y, nullptr, n->D[L], B));
+    LAUNCH(n, "bf16_transpose_delta", ghip_bf16_transpose(n->D[L], n->DT[L], B, s.sizes[L], n->stream));
+    for (int l = L - 1; l >= 0; --l) {
+        const int ni = s.sizes[l], no = s.sizes[l + 1];
+        GemmLpArgs g;
+        if (l > 0) {
+            memset(&g, 0, sizeof(g));
+            g.A = n->D[l + 1]; g.B = n->WhT[l]; g.M = B; g.N = ni; g.K = no;
+            g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.aux = n->H[l];
+            g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1];
+            LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));
+        }
+        LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+        memset(&g, 0, sizeof(g));
+        g.A = n->DT[l + 1]; g.B = n->HT[l]; g.M = no; g.N = ni; g.K = B;
+        g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l];
+        g.master = n->W[l]; g.mom = n->vW[l];
+        g.lr = s.lr[l]; g.momf = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l]; g.gscale = 1.0f / (float)B;
+        LAUNCH(n, "gemm_bf16_wgrad_sgd", ghip_gemm_lp(g, n->stream));
+    }
+    return 0;
+}
+
+// ---- fp8 inference ----
+int forward_fp8(ghip_net* n, const uint16_t* Xbf, int B, float* dev_out)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    if (!n->quantized) return fail(GHIP_ESTATE, "call ghip_net_quantize_fp8 first");
+    int cur = 0;
+    LAUNCH(n, "quant_rows_e4m3", ghip_quant_rows_e4m3(Xbf, 1, B, s.sizes[0], n->Aq[0], n->ascale[0], nullptr, n->stream));
+    for (int l = 0; l < L; ++l) {
+        GemmLpArgs g;
+        memset(&g, 0, sizeof(g));
+        g.A = n->Aq[cur]; g.B = n->Wq[l]; g.M = B; g.N = s.sizes[l + 1]; g.K = s.sizes[l];
+        g.fp8 = 1; g.row_scale = n->ascale[cur]; g.col_scale = n->wscale[l];
+        g.act = out_act(s, l, &g.act_param);
+        if (l < L - 1) {
+            LAUNCH(n, "fill_amax", ghip_fill_u32(n->amax_bits, B, 0u, n->stream));
+            g.epilogue = LP_FP8_ACT; g.out = n->Hq; g.row_amax_bits = n->amax_bits;
+            LAUNCH(n, "gemm_fp8_forward", ghip_gemm_lp(g, n->stream));
+            LAUNCH(n, "requant_rows_e4m3", ghip_quant_rows_e4m3(n->Hq, 1, B, s.sizes[l + 1], n->Aq[cur ^ 1], n->ascale[cur ^ 1],
+                                                                n->amax_bits, n->stream));
+            cur ^= 1;
+        } else {
+            g.epilogue = LP_FP8_F32; g.out = dev_out;
+            LAUNCH(n, "gemm_fp8_forward_out", ghip_gemm_lp(g, n->stream));
+        }
+    }
+    return 0;
+}
+
+int fetch_metrics(ghip_net* n, ghip_metrics* m)
+{
+    double acc[4];
+    HIP_TRY(hipMemcpyAsync(acc, n->dAcc, sizeof(acc), hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    const int B = n->last_batch > 0 ? n->last_batch : 1;
+    m->loss = (float)(acc[0] / (double)B);
+    m->accuracy = (float)(acc[1] / ((double)B * n->spec.sizes[n->spec.n_layers]));
+    m->correct = (int64_t)(acc[2] + 0.5);
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* ghip_last_error(void) { return g_err.c_str(); }
+const char* ghip_version(void) { return "glades-hip 0.1 (gfx950)"; }
+
+int ghip_init(int device_ordinal)
+{
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) return fail(GHIP_ENODEV, "no HIP device: %s", hipGetErrorString(e));
+    if (device_ordinal < 0 || device_ordinal >= count) return fail(GHIP_EINVAL, "device %d of %d", device_ordinal, count);
+    HIP_TRY(hipSetDevice(device_ordinal));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device_ordinal));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(GHIP_ENODEV, "device %d is %s; this library is built for gfx950 only", device_ordinal, prop.gcnArchName);
+    int lds = 0;
+    if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device_ordinal) == hipSuccess && lds > 0)
+        g_max_lds = lds;
+    g_device = device_ordinal;
+    return 0;
+}
+
+int ghip_net_create(const ghip_net_spec* spec, ghip_net** out)
+{
+    if (!out) return fail(GHIP_EINVAL, "out is NULL");
+    *out = nullptr;
+    if (g_device < 0) TRY(ghip_init(0));
+    TRY(check_spec(spec));
+    ghip_net* n = new ghip_net();
+    n->spec = *spec;
+    n->L = spec->n_layers;
+    hipError_t e = hipStreamCreate(&n->stream);
+    if (e != hipSuccess) { delete n; return fail(GHIP_EHIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
+    int r = (spec->mode == GHIP_MODE_EXACT) ? setup_exact(n) : setup_canon(n);
+    if (r != 0) { std::string keep = g_err; ghip_net_destroy(n); g_err = keep; return r; }
+    *out = n;
+    return 0;
+}
+
+int ghip_net_destroy(ghip_net* n)
+{
+    if (!n) return 0;
+    if (n->stream) (void)hipStreamSynchronize(n->stream);
+    prof_collect(n);
+    free_batch_buffers(n);
+    dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf);
+    dfree(n->exW); dfree(n->exSum); dfree(n->exLast); dfree(n->exBias); dfree(n->exPreds);
+    dfree(n->exMetrics); dfree(n->exEpochs);
+    for (int l = 0; l < GHIP_MAX_LAYERS; ++l) {
+        dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]); dfree(n->gW[l]);
+        dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
+    }
+    dfree(n->dAcc);
+    if (n->stream) (void)hipStreamDestroy(n->stream);
+    delete n;
+    return 0;
+}
+
+int ghip_net_set_params(ghip_net* n, int layer, const float* host_W, const float* host_bias, int bias_len)
+{
+    if (!n || layer < 0 || layer >= n->L) return fail(GHIP_EINVAL, "bad net or layer");
+    const ghip_net_spec& s = n->spec;
+    const int ni = s.sizes[layer], no = s.sizes[layer + 1];
+    if (s.mode == GHIP_MODE_EXACT) {
+        if (bias_len != 0 && bias_len != 1) return fail(GHIP_EINVAL, "exact mode bias is one scalar per layer");
+        if (host_W) {
+            const int ld = n->ex.ld[layer];
+            std::vector<float> pad((size_t)ld * no, 0.0f);
+            for (int o = 0; o < no; ++o) memcpy(&pad[(size_t)o * ld], host_W + (size_t)o * ni, sizeof(float) * ni);
+            HIP_TRY(hipMemcpyAsync(n->exW + n->ex.woff[layer], pad.data(), pad.size() * 4, hipMemcpyHostToDevice, n->stream));
+            HIP_TRY(hipMemsetAsync(n->exSum + n->ex.woff[layer], 0, pad.size() * 4, n->stream));
+            HIP_TRY(hipMemsetAsync(n->exLast + n->ex.woff[layer], 0, pad.size() * 4, n->stream));
+            HIP_TRY(hipStreamSynchronize(n->stream));
+        }
+        if (host_bias && bias_len == 1) {
+            HIP_TRY(hipMemcpyAsync(n->exBias + layer, host_bias, 4, hipMemcpyHostToDevice, n->stream));
+            HIP_TRY(hipStreamSynchronize(n->stream));
+        }
+        return 0;
+    }
+    if (bias_len != 0 && bias_len != no) return fail(GHIP_EINVAL, "canonical bias has one entry per output channel (%d), got %d", no, bias_len);
+    const size_t cnt = (size_t)ni * no;
+    if (host_W) {
+        HIP_TRY(hipMemcpyAsync(n->W[layer], host_W, cnt * 4, hipMemcpyHostToDevice, n->stream));
+        if (n->vW[layer]) HIP_TRY(hipMemsetAsync(n->vW[layer], 0, cnt * 4, n->stream));
+        n->shadow_dirty = true;
+        n->quantized = false;
+    }
+    if (host_bias && bias_len == no) HIP_TRY(hipMemcpyAsync(n->b[layer], host_bias, (size_t)no * 4, hipMemcpyHostToDevice, n->stream));
+    else if (host_W) HIP_TRY(hipMemsetAsync(n->b[layer], 0, (size_t)no * 4, n->stream));
+    if (n->vb[layer]) HIP_TRY(hipMemsetAsync(n->vb[layer], 0, (size_t)no * 4, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    return 0;
+}
+
+int ghip_net_get_params(ghip_net* n, int layer, float* host_W, float* host_bias, int bias_len)
+{
+    if (!n || layer < 0 || layer >= n->L) return fail(GHIP_EINVAL, "bad net or layer");
+    const ghip_net_spec& s = n->spec;
+    const int ni = s.sizes[layer], no = s.sizes[layer + 1];
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    if (s.mode == GHIP_MODE_EXACT) {
+        if (host_W) {
+            const int ld = n->ex.ld[layer];
+            std::vector<float> pad((size_t)ld * no);
+            HIP_TRY(hipMemcpy(pad.data(), n->exW + n->ex.woff[layer], pad.size() * 4, hipMemcpyDeviceToHost));
+            for (int o = 0; o < no; ++o) memcpy(host_W + (size_t)o * ni, &pad[(size_t)o * ld], sizeof(float) * ni);
+        }
+        if (host_bias && bias_len >= 1) HIP_TRY(hipMemcpy(host_bias, n->exBias + layer, 4, hipMemcpyDeviceToHost));
+        return 0;
+    }
+    if (host_W) HIP_TRY(hipMemcpy(host_W, n->W[layer], (size_t)ni * no * 4, hipMemcpyDeviceToHost));
+    if (host_bias) {
+        if (bias_len != no) return fail(GHIP_EINVAL, "bias_len %d != %d", bias_len, no);
+        HIP_TRY(hipMemcpy(host_bias, n->b[layer], (size_t)no * 4, hipMemcpyDeviceToHost));
+    }
+    return 0;
+}
+
+static int make_bf16_table(ghip_net* n)
+{
+    const ghip_net_spec& s = n->spec;
+    if (s.mode != GHIP_MODE_CANONICAL || s.dtype == GHIP_F32) return 0;
+    dfree(n->Xbf);
+    TRY(dalloc(&n->Xbf, (size_t)n->n_rows * s.sizes[0]));
+    // convert in slabs of rows to keep the grid small
+    const int64_t slab = 65536;
+    for (int64_t r = 0; r < n->n_rows; r += slab) {
+        const int rows = (int)((n->n_rows - r) < slab ? (n->n_rows - r) : slab);
+        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d(n->dX + r * s.sizes[0], n->Xbf + r * s.sizes[0], nullptr, rows,
+                                                          s.sizes[0], n->stream));
+    }
+    return 0;
+}
+
+int ghip_net_set_dataset(ghip_net* n, const float* host_X, const float* host_Y, int64_t n_rows)
+{
+    if (!n || !host_X || n_rows <= 0) return fail(GHIP_EINVAL, "bad dataset arguments");
+    const ghip_net_spec& s = n->spec;
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    dfree(n->ownX); dfree(n->ownY);
+    const size_t nx = (size_t)n_rows * s.sizes[0], ny = (size_t)n_rows * s.sizes[s.n_layers];
+    TRY(dalloc(&n->ownX, nx));
+    HIP_TRY(hipMemcpy(n->ownX, host_X, nx * 4, hipMemcpyHostToDevice));
+    if (host_Y) {
+        TRY(dalloc(&n->ownY, ny));
+        HIP_TRY(hipMemcpy(n->ownY, host_Y, ny * 4, hipMemcpyHostToDevice));
+    }
+    n->dX = n->ownX; n->dY = n->ownY; n->n_rows = n_rows;
+    return make_bf16_table(n);
+}
+
+int ghip_net_set_dataset_device(ghip_net* n, const float* dev_X, const float* dev_Y, int64_t n_rows)
+{
+    if (!n || !dev_X || n_rows <= 0) return fail(GHIP_EINVAL, "bad dataset arguments");
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    dfree(n->ownX); dfree(n->ownY);
+    n->dX = dev_X; n->dY = dev_Y; n->n_rows = n_rows;
+    return make_bf16_table(n);
+}
+
+int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_accuracy,
+                              ghip_metrics* host_metrics, int* epochs_run, float* host_preds)
+{
+    if (!n || n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
+    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "network is not in exact mode");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
+    const int nout = n->spec.sizes[n->L];
+    if (n_epochs > n->exMetricsCap) {
+        HIP_TRY(hipStreamSynchronize(n->stream));
+        dfree(n->exMetrics);
+        TRY(dalloc(&n->exMetrics, (size_t)n_epochs));
+        n->exMetricsCap = n_epochs;
+    }
+    if (host_preds && n->n_rows * nout > n->exPredsCap) {
+        HIP_TRY(hipStreamSynchronize(n->stream));
+        dfree(n->exPreds);
+        TRY(dalloc(&n->exPreds, (size_t)n->n_rows * nout));
+        n->exPredsCap = n->n_rows * nout;
+    }
+    ExactLaunch e = n->ex;
+    e.X = n->dX; e.Y = n->dY; e.n_rows = n->n_rows;
+    e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
+    e.preds = host_preds ? n->exPreds : nullptr;
+    e.metrics = (float*)n->exMetrics;
+    LAUNCH(n, "exact_epochs", ghip_launch_exact(e, n->ex_threads, n->ex_lds, n->stream));
+    int ran = 0;
+    HIP_TRY(hipMemcpyAsync(&ran, n->exEpochs, sizeof(int), hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    if (epochs_run) *epochs_run = ran;
+    if (host_metrics && ran > 0) HIP_TRY(hipMemcpy(host_metrics, n->exMetrics, sizeof(ghip_metrics) * ran, hipMemcpyDeviceToHost));
+    if (host_preds) HIP_TRY(hipMemcpy(host_preds, n->exPreds, sizeof(float) * n->n_rows * nout, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int ghip_net_train_step(ghip_net* n, int64_t row0, int batch, ghip_metrics* host_metrics)
+{
+    if (!n || batch < 1 || row0 < 0) return fail(GHIP_EINVAL, "bad arguments");
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    if (n->spec.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "fp8 networks are inference only");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
+    if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows [%lld,%lld) exceed the table (%lld rows)", (long long)row0, (long long)(row0 + batch), (long long)n->n_rows);
+    if (n->spec.dtype == GHIP_BF16 && (batch % 256)) return fail(GHIP_EINVAL, "bf16 path needs a batch that is a multiple of 256");
+    TRY(reserve_batch(n, batch));
+    n->last_batch = batch;
+    if (n->spec.dtype == GHIP_F32) TRY(step_f32(n, row0, batch));
+    else TRY(step_bf16(n, row0, batch));
+    if (host_metrics) return fetch_metrics(n, host_metrics);
+    return 0;
+}
+
+int ghip_net_last_metrics(ghip_net* n, ghip_metrics* m)
+{
+    if (!n || !m) return fail(GHIP_EINVAL, "bad arguments");
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    return fetch_metrics(n, m);
+}
+
+static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xbf, int batch, float** result)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    if (s.dtype == GHIP_F32) {
+        TRY(forward_f32(n, dev_X32, batch));
+        if (s.act[L - 1] == GHIP_SOFTMAX) {
+            DeltaArgs a;
+            memset(&a, 0, sizeof(a));
+            a.P = n->act[L]; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
+            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc;
+            LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
+        }
+        *result = n->act[L];
+    } else if (s.dtype == GHIP_BF16) {
+        TRY(refresh_shadows(n));
+        TRY(forward_bf16(n, dev_Xbf, batch));
+        if (s.act[L - 1] == GHIP_SOFTMAX) {
+            DeltaArgs a;
+            memset(&a, 0, sizeof(a));
+            a.P = n->logits; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
+            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc;
+            LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
+        }
+        *result = n->logits;
+    } else {
+        TRY(forward_fp8(n, dev_Xbf, batch, n->out8));
+        *result = n->out8;
+    }
+    return 0;
+}
+
+int ghip_net_forward(ghip_net* n, const float* host_X, int batch, float* host_out)
+{
+    if (!n || !host_X || !host_out || batch < 1) return fail(GHIP_EINVAL, "bad arguments");
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    const ghip_net_spec& s = n->spec;
+    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
+    TRY(reserve_batch(n, batch));
+    HIP_TRY(hipMemcpyAsync(n->stageX, host_X, (size_t)batch * s.sizes[0] * 4, hipMemcpyHostToDevice, n->stream));
+    uint16_t* xbf = nullptr;
+    if (s.dtype != GHIP_F32) {
+        // the bf16 copy of the staged rows goes to a buffer the forward pass only overwrites after
+        // having consumed it (transposed-input buffer for bf16, activation scratch for fp8)
+        xbf = (s.dtype == GHIP_BF16) ? n->HT[0] : n->Hq;
+        LAUNCH(n, "f32_to_bf16_input", ghip_f32_to_bf16_2d(n->stageX, xbf, nullptr, batch, s.sizes[0], n->stream));
+    }
+    float* res = nullptr;
+    TRY(forward_any(n, n->stageX, xbf, batch, &res));
+    HIP_TRY(hipMemcpyAsync(host_out, res, (size_t)batch * s.sizes[s.n_layers] * 4, hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    return 0;
+}
+
+int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_out)
+{
+    if (!n || batch < 1 || row0 < 0) return fail(GHIP_EINVAL, "bad arguments");
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    if (!n->dX) return fail(GHIP_ESTATE, "no dataset");
+    if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
+    const ghip_net_spec& s = n->spec;
+    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
+    TRY(reserve_batch(n, batch));
+    float* res = nullptr;
+    TRY(forward_any(n, n->dX + row0 * s.sizes[0], n->Xbf ? n->Xbf + row0 * s.sizes[0] : nullptr, batch, &res));
+    if (dev_out) HIP_TRY(hipMemcpyAsync(dev_out, res, (size_t)batch * s.sizes[s.n_layers] * 4, hipMemcpyDeviceToDevice, n->stream));
+    return 0;
+}
+
+int ghip_net_quantize_fp8(ghip_net* n, float* const* host_scales, uint8_t* const* host_codes)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    const ghip_net_spec& s = n->spec;
+    if (!is_canon(n) || s.dtype != GHIP_FP8_INFER) return fail(GHIP_ESTATE, "network was not created with GHIP_FP8_INFER");
+    for (int l = 0; l < s.n_layers; ++l)
+        LAUNCH(n, "quant_weights_e4m3", ghip_quant_rows_e4m3(n->W[l], 0, s.sizes[l + 1], s.sizes[l], n->Wq[l], n->wscale[l], nullptr, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    n->quantized = true;
+    for (int l = 0; l < s.n_layers; ++l) {
+        if (host_scales && host_scales[l]) HIP_TRY(hipMemcpy(host_scales[l], n->wscale[l], (size_t)s.sizes[l + 1] * 4, hipMemcpyDeviceToHost));
+        if (host_codes && host_codes[l]) HIP_TRY(hipMemcpy(host_codes[l], n->Wq[l], (size_t)s.sizes[l + 1] * s.sizes[l], hipMemcpyDeviceToHost));
+    }
+    return 0;
+}
+
+int ghip_net_sync(ghip_net* n)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    return 0;
+}
+
+int ghip_net_profile(ghip_net* n, int enable)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    prof_collect(n);
+    n->prof = enable != 0;
+    return 0;
+}
+int ghip_net_profile_count(ghip_net* n)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    prof_collect(n);
+    return (int)n->aggs.size();
+}
+int ghip_net_profile_entry(ghip_net* n, int index, char* name, int name_len, double* total_ms, int64_t* launches)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    prof_collect(n);
+    if (index < 0 || index >= (int)n->aggs.size()) return fail(GHIP_EINVAL, "profile index out of range");
+    const ProfAgg& g = n->aggs[index];
+    if (name && name_len > 0) { strncpy(name, g.name.c_str(), name_len - 1); name[name_len - 1] = 0; }
+    if (total_ms) *total_ms = g.ms;
+    if (launches) *launches = g.n;
+    return 0;
+}
+int ghip_net_profile_reset(ghip_net* n)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    prof_collect(n);
+    n->aggs.clear();
+    return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,299 @@
+// HBM-bound kernels of the canonical path: output delta / loss / metrics, fused SGD update,
+// bias update, precision conversion, transposition, per-row e4m3 quantisation.
+
+#include "ghip_internal.h"
+
+namespace {
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_sum_d(double v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// One wavefront per row, 16 rows per wavefront, 4 wavefronts per workgroup.
+// Output layer of the canonical mode: softmax (if asked), per-sample loss = sum over outputs of
+// the reference's cost (gmath.cpp:272-321 without the 1/dataSize), the reference's accuracy term
+// (network.cpp:541-547), argmax agreement under gmath.cpp:412-455, and delta = dLoss/dz.
+constexpr int kRowsPerWave = 16;
+__global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
+{
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int row0 = (blockIdx.x * 4 + w) * kRowsPerWave;
+    double loss = 0.0, accs = 0.0, corr = 0.0;
+    const bool softmax = a.act == GHIP_SOFTMAX;
+    const bool sig_bce = (a.act == GHIP_SIGMOID || a.act == GHIP_SIGMOIDP) && a.cost == GHIP_CLASSIFICATION;
+    for (int rr = 0; rr < kRowsPerWave; ++rr) {
+        const int b = row0 + rr;
+        if (b >= a.B) break;
+        float* p = a.P + (long long)b * a.ldp;
+        const float* y = a.Y ? a.Y + (long long)b * a.ldy : nullptr;
+        float inv = 1.0f, mx = 0.0f;
+        if (softmax) {
+            float m = -3.0e38f;
+            for (int o = lane; o < a.n; o += 64) m = fmaxf(m, p[o]);
+            mx = wave_max(m);
+            float s = 0.0f;
+            for (int o = lane; o < a.n; o += 64) s += expf(p[o] - mx);
+            inv = 1.0f / wave_sum(s);
+        }
+        float l = 0.0f, ac = 0.0f;
+        float bp = 0.0f, by = 0.0f;  // running maxima for the argmax rule (start at 0, strict >)
+        int ip = 0x7fffffff, iy = 0x7fffffff;
+        for (int o = lane; o < a.n; o += 64) {
+            float pv = p[o];
+            const float yv = y ? y[o] : 0.0f;
+            float d;
+            if (softmax) {
+                pv = expf(pv - mx) * inv;
+                p[o] = pv;
+                if (yv != 0.0f) l += -(yv * logf(fmaxf(pv, 1e-30f)));
+                d = pv - yv;
+            } else {
+                l += ghip_cost<false>(yv, pv, 1.0f, a.cost);
+                d = sig_bce ? (pv - yv) : ghip_cost_der(yv, pv, a.cost) * ghip_act_der_canon(pv, a.act, a.act_param);
+            }
+            ac += ghip_accuracy_term(pv, yv);
+            if (pv > bp) { bp = pv; ip = o; }
+            if (yv > by) { by = yv; iy = o; }
+            if (a.D) a.D[(long long)b * a.n + o] = d;
+            if (a.Dbf) a.Dbf[(long long)b * a.n + o] = ghip_f32_to_bf16(d);
+        }
+        // argmax across lanes: largest value, lowest index on ties; "no element above 0" = none
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            float ov = __shfl_xor(bp, o, 64); int oi = __shfl_xor(ip, o, 64);
+            if (ov > bp || (ov == bp && oi < ip)) { bp = ov; ip = oi; }
+            ov = __shfl_xor(by, o, 64); oi = __shfl_xor(iy, o, 64);
+            if (ov > by || (ov == by && oi < iy)) { by = ov; iy = oi; }
+        }
+        loss += (double)wave_sum(l);
+        accs += (double)wave_sum(ac);
+        if (ip == iy) corr += 1.0;
+    }
+    __shared__ double red[4][3];
+    if (lane == 0) { red[w][0] = loss; red[w][1] = accs; red[w][2] = corr; }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        double v = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+        atomicAdd(&a.acc[threadIdx.x], v);
+    }
+}
+
+__global__ void __launch_bounds__(256)
+sgd_update_f32_kernel(float* __restrict__ W, float* __restrict__ V, const float* __restrict__ G,
+                      long long n, float lr, float mom, float wd1, float wd2, float gscale)
+{
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long stride = (long long)gridDim.x * 256;
+    for (; i < n; i += stride) {
+        const float w = W[i];
+        const float sg = (w > 0.0f) ? 1.0f : ((w < 0.0f) ? -1.0f : 0.0f);
+        const float g = G[i] * gscale + wd1 * sg + wd2 * w;
+        const float d = lr * g + mom * V[i];
+        V[i] = d;
+        W[i] = w - d;
+    }
+}
+
+// one workgroup per 64 output channels; lanes walk channels (coalesced), wavefronts split rows
+__global__ void __launch_bounds__(256)
+bias_update_f32_kernel(const float* __restrict__ D, int B, int n, int ldd, float* __restrict__ bias,
+                       float* __restrict__ vb, float lr, float mom)
+{
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int o = blockIdx.x * 64 + lane;
+    float s = 0.0f;
+    if (o < n)
+        for (int b = w; b < B; b += 4) s += D[(long long)b * ldd + o];
+    __shared__ float red[4][64];
+    red[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && o < n) {
+        const float g = (red[0][lane] + red[1][lane] + red[2][lane] + red[3][lane]) / (float)B;
+        const float d = lr * g + mom * vb[o];
+        vb[o] = d;
+        bias[o] = bias[o] - d;
+    }
+}
+
+// bf16 delta^T [n][B]: one workgroup per channel
+__global__ void __launch_bounds__(256)
+bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* __restrict__ bias,
+                         float* __restrict__ vb, float lr, float mom)
+{
+    const int o = blockIdx.x;
+    const uint16_t* row = DT + (long long)o * B;
+    float s = 0.0f;
+    for (int b = threadIdx.x; b < B; b += 256) s += ghip_bf16_to_f32(row[b]);
+    s = wave_sum(s);
+    __shared__ float red[4];
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const float g = (red[0] + red[1] + red[2] + red[3]) / (float)B;
+        const float d = lr * g + mom * vb[o];
+        vb[o] = d;
+        bias[o] = bias[o] - d;
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) fill_kernel(T* p, long long n, T v)
+{
+    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long stride = (long long)gridDim.x * 256;
+    for (; i < n; i += stride) p[i] = v;
+}
+
+// 64x64 tile through LDS: dst[r][c] = bf16(src[r][c]) and dstT[c][r]; src fp32 or bf16
+template <typename SrcT>
+__global__ void __launch_bounds__(256)
+convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ dst,
+                         uint16_t* __restrict__ dstT, int rows, int cols)
+{
+    __shared__ uint16_t tile[64][64 + 2];
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int j = ty; j < 64; j += 4) {
+        const int r = r0 + j, c = c0 + tx;
+        uint16_t v = 0;
+        if (r < rows && c < cols) {
+            if (sizeof(SrcT) == 4) v = ghip_f32_to_bf16(((const float*)src)[(long long)r * cols + c]);
+            else v = ((const uint16_t*)src)[(long long)r * cols + c];
+            if (dst) dst[(long long)r * cols + c] = v;
+        }
+        tile[j][tx] = v;
+    }
+    __syncthreads();
+    if (dstT) {
+        for (int j = ty; j < 64; j += 4) {
+            const int c = c0 + j, r = r0 + tx;
+            if (r < rows && c < cols) dstT[(long long)c * rows + r] = tile[tx][j];
+        }
+    }
+}
+
+// one workgroup per row: amax (or a given amax), scale = amax/448, q = e4m3(x / scale)
+template <typename SrcT>
+__global__ void __launch_bounds__(256)
+quant_rows_kernel(const SrcT* __restrict__ src, int rows, int cols, uint8_t* __restrict__ q,
+                  float* __restrict__ scale, const unsigned int* __restrict__ amax_bits)
+{
+    const int r = blockIdx.x;
+    const SrcT* x = src + (long long)r * cols;
+    __shared__ float red[4];
+    float amax;
+    if (amax_bits) {
+        amax = __uint_as_float(amax_bits[r]);
+    } else {
+        float m = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += 256) {
+            float v = (sizeof(SrcT) == 4) ? ((const float*)x)[c] : ghip_bf16_to_f32(((const uint16_t*)x)[c]);
+            m = fmaxf(m, fabsf(v));
+        }
+        m = wave_max(m);
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+        __syncthreads();
+        amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    }
+    const float sc = (amax > 0.0f) ? __fdiv_rn(amax, 448.0f) : 1.0f;
+    if (threadIdx.x == 0) scale[r] = sc;
+    uint8_t* qr = q + (long long)r * cols;
+    for (int c = threadIdx.x; c < cols; c += 256) {
+        float v = (sizeof(SrcT) == 4) ? ((const float*)x)[c] : ghip_bf16_to_f32(((const uint16_t*)x)[c]);
+        qr[c] = ghip_f32_to_e4m3(__fdiv_rn(v, sc));
+    }
+}
+
+inline int grid_for(long long n, int cap = 65535 * 4)
+{
+    long long b = (n + 255) / 256;
+    if (b > cap) b = cap;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+}  // namespace
+
+hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
+{
+    const int rows_per_block = 4 * kRowsPerWave;
+    hipLaunchKernelGGL(output_delta_kernel, dim3((a.B + rows_per_block - 1) / rows_per_block), dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+hipError_t ghip_sgd_update_f32(float* W, float* V, const float* G, long long n, float lr, float mom,
+                               float wd1, float wd2, float gscale, hipStream_t s)
+{
+    hipLaunchKernelGGL(sgd_update_f32_kernel, dim3(grid_for(n, 4096)), dim3(256), 0, s, W, V, G, n, lr, mom,
+                       wd1, wd2, gscale);
+    return hipGetLastError();
+}
+
+hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bias, float* vb, float lr,
+                                float mom, hipStream_t s)
+{
+    hipLaunchKernelGGL(bias_update_f32_kernel, dim3((n + 63) / 64), dim3(256), 0, s, D, B, n, ldd, bias, vb, lr, mom);
+    return hipGetLastError();
+}
+
+hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vb, float lr,
+                                  float mom, hipStream_t s)
+{
+    hipLaunchKernelGGL(bias_update_bf16T_kernel, dim3(n), dim3(256), 0, s, DT, n, B, bias, vb, lr, mom);
+    return hipGetLastError();
+}
+
+hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s)
+{
+    hipLaunchKernelGGL(fill_kernel<float>, dim3(grid_for(n, 2048)), dim3(256), 0, s, p, n, v);
+    return hipGetLastError();
+}
+hipError_t ghip_fill_f64(double* p, long long n, double v, hipStream_t s)
+{
+    hipLaunchKernelGGL(fill_kernel<double>, dim3(grid_for(n, 2048)), dim3(256), 0, s, p, n, v);
+    return hipGetLastError();
+}
+hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream_t s)
+{
+    hipLaunchKernelGGL(fill_kernel<unsigned int>, dim3(grid_for(n, 2048)), dim3(256), 0, s, p, n, v);
+    return hipGetLastError();
+}
+
+hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s)
+{
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, dst, dstT, rows, cols);
+    return hipGetLastError();
+}
+
+hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s)
+{
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols);
+    return hipGetLastError();
+}
+
+hipError_t ghip_quant_rows_e4m3(const void* src, int src_is_bf16, int rows, int cols, uint8_t* q,
+                                float* scale, const unsigned int* amax_bits, hipStream_t s)
+{
+    if (src_is_bf16)
+        hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, dim3(rows), dim3(256), 0, s, (const uint16_t*)src, rows, cols, q, scale, amax_bits);
+    else
+        hipLaunchKernelGGL(quant_rows_kernel<float>, dim3(rows), dim3(256), 0, s, (const float*)src, rows, cols, q, scale, amax_bits);
+    return hipGetLastError();
+}

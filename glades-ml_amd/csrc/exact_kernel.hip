@@ -1,0 +1,286 @@
+// Exact mode: the reference's per-sample sequential training as ONE persistent workgroup.
+//
+// Follows NNetwork::SGDHelper / ForwardPass / BackPropagation
+// ("Backend/Machine Learning/Networks/network.cpp":399-668) and Node::getDelta / applyDeltas
+// ("Backend/Machine Learning/State/node.cpp":278-307) for every row in order.  Samples are
+// strictly sequential (the scalar layer bias and the weights change inside a "minibatch"), so
+// the parallelism is inside a layer only:
+//   forward      one lane per output node, inputs summed in ascending order (node.cpp:82-93)
+//   edge update  one lane per edge (delta push, window sum, conditional apply)
+//   back-prop    one lane per input node, outputs visited in ascending order with the
+//                reference's doubling accumulator  e <- e + (e + d*w)   (network.cpp:660-662)
+//   bias, loss   one designated lane, in the reference's visiting order
+// Every fp32 operation is written with explicit round-to-nearest intrinsics so that nothing is
+// contracted into an FMA or re-associated: the arithmetic order is the reference's.
+//
+// Weights, pending-delta sums and last deltas live in LDS for the whole call (3 floats per edge,
+// rows padded to an odd stride so that lane-per-row and lane-per-column walks are both free of
+// bank conflicts); networks too large for LDS keep them in global memory (L2 resident).
+
+#include "ghip_internal.h"
+
+namespace {
+
+constexpr int kPrefetch = 4;  // values per lane of the next row held in registers
+
+template <bool kLds>
+__global__ void __launch_bounds__(1024)
+exact_kernel(ExactLaunch p)
+{
+    extern __shared__ float smem[];
+    const int tid = threadIdx.x;
+    const int T = blockDim.x;
+    const int serial = T - 1;  // lane that carries the order-dependent scalar chains
+    const int L = p.n_layers;
+    const int n0 = p.sizes[0];
+    const int nout = p.sizes[L];
+    const int S = p.state_floats;
+
+    float* sW;
+    float* sSum;
+    float* sLast;
+    float* nodes;
+    if (kLds) {
+        sW = smem;
+        sSum = smem + S;
+        sLast = smem + 2 * S;
+        nodes = smem + 3 * S;
+    } else {
+        sW = p.W;
+        sSum = p.wsum;
+        sLast = p.wlast;
+        nodes = smem;
+    }
+    float* sa = nodes;                      // node values, all layers
+    float* sd = nodes + p.node_floats;      // d = errDer * derivative of the layer being updated
+    float* sbase = nodes + 2 * p.node_floats;  // lr * d
+    float* sy = nodes + 3 * p.node_floats;  // expected row
+    float* sbias = sy + nout;               // GHIP_MAX_LAYERS scalars
+    int* sflag = (int*)(sbias + GHIP_MAX_LAYERS);
+
+    if (kLds) {
+        for (int k = tid; k < S; k += T) {
+            sW[k] = p.W[k];
+            sSum[k] = p.wsum[k];
+            sLast[k] = p.wlast[k];
+        }
+    }
+    if (tid < GHIP_MAX_LAYERS) sbias[tid] = p.bias[tid];
+    if (tid == 0) sflag[0] = 0;
+
+    const float data_size = (float)((unsigned)p.n_rows * (unsigned)nout);
+    const float fmb = (float)p.mb;
+    const bool small_row = (n0 <= kPrefetch * T) && (nout <= kPrefetch * T);
+
+    // first row into registers
+    float px[kPrefetch], py[kPrefetch];
+#pragma unroll
+    for (int j = 0; j < kPrefetch; ++j) {
+        int i = tid + j * T;
+        px[j] = (small_row && i < n0) ? p.X[i] : 0.0f;
+        py[j] = (small_row && i < nout) ? p.Y[i] : 0.0f;
+    }
+    __syncthreads();
+
+    int ep = 0;
+    for (; ep < p.n_epochs; ++ep) {
+        float tot_err = 0.0f, tot_acc = 0.0f;
+        long long correct = 0;
+        const bool last_epoch = (ep == p.n_epochs - 1) || (p.stop_accuracy > 0.0f);
+        for (long long r = 0; r < p.n_rows; ++r) {
+            // ---- stage the row (prefetched) and start fetching the next one
+            if (small_row) {
+#pragma unroll
+                for (int j = 0; j < kPrefetch; ++j) {
+                    int i = tid + j * T;
+                    if (i < n0) sa[i] = px[j];
+                    if (i < nout) sy[i] = py[j];
+                }
+                long long rn = r + 1;
+                if (rn == p.n_rows) rn = 0;
+                const float* xn = p.X + rn * n0;
+                const float* yn = p.Y + rn * nout;
+#pragma unroll
+                for (int j = 0; j < kPrefetch; ++j) {
+                    int i = tid + j * T;
+                    px[j] = (i < n0) ? xn[i] : 0.0f;
+                    py[j] = (i < nout) ? yn[i] : 0.0f;
+                }
+            } else {
+                for (int i = tid; i < n0; i += T) sa[i] = p.X[r * n0 + i];
+                for (int i = tid; i < nout; i += T) sy[i] = p.Y[r * nout + i];
+            }
+            __syncthreads();
+
+            // ---- ForwardPass (network.cpp:457-516)
+            for (int l = 0; l < L; ++l) {
+                const int ni = p.sizes[l], no = p.sizes[l + 1], ld = p.ld[l];
+                const float* Wl = sW + p.woff[l];
+                const float* ain = sa + p.aoff[l];
+                float* aout = sa + p.aoff[l + 1];
+                const int act = p.act[l];
+                const float par = p.act_param[l];
+                const float bl = sbias[l];
+                for (int o = tid; o < no; o += T) {
+                    const float* w = Wl + o * ld;
+                    float z = 0.0f;
+#pragma unroll 8
+                    for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
+                    if (l != 0) z = __fadd_rn(z, bl);
+                    aout[o] = ghip_squash<true>(z, act, par);
+                }
+                __syncthreads();
+            }
+            const float* pred = sa + p.aoff[L];
+            if (p.preds && last_epoch)
+                for (int o = tid; o < nout; o += T) p.preds[r * nout + o] = pred[o];
+
+            // ---- output metrics in visiting order (network.cpp:519-559)
+            if (tid == serial) {
+                float mp = 0.0f, my = 0.0f;
+                int ip = -1, iy = -1;
+                for (int o = 0; o < nout; ++o) {
+                    const float pr = pred[o], ex = sy[o];
+                    tot_err = __fadd_rn(tot_err, ghip_cost<true>(ex, pr, data_size, p.cost));
+                    tot_acc = __fadd_rn(tot_acc, ghip_accuracy_term(pr, ex));
+                    if (pr > mp) { mp = pr; ip = o; }
+                    if (ex > my) { my = ex; iy = o; }
+                }
+                if (ip == iy) ++correct;
+            }
+
+            if (p.train) {
+                // output layer: errDer = 0 + costErrDer, derivative 1 (network.cpp:599-612)
+                {
+                    float* dl = sd + p.aoff[L];
+                    float* bs = sbase + p.aoff[L];
+                    const float lr = p.lr[L - 1];
+                    for (int o = tid; o < nout; o += T) {
+                        float e = __fadd_rn(0.0f, ghip_cost_der(sy[o], pred[o], p.cost));
+                        dl[o] = e;
+                        bs[o] = __fmul_rn(lr, e);
+                    }
+                }
+                __syncthreads();
+                const bool apply = (r % p.mb) == 0;
+                for (int Lo = L; Lo > 0; --Lo) {
+                    const int l = Lo - 1;
+                    const int ni = p.sizes[l], no = p.sizes[Lo], ld = p.ld[l];
+                    float* Wl = sW + p.woff[l];
+                    float* Sl = sSum + p.woff[l];
+                    float* Ll = sLast + p.woff[l];
+                    const float* ain = sa + p.aoff[l];
+                    const float* dl = sd + p.aoff[Lo];
+                    const float* bs = sbase + p.aoff[Lo];
+                    const float lr = p.lr[l], mom = p.mom[l];
+                    const float w1 = __fmul_rn(p.wd1[l], lr), w2 = __fmul_rn(p.wd2[l], lr);
+                    // ---- per-edge delta push and conditional apply (node.cpp:278-307)
+                    {
+                        const int sh = p.tw_log2[l];
+                        const int tw = 1 << sh;
+                        const int i0 = tid & (tw - 1), o0 = tid >> sh, rpp = T >> sh;
+                        for (int i = i0; i < ni; i += tw) {
+                            const float a = ain[i];
+                            const float t1 = __fmul_rn(w1, fabsf(a));
+                            const float t2 = __fmul_rn(w2, a);
+                            for (int o = o0; o < no; o += rpp) {
+                                const int k = o * ld + i;
+                                float dW = __fadd_rn(__fmul_rn(bs[o], a), __fmul_rn(mom, Ll[k]));
+                                dW = __fadd_rn(dW, t1);
+                                dW = __fadd_rn(dW, t2);
+                                float s = __fadd_rn(Sl[k], dW);
+                                if (apply) {
+                                    Wl[k] = __fsub_rn(Wl[k], __fdiv_rn(s, fmb));
+                                    Sl[k] = 0.0f;
+                                    Ll[k] = 0.0f;
+                                } else {
+                                    Sl[k] = s;
+                                    Ll[k] = dW;
+                                }
+                            }
+                        }
+                    }
+                    // ---- scalar bias of the in-layer (network.cpp:654-656)
+                    if (tid == serial && l != 0) {
+                        float b = sbias[l];
+                        if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
+                            for (int i = 0; i < ni; ++i) {
+#pragma unroll 8
+                                for (int o = 0; o < no; ++o) b = __fsub_rn(b, bs[o]);
+                            }
+                        } else {
+                            float s = 0.0f;
+                            for (int o = 0; o < no; ++o) s = __fadd_rn(s, bs[o]);
+                            b = __fsub_rn(b, __fmul_rn((float)ni, s));
+                        }
+                        sbias[l] = b;
+                    }
+                    __syncthreads();
+                    // ---- error partials of the in-layer with the UPDATED weights
+                    //      (network.cpp:660-662), then its own d and lr*d for the next round
+                    if (l != 0) {
+                        float* dn = sd + p.aoff[l];
+                        float* bn = sbase + p.aoff[l];
+                        const int actp = p.act[l - 1];
+                        const float lrn = p.lr[l - 1];
+                        for (int i = tid; i < ni; i += T) {
+                            float e = 0.0f;
+#pragma unroll 8
+                            for (int o = 0; o < no; ++o)
+                                e = __fadd_rn(e, __fadd_rn(e, __fmul_rn(dl[o], Wl[o * ld + i])));
+                            // the reference always passes 0.01 here (network.cpp:617-618)
+                            float d = __fmul_rn(e, ghip_act_der_ref(ain[i], actp, 0.01f));
+                            dn[i] = d;
+                            bn[i] = __fmul_rn(lrn, d);
+                        }
+                        __syncthreads();
+                    }
+                }
+            }
+        }
+        // ---- end of epoch (network.cpp:193-195, Terminator.cpp:73-74)
+        if (tid == serial) {
+            float acc = __fdiv_rn(tot_acc, __fmul_rn((float)(unsigned)p.n_rows, (float)(unsigned)nout));
+            ghip_metrics* m = ((ghip_metrics*)p.metrics) + ep;
+            m->loss = tot_err;
+            m->accuracy = acc;
+            m->correct = correct;
+            if (p.stop_accuracy > 0.0f && acc >= p.stop_accuracy) sflag[0] = 1;
+        }
+        __syncthreads();
+        if (sflag[0]) { ++ep; break; }
+    }
+
+    if (kLds) {
+        for (int k = tid; k < S; k += T) {
+            p.W[k] = sW[k];
+            p.wsum[k] = sSum[k];
+            p.wlast[k] = sLast[k];
+        }
+    }
+    if (tid < GHIP_MAX_LAYERS) p.bias[tid] = sbias[tid];
+    if (tid == 0) p.epochs_run[0] = ep;
+}
+
+}  // namespace
+
+size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds)
+{
+    size_t f = (size_t)3 * p.node_floats + p.sizes[p.n_layers] + GHIP_MAX_LAYERS + 4;
+    if (state_in_lds) f += (size_t)3 * p.state_floats;
+    return f * sizeof(float);
+}
+
+hipError_t ghip_launch_exact(const ExactLaunch& p, int threads, size_t lds_bytes, hipStream_t s)
+{
+    hipError_t e;
+    if (p.state_in_lds) {
+        e = hipFuncSetAttribute((const void*)exact_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(exact_kernel<true>, dim3(1), dim3(threads), lds_bytes, s, p);
+    } else {
+        hipLaunchKernelGGL(exact_kernel<false>, dim3(1), dim3(threads), lds_bytes, s, p);
+    }
+    return hipGetLastError();
+}

@@ -1,0 +1,274 @@
+// Internal declarations shared by the HIP translation units of libglades_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/glades_hip.h"
+
+#define GHIP_OUTLIER 0.046f  // knee of RELU / LEAKY in the reference (gmath.h:35, gmath.cpp:62-82)
+
+// ---------------------------------------------------------------- element-wise device functions
+
+// Reference GMath::squash (gmath.cpp:22-101).  kPrecise selects transcendental evaluation in
+// double rounded once to float, which tracks glibc's float routines to the last bit far more
+// often than the fast fp32 device routines do (exact mode is sequential and order-faithful,
+// so the transcendental is the only remaining source of divergence from the CPU path).
+template <bool kPrecise>
+__device__ __forceinline__ float ghip_tanh(float z)
+{
+    if (kPrecise) return (float)tanh((double)z);
+    return tanhf(z);
+}
+template <bool kPrecise>
+__device__ __forceinline__ float ghip_exp(float z)
+{
+    if (kPrecise) return (float)exp((double)z);
+    return expf(z);
+}
+template <bool kPrecise>
+__device__ __forceinline__ float ghip_log(float z)
+{
+    if (kPrecise) return (float)log((double)z);
+    return logf(z);
+}
+
+template <bool kPrecise>
+__device__ __forceinline__ float ghip_squash(float z, int act, float p)
+{
+    switch (act) {
+    case GHIP_TANH: return ghip_tanh<kPrecise>(z);
+    case GHIP_TANHP:
+        if (z > 1.0f - p) return 1.0f;
+        if (z < p - 1.0f) return -1.0f;
+        return ghip_tanh<kPrecise>(z);
+    case GHIP_SIGMOID: return __fdiv_rn(1.0f, __fadd_rn(1.0f, ghip_exp<kPrecise>(-z)));
+    case GHIP_SIGMOIDP:
+        if (z < p) return 0.01f;
+        if (z > 1.0f - p) return 0.99f;
+        return __fdiv_rn(1.0f, __fadd_rn(1.0f, ghip_exp<kPrecise>(-z)));
+    case GHIP_RELU: return (z < GHIP_OUTLIER) ? 0.0f : z;
+    case GHIP_LEAKY: return (z < GHIP_OUTLIER) ? __fmul_rn(p, z) : z;
+    case GHIP_LINEAR: return __fmul_rn(p, z);
+    case GHIP_STEP: return (z < p) ? 0.0f : 1.0f;
+    }
+    return 0.0f;
+}
+
+// Reference GMath::activationErrDer (gmath.cpp:182-245), in terms of the activation's output.
+__device__ __forceinline__ float ghip_act_der_ref(float a, int act, float p)
+{
+    switch (act) {
+    case GHIP_TANH:
+    case GHIP_TANHP: return __fsub_rn(1.0f, __fmul_rn(a, a));
+    case GHIP_SIGMOID:
+    case GHIP_SIGMOIDP: return __fmul_rn(a, __fsub_rn(1.0f, a));
+    case GHIP_RELU: return (a > 0.0f) ? 1.0f : 0.0f;
+    case GHIP_LEAKY:
+        if (a > 0.0f) return 1.0f;
+        return (p < 0) ? p : -p;
+    case GHIP_LINEAR: return p;
+    case GHIP_STEP: return 0.0f;
+    }
+    return 1.0f;
+}
+
+// Canonical-mode derivative: the layer's own parameter, LEAKY slope = +param.
+__device__ __forceinline__ float ghip_act_der_canon(float a, int act, float p)
+{
+    if (act == GHIP_LEAKY) return (a > 0.0f) ? 1.0f : p;
+    return ghip_act_der_ref(a, act, p);
+}
+
+// Reference GMath::outputNodeCost (gmath.cpp:272-321)
+template <bool kPrecise>
+__device__ __forceinline__ float ghip_cost(float e, float p, float data_size, int cost)
+{
+    float c = 0.0f;
+    switch (cost) {
+    case GHIP_REGRESSION: {
+        float d = __fsub_rn(e, p);
+        c = __fdiv_rn(__fmul_rn(d, d), data_size);
+        break;
+    }
+    case GHIP_CLASSIFICATION: {
+        float t0 = __fmul_rn(e, ghip_log<kPrecise>(p));
+        float t1 = __fmul_rn(__fsub_rn(1.0f, e), ghip_log<kPrecise>(__fsub_rn(1.0f, p)));
+        c = __fdiv_rn(-__fadd_rn(t0, t1), data_size);
+        break;
+    }
+    case GHIP_KL: c = __fdiv_rn(ghip_log<kPrecise>(__fdiv_rn(e, p)), data_size); break;
+    }
+    return c;
+}
+
+// Reference GMath::costErrDer (gmath.cpp:323-353)
+__device__ __forceinline__ float ghip_cost_der(float e, float p, int cost)
+{
+    switch (cost) {
+    case GHIP_REGRESSION: return __fmul_rn(2.0f, __fsub_rn(p, e));
+    case GHIP_CLASSIFICATION:
+        return __fdiv_rn(__fsub_rn(p, e), __fmul_rn(__fsub_rn(1.0f, p), p));
+    case GHIP_KL: return -__fdiv_rn(e, p);
+    }
+    return 1.0f;
+}
+
+// Reference accuracy contribution (network.cpp:541-547 + gmath.cpp:252-270)
+__device__ __forceinline__ float ghip_accuracy_term(float pred, float expect)
+{
+    float pe = __fsub_rn(pred, expect);
+    if (pe < 0.0f) pe = -pe;
+    if (pe > 1.0f) pe = 1.0f;
+    float acc = __fmul_rn(__fsub_rn(1.0f, pe), 100.0f);
+    return acc < 0.0f ? 0.0f : acc;
+}
+
+// ---------------------------------------------------------------- bf16 helpers (bit level)
+
+__device__ __forceinline__ uint16_t ghip_f32_to_bf16(float x)
+{
+    uint32_t u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float ghip_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+
+// OCP e4m3 (finite only) encode, round-to-nearest-even, saturating at 448.
+__device__ __forceinline__ uint8_t ghip_f32_to_e4m3(float x)
+{
+    uint32_t u = __float_as_uint(x);
+    uint8_t sign = (uint8_t)((u >> 31) << 7);
+    float a = fabsf(x);
+    if (a != a) return (uint8_t)(sign | 0x7f);
+    if (a >= 448.0f) return (uint8_t)(sign | 0x7e);
+    if (a < 0.015625f) return (uint8_t)(sign | (int)rintf(a * 512.0f));
+    uint32_t ua = __float_as_uint(a);
+    int ex = (int)(ua >> 23) - 127;
+    // keep 3 mantissa bits, RNE on the 20 dropped bits
+    uint32_t mant = ua & 0x7fffffu;
+    uint32_t q = mant >> 20;
+    uint32_t rem = mant & 0xfffffu;
+    if (rem > 0x80000u || (rem == 0x80000u && (q & 1u))) ++q;
+    if (q == 8) { q = 0; ++ex; }
+    int code = ((ex + 7) << 3) | (int)q;
+    if (code > 0x7e) code = 0x7e;
+    return (uint8_t)(sign | code);
+}
+
+// ---------------------------------------------------------------- exact mode (exact_kernel.hip)
+
+struct ExactLaunch {
+    int   n_layers;
+    int   sizes[GHIP_MAX_LAYERS + 1];
+    int   ld[GHIP_MAX_LAYERS];      // padded row stride of layer l in the state arrays (odd)
+    int   woff[GHIP_MAX_LAYERS];    // offset of layer l in the state arrays
+    int   aoff[GHIP_MAX_LAYERS + 1];// offset of layer l's node values in the node arrays
+    int   tw_log2[GHIP_MAX_LAYERS]; // log2 of the lane group width used to walk layer l's edges
+    float lr[GHIP_MAX_LAYERS], mom[GHIP_MAX_LAYERS], wd1[GHIP_MAX_LAYERS], wd2[GHIP_MAX_LAYERS];
+    int   act[GHIP_MAX_LAYERS];
+    float act_param[GHIP_MAX_LAYERS];
+    int   mb, cost, bias_mode;
+    int   state_floats;             // total padded floats of one state array
+    int   node_floats;              // total node values
+    int   n_epochs, train;
+    float stop_accuracy;
+    long long n_rows;
+    const float* X;
+    const float* Y;
+    float* W;      // [state_floats] padded weights (global copy, read at start, written at end)
+    float* wsum;   // pending-delta running sums
+    float* wlast;  // last pending delta
+    float* bias;   // [GHIP_MAX_LAYERS] scalar layer biases
+    float* preds;  // n_rows x n_out or NULL
+    float* metrics;// per epoch: loss, accuracy, correct (as float bits of an int), spare
+    int*   epochs_run;
+    int    state_in_lds;
+};
+
+hipError_t ghip_launch_exact(const ExactLaunch& p, int threads, size_t lds_bytes, hipStream_t s);
+size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds);
+
+// ---------------------------------------------------------------- canonical kernels
+
+// C[M][N] (+epilogue) = A x B, fp32 via MFMA.  a_kmajor: A is stored [K][M] (else [M][K]);
+// b_kmajor: B is stored [K][N] (else [N][K]).
+enum GemmEpilogue {
+    EPI_STORE = 0,        // C = acc * alpha
+    EPI_BIAS_ACT = 1,     // C = squash(acc + bias[n])
+    EPI_MUL_DER = 2,      // C = acc * act_der(aux[m][n])
+};
+struct GemmF32Args {
+    const float* A; const float* B; float* C;
+    int M, N, K;
+    int lda, ldb, ldc;
+    int a_kmajor, b_kmajor;
+    int epilogue;
+    const float* bias;   // EPI_BIAS_ACT (may be NULL)
+    const float* aux;    // EPI_MUL_DER: activations [M][N], ld = ldc
+    int act; float act_param;
+    float alpha;
+};
+hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s);
+
+// softmax / output delta / metrics for fp32 logits-or-activations P[B][n] against Y[B][n].
+// If act == SOFTMAX, P holds pre-softmax logits and is overwritten with probabilities.
+// D (fp32, may be NULL) receives dL/dz; Dbf/DbfT (bf16 [B][n] and [n][B], may be NULL) too.
+// acc: 4 doubles {loss sum, accuracy sum, correct count, unused}, atomically accumulated.
+struct DeltaArgs {
+    float* P; const float* Y; float* D; uint16_t* Dbf; uint16_t* DbfT;
+    int B, n, ldp, ldy;
+    int act; float act_param; int cost;
+    double* acc;
+};
+hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s);
+
+// Fused SGD + momentum + L1/L2 update:  d = lr*(g*gscale + wd1*sign(w) + wd2*w) + mom*v; v = d; w -= d
+hipError_t ghip_sgd_update_f32(float* W, float* V, const float* G, long long n, float lr, float mom,
+                               float wd1, float wd2, float gscale, hipStream_t s);
+// gb[o] = sum_b D[b][o] (fp32 D [B][n]) fused with the bias update (no decay)
+hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bias, float* vbias,
+                                float lr, float mom, hipStream_t s);
+hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s);
+hipError_t ghip_fill_f64(double* p, long long n, double v, hipStream_t s);
+
+// ---------------------------------------------------------------- low precision (gemm_lp.hip)
+
+enum LpEpilogue {
+    LP_FWD_ACT = 0,     // out bf16 [M][N] (+ transposed copy [N][M]) = squash(acc + bias[n])
+    LP_FWD_F32 = 1,     // out fp32 [M][N] = squash(acc + bias[n])   (output layer; softmax logits use LINEAR 1)
+    LP_DGRAD = 2,       // out bf16 (+T) = acc * act_der(aux bf16 [M][N])
+    LP_WGRAD_SGD = 3,   // acc = batch-summed gradient tile [M=n_out][N=n_in]: fused update of
+                        // fp32 master + momentum, writes bf16 W [M][N] and W^T [N][M]
+    LP_FP8_ACT = 4,     // fp8 inference: v = squash(acc * rs[m] * cs[n]); bf16 out + row amax
+    LP_FP8_F32 = 5      // fp8 inference last layer: fp32 out = squash(acc * rs[m] * cs[n])
+};
+struct GemmLpArgs {
+    const void* A; const void* B;    // [M][K], [N][K], K contiguous; bf16 or e4m3
+    int M, N, K;
+    int fp8;                          // 0: bf16 operands, 1: e4m3 operands
+    int epilogue;
+    void* out; void* outT;            // see LpEpilogue; outT may be NULL
+    const float* bias;                // [N] or NULL
+    const uint16_t* aux;              // LP_DGRAD: activations bf16 [M][N]
+    int act; float act_param;
+    // LP_WGRAD_SGD
+    float* master; float* mom; float lr, momf, wd1, wd2, gscale;
+    // fp8
+    const float* row_scale; const float* col_scale; unsigned int* row_amax_bits;
+};
+hipError_t ghip_gemm_lp(const GemmLpArgs& a, hipStream_t s);
+bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8);
+
+hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
+hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s);
+// bias update from bf16 delta^T [n][B] rows (contiguous): gb[o] = sum_b
+hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vbias, float lr,
+                                  float mom, hipStream_t s);
+// per-row e4m3 quantisation: src fp32/bf16 [rows][cols]; scale = amax/448 (1 if row is zero).
+// amax_bits: if non-NULL the row amax is taken from there (uint bits of a non-negative float)
+// instead of being reduced from the row.
+hipError_t ghip_quant_rows_e4m3(const void* src, int src_is_bf16, int rows, int cols, uint8_t* q,
+                                float* scale, const unsigned int* amax_bits, hipStream_t s);
+hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream_t s);

@@ -1,0 +1,245 @@
+"""ctypes binding of libglades_hip.so (the C ABI in include/glades_hip.h).
+
+No CPU fallback: if the library is missing or no gfx950 device is usable, calls raise.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.dirname(HERE)
+LIB_PATH = os.path.join(PKG, "libglades_hip.so")
+MAX_LAYERS = 16
+
+TANH, TANHP, SIGMOID, SIGMOIDP, LINEAR, RELU, LEAKY, STEP, SOFTMAX = range(9)
+REGRESSION, CLASSIFICATION, KL = range(3)
+MODE_EXACT, MODE_CANONICAL = 0, 1
+F32, BF16, FP8_INFER = 0, 1, 2
+BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
+
+EXPORTS = [
+    "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
+    "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact",
+    "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident",
+    "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
+    "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
+]
+
+
+class Spec(C.Structure):
+    _fields_ = [
+        ("n_layers", C.c_int),
+        ("sizes", C.c_int * (MAX_LAYERS + 1)),
+        ("lr", C.c_float * MAX_LAYERS),
+        ("mom", C.c_float * MAX_LAYERS),
+        ("wd1", C.c_float * MAX_LAYERS),
+        ("wd2", C.c_float * MAX_LAYERS),
+        ("act", C.c_int * MAX_LAYERS),
+        ("act_param", C.c_float * MAX_LAYERS),
+        ("batch", C.c_int),
+        ("cost", C.c_int),
+        ("mode", C.c_int),
+        ("dtype", C.c_int),
+        ("bias_mode", C.c_int),
+    ]
+
+
+class Metrics(C.Structure):
+    _fields_ = [("loss", C.c_float), ("accuracy", C.c_float), ("correct", C.c_int64)]
+
+
+class GladesHipError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load():
+    """Loads the built library (raises if it was not built: there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise GladesHipError(f"{LIB_PATH} is missing: build it with `python glades-ml_amd/build.py`")
+        L = C.CDLL(LIB_PATH)
+        vp, i, f, i64 = C.c_void_p, C.c_int, C.c_float, C.c_int64
+        sig = {
+            "ghip_init": (i, [i]),
+            "ghip_net_create": (i, [C.POINTER(Spec), C.POINTER(vp)]),
+            "ghip_net_destroy": (i, [vp]),
+            "ghip_net_set_params": (i, [vp, i, vp, vp, i]),
+            "ghip_net_get_params": (i, [vp, i, vp, vp, i]),
+            "ghip_net_set_dataset": (i, [vp, vp, vp, i64]),
+            "ghip_net_set_dataset_device": (i, [vp, vp, vp, i64]),
+            "ghip_net_run_epochs_exact": (i, [vp, i, i, f, vp, C.POINTER(i), vp]),
+            "ghip_net_train_step": (i, [vp, i64, i, vp]),
+            "ghip_net_last_metrics": (i, [vp, C.POINTER(Metrics)]),
+            "ghip_net_forward": (i, [vp, vp, i, vp]),
+            "ghip_net_forward_resident": (i, [vp, i64, i, vp]),
+            "ghip_net_quantize_fp8": (i, [vp, vp, vp]),
+            "ghip_net_sync": (i, [vp]),
+            "ghip_net_profile": (i, [vp, i]),
+            "ghip_net_profile_count": (i, [vp]),
+            "ghip_net_profile_entry": (i, [vp, i, C.c_char_p, i, C.POINTER(C.c_double), C.POINTER(i64)]),
+            "ghip_net_profile_reset": (i, [vp]),
+            "ghip_last_error": (C.c_char_p, []),
+            "ghip_version": (C.c_char_p, []),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def _check(rc):
+    if rc != 0:
+        raise GladesHipError(f"[{rc}] {load().ghip_last_error().decode()}")
+
+
+def make_spec(sizes, acts, lr=0.01, mom=0.0, wd1=0.0, wd2=0.0, act_params=0.0, batch=1, cost=REGRESSION,
+              mode=MODE_EXACT, dtype=F32, bias_mode=BIAS_SEQUENTIAL):
+    nl = len(sizes) - 1
+
+    def per(v):
+        return list(v) if isinstance(v, (list, tuple, np.ndarray)) else [v] * nl
+
+    s = Spec()
+    s.n_layers = nl
+    for k, v in enumerate(sizes):
+        s.sizes[k] = int(v)
+    for name, v in (("lr", lr), ("mom", mom), ("wd1", wd1), ("wd2", wd2), ("act_param", act_params)):
+        arr = getattr(s, name)
+        for k, x in enumerate(per(v)):
+            arr[k] = float(x)
+    for k, a in enumerate(per(acts)):
+        s.act[k] = int(a)
+    s.batch, s.cost, s.mode, s.dtype, s.bias_mode = int(batch), int(cost), int(mode), int(dtype), int(bias_mode)
+    return s
+
+
+def _ptr(a):
+    return None if a is None else C.c_void_p(a.ctypes.data)
+
+
+class Net:
+    """One device-side network (owns a stream).  Host arrays are numpy float32."""
+
+    def __init__(self, spec, device=0):
+        self.lib = load()
+        _check(self.lib.ghip_init(device))
+        self.spec = spec
+        self.sizes = [spec.sizes[k] for k in range(spec.n_layers + 1)]
+        self.nl = spec.n_layers
+        h = C.c_void_p()
+        _check(self.lib.ghip_net_create(C.byref(spec), C.byref(h)))
+        self.h = h
+        self.n_rows = 0
+
+    def close(self):
+        if getattr(self, "h", None):
+            self.lib.ghip_net_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    # ---- parameters
+    def set_params(self, l, W, bias=None):
+        W = np.ascontiguousarray(W, np.float32)
+        assert W.shape == (self.sizes[l + 1], self.sizes[l])
+        if bias is None:
+            _check(self.lib.ghip_net_set_params(self.h, l, _ptr(W), None, 0))
+        else:
+            b = np.ascontiguousarray(np.atleast_1d(bias), np.float32)
+            _check(self.lib.ghip_net_set_params(self.h, l, _ptr(W), _ptr(b), b.size))
+
+    def get_params(self, l):
+        W = np.empty((self.sizes[l + 1], self.sizes[l]), np.float32)
+        blen = 1 if self.spec.mode == MODE_EXACT else self.sizes[l + 1]
+        b = np.zeros((blen,), np.float32)
+        _check(self.lib.ghip_net_get_params(self.h, l, _ptr(W), _ptr(b), blen))
+        return W, b
+
+    # ---- data
+    def set_dataset(self, X, Y):
+        X = np.ascontiguousarray(X, np.float32)
+        Y = None if Y is None else np.ascontiguousarray(Y, np.float32)
+        assert X.shape[1] == self.sizes[0]
+        _check(self.lib.ghip_net_set_dataset(self.h, _ptr(X), _ptr(Y), X.shape[0]))
+        self.n_rows = X.shape[0]
+
+    def set_dataset_device(self, x_ptr, y_ptr, n_rows):
+        """x_ptr / y_ptr: integer device addresses of fp32 tables the caller keeps alive."""
+        _check(self.lib.ghip_net_set_dataset_device(self.h, C.c_void_p(x_ptr), C.c_void_p(y_ptr) if y_ptr else None, n_rows))
+        self.n_rows = n_rows
+
+    # ---- exact mode
+    def run_epochs_exact(self, n_epochs, train=True, stop_accuracy=0.0, want_preds=False):
+        ms = (Metrics * n_epochs)()
+        ran = C.c_int(0)
+        preds = np.empty((self.n_rows, self.sizes[-1]), np.float32) if want_preds else None
+        _check(self.lib.ghip_net_run_epochs_exact(self.h, n_epochs, 1 if train else 0, float(stop_accuracy),
+                                                  C.cast(ms, C.c_void_p), C.byref(ran), _ptr(preds)))
+        out = [(ms[k].loss, ms[k].accuracy, ms[k].correct) for k in range(ran.value)]
+        return out, preds
+
+    # ---- canonical mode
+    def train_step(self, row0, batch, want_metrics=True):
+        if want_metrics:
+            m = Metrics()
+            _check(self.lib.ghip_net_train_step(self.h, row0, batch, C.cast(C.byref(m), C.c_void_p)))
+            return m
+        _check(self.lib.ghip_net_train_step(self.h, row0, batch, None))
+        return None
+
+    def last_metrics(self):
+        m = Metrics()
+        _check(self.lib.ghip_net_last_metrics(self.h, C.byref(m)))
+        return m
+
+    def forward(self, X):
+        X = np.ascontiguousarray(X, np.float32)
+        out = np.empty((X.shape[0], self.sizes[-1]), np.float32)
+        _check(self.lib.ghip_net_forward(self.h, _ptr(X), X.shape[0], _ptr(out)))
+        return out
+
+    def forward_resident(self, row0, batch, out_ptr=None):
+        _check(self.lib.ghip_net_forward_resident(self.h, row0, batch, C.c_void_p(out_ptr) if out_ptr else None))
+
+    def quantize_fp8(self, want=True):
+        if not want:
+            _check(self.lib.ghip_net_quantize_fp8(self.h, None, None))
+            return None, None
+        scales = [np.empty((self.sizes[l + 1],), np.float32) for l in range(self.nl)]
+        codes = [np.empty((self.sizes[l + 1], self.sizes[l]), np.uint8) for l in range(self.nl)]
+        sp = (C.c_void_p * self.nl)(*[s.ctypes.data for s in scales])
+        cp = (C.c_void_p * self.nl)(*[c.ctypes.data for c in codes])
+        _check(self.lib.ghip_net_quantize_fp8(self.h, C.cast(sp, C.c_void_p), C.cast(cp, C.c_void_p)))
+        return codes, scales
+
+    def sync(self):
+        _check(self.lib.ghip_net_sync(self.h))
+
+    # ---- profiling
+    def profile(self, enable=True):
+        _check(self.lib.ghip_net_profile(self.h, 1 if enable else 0))
+
+    def profile_reset(self):
+        _check(self.lib.ghip_net_profile_reset(self.h))
+
+    def profile_table(self):
+        n = self.lib.ghip_net_profile_count(self.h)
+        out = {}
+        for k in range(n):
+            name = C.create_string_buffer(96)
+            ms = C.c_double()
+            cnt = C.c_int64()
+            _check(self.lib.ghip_net_profile_entry(self.h, k, name, 96, C.byref(ms), C.byref(cnt)))
+            out[name.value.decode()] = (ms.value, cnt.value)
+        return out

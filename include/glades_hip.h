@@ -1,0 +1,163 @@
+/*
+ * glades_hip.h -- C ABI of the MI355X (gfx950) dense feed-forward path for Glades.
+ *
+ * The reference (Gattic/glades-ml) has no plugin or FFI interface: its boundary for this
+ * path is the C++ class API (NNInfo / NNetwork / Terminator / DataInput / glades::train).
+ * These entry points are what a binding of that API to the GPU needs; each one names the
+ * reference code it stands in for ("ML/" = "Backend/Machine Learning/").  The C++ mirror of
+ * the class API that sits on top of this header is glades-ml_amd/host/glades.h.
+ *
+ * Conventions: every function returns 0 on success and a negative GHIP_E* code on failure
+ * (no exceptions, nothing is thrown across the boundary); ghip_last_error() gives the
+ * message of the calling thread's last failure.  Pointers named host_* are host memory the
+ * caller owns; pointers named dev_* are device memory the caller owns and keeps alive while
+ * the network uses it.  Everything else on the device is owned by the handle.  A handle owns
+ * one HIP stream; calls on one handle must not overlap (same as the reference: single
+ * threaded per network); different handles are independent.
+ *
+ * Matrices are dense row-major.  Weights of weight-layer l are [sizes[l+1]][sizes[l]]
+ * (row o = the incoming edges of node o, the reference's Node::edges order, node.h:45).
+ */
+#ifndef GLADES_HIP_H
+#define GLADES_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GHIP_MAX_LAYERS 16
+
+/* activation ids = ML/GMath/gmath.h:43-50; SOFTMAX (canonical mode, output layer only) is an
+ * extension the reference does not have */
+enum { GHIP_TANH = 0, GHIP_TANHP = 1, GHIP_SIGMOID = 2, GHIP_SIGMOIDP = 3, GHIP_LINEAR = 4,
+       GHIP_RELU = 5, GHIP_LEAKY = 6, GHIP_STEP = 7, GHIP_SOFTMAX = 8 };
+/* cost ids = ML/GMath/gmath.h:38-40 */
+enum { GHIP_REGRESSION = 0, GHIP_CLASSIFICATION = 1, GHIP_KL = 2 };
+
+enum {
+    GHIP_MODE_EXACT = 0,     /* the reference's per-sample sequential semantics, quirk for quirk
+                                (ML/Networks/network.cpp:399-668) */
+    GHIP_MODE_CANONICAL = 1  /* batched training: reference forward, true dL/dz backward,
+                                per-channel bias, momentum across steps */
+};
+enum {
+    GHIP_F32 = 0,       /* fp32 storage and arithmetic */
+    GHIP_BF16 = 1,      /* canonical only: bf16 weights/activations, fp32 accumulate, fp32 master */
+    GHIP_FP8_INFER = 2  /* canonical, forward only: e4m3 weights (per-output-channel scale) and
+                           e4m3 activations (per-row scale), fp32 accumulate */
+};
+enum { GHIP_BIAS_SEQUENTIAL = 0, /* exact mode: repeat "bias -= lr*delta" once per (input, output)
+                                    pair in the reference's order (network.cpp:654-656) */
+       GHIP_BIAS_CLOSED_FORM = 1 /* exact mode: bias -= n_in * sum_o(lr*delta_o), one rounding
+                                    instead of n_in*n_out; faster, not bit-faithful */ };
+
+#define GHIP_EINVAL   (-1)  /* bad argument / unsupported shape for the chosen dtype */
+#define GHIP_ENOMEM   (-2)
+#define GHIP_EHIP     (-3)  /* a HIP runtime call failed */
+#define GHIP_ESTATE   (-4)  /* call order: no dataset, wrong mode, ... */
+#define GHIP_ENODEV   (-5)  /* no usable gfx950 device */
+
+typedef struct ghip_net ghip_net;
+
+/* Resolved hyper-parameters: what NNInfo's index-shifted getters return for weight layer l
+ * (ML/Structure/nninfo.cpp:240-373: index 0 reads the input row, index k the hidden row k-1). */
+typedef struct {
+    int   n_layers;                    /* weight layers = hidden layers + 1, 1..GHIP_MAX_LAYERS */
+    int   sizes[GHIP_MAX_LAYERS + 1];  /* sizes[0] features ... sizes[n_layers] outputs */
+    float lr[GHIP_MAX_LAYERS];
+    float mom[GHIP_MAX_LAYERS];
+    float wd1[GHIP_MAX_LAYERS];
+    float wd2[GHIP_MAX_LAYERS];
+    int   act[GHIP_MAX_LAYERS];        /* activation producing layer l+1 */
+    float act_param[GHIP_MAX_LAYERS];
+    int   batch;                       /* NNInfo::getBatchSize(); exact mode needs >= 1 */
+    int   cost;                        /* NNInfo::getOutputType() */
+    int   mode;                        /* GHIP_MODE_* */
+    int   dtype;                       /* GHIP_F32 / GHIP_BF16 / GHIP_FP8_INFER */
+    int   bias_mode;                   /* GHIP_BIAS_* (exact mode) */
+} ghip_net_spec;
+
+/* Per-epoch (exact) or per-step (canonical) figures.
+ * exact:     loss = overallTotalError, accuracy = overallTotalAccuracy (network.cpp:533-547,194-195)
+ * canonical: loss = mean per-sample loss, accuracy = the same 0..100 measure over the batch
+ * correct = rows whose argmax equals the label's under the reference rule (gmath.cpp:412-455) */
+typedef struct {
+    float   loss;
+    float   accuracy;
+    int64_t correct;
+} ghip_metrics;
+
+/* Selects the device and checks that it is a gfx950.  Stands in for glades::init()
+ * (ML/main.cpp:51-56) as the once-per-process set-up call. */
+int ghip_init(int device_ordinal);
+
+/* Builds the device-side network: replaces LayerBuilder::build (ML/State/LayerBuilder.cpp:54-98)
+ * minus the weight sampling, which stays with the caller (ghip_net_set_params). */
+int ghip_net_create(const ghip_net_spec* spec, ghip_net** out);
+int ghip_net_destroy(ghip_net* net);
+
+/* Weight / bias transfer: replaces Node::setEdgeWeight / getEdgeWeight (ML/State/node.cpp:60-66,
+ * 142-148) and Layer::setBiasWeight / getBiasWeight (ML/State/layer.cpp:52-74).
+ * exact mode:     bias_len is 0 or 1; the scalar is the bias of layer `layer` (added to layer
+ *                 layer+1; ignored for layer 0, network.cpp:501-502).
+ * canonical mode: bias_len is 0 or sizes[layer+1] (per output channel).
+ * host_W may be NULL in get to fetch the bias only.  Setting parameters clears momentum. */
+int ghip_net_set_params(ghip_net* net, int layer, const float* host_W, const float* host_bias, int bias_len);
+int ghip_net_get_params(ghip_net* net, int layer, float* host_W, float* host_bias, int bias_len);
+
+/* Uploads the training table once: replaces LayerBuilder::buildInputLayers
+ * (ML/State/LayerBuilder.cpp:100-190) and DataInput::getTrainRow / getTrainExpectedRow
+ * (ML/DataObjects/DataInput.h:39-40).  X is N x sizes[0], Y is N x sizes[n_layers]. */
+int ghip_net_set_dataset(ghip_net* net, const float* host_X, const float* host_Y, int64_t n_rows);
+/* Same, for tables already resident in device memory (fp32); nothing is copied. */
+int ghip_net_set_dataset_device(ghip_net* net, const float* dev_X, const float* dev_Y, int64_t n_rows);
+
+/* Exact mode: n_epochs passes over the rows in order, each row = SGDHelper
+ * (ML/Networks/network.cpp:399-455: ForwardPass :457-575, BackPropagation :577-668), one kernel
+ * launch for the whole call.  train = 0 is the RUN_TEST pass (forward and metrics only).
+ * stop_accuracy > 0 ends the call after the first epoch whose accuracy reaches it
+ * (Terminator::triggered, ML/State/Terminator.cpp:73-74).  host_metrics receives one entry per
+ * epoch run (n_epochs entries of room); *epochs_run says how many.  host_preds (may be NULL)
+ * receives the last epoch's predictions, n_rows x sizes[n_layers]. */
+int ghip_net_run_epochs_exact(ghip_net* net, int n_epochs, int train, float stop_accuracy,
+                              ghip_metrics* host_metrics, int* epochs_run, float* host_preds);
+
+/* Canonical mode: one training step (forward, backward, update) on rows [row0, row0+batch) of
+ * the resident table.  host_metrics may be NULL (then the call does not synchronise). */
+int ghip_net_train_step(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);
+/* Metrics of the most recent ghip_net_train_step (synchronises). */
+int ghip_net_last_metrics(ghip_net* net, ghip_metrics* host_metrics);
+
+/* Canonical mode forward of `batch` rows: the reference forward (network.cpp:457-516) as GEMMs.
+ * host_X: batch x sizes[0] fp32, host_out: batch x sizes[n_layers] fp32. */
+int ghip_net_forward(ghip_net* net, const float* host_X, int batch, float* host_out);
+/* Forward of rows [row0,row0+batch) of the resident table; the result stays on the device and
+ * dev_out (fp32, batch x sizes[n_layers], may be NULL) receives a device-to-device copy. */
+int ghip_net_forward_resident(ghip_net* net, int64_t row0, int batch, float* dev_out);
+
+/* GHIP_FP8_INFER: quantises the current fp32 weights to e4m3 with one fp32 scale per output
+ * channel (scale = amax(row)/448).  host_scales[l] (may be NULL) receives sizes[l+1] scales and
+ * host_codes[l] (may be NULL) the sizes[l+1]*sizes[l] code bytes.  No reference counterpart (the
+ * reference is fp32 only); checked against its fp32 forward on the dequantised weights. */
+int ghip_net_quantize_fp8(ghip_net* net, float* const* host_scales, uint8_t* const* host_codes);
+
+/* Blocks until everything queued on the handle's stream has finished. */
+int ghip_net_sync(ghip_net* net);
+
+/* Per-kernel timing with HIP events on the handle's stream.  While enabled, every kernel launch
+ * of this handle is bracketed by events and accumulated under its name. */
+int ghip_net_profile(ghip_net* net, int enable);
+int ghip_net_profile_count(ghip_net* net);
+int ghip_net_profile_entry(ghip_net* net, int index, char* name, int name_len, double* total_ms,
+                           int64_t* launches);
+int ghip_net_profile_reset(ghip_net* net);
+
+const char* ghip_last_error(void);
+const char* ghip_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,106 @@
+"""Canonical (batched) fp32 path on the GPU through the C ABI against the CPU restatement on the
+same arrays.  Bar: 1e-4 relative on logits and loss after N steps, identical argmax."""
+import numpy as np
+import pytest
+
+import pyoracle as po
+
+pytestmark = pytest.mark.gpu
+
+
+def build_pair(sizes, acts, params, cost, lr, mom, wd1, wd2, seed, bias=True):
+    import pyglades as pg
+    rng = np.random.default_rng(seed)
+    nl = len(sizes) - 1
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (1.2 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(nl)]
+    bs = [(rng.standard_normal(sizes[l + 1]) * 0.1).astype(np.float32) if bias else None for l in range(nl)]
+    o = po.CanonNet(po.make_spec(sizes, acts, lr=lr, mom=mom, wd1=wd1, wd2=wd2, act_params=params, cost=cost))
+    g = pg.Net(pg.make_spec(sizes, acts, lr=lr, mom=mom, wd1=wd1, wd2=wd2, act_params=params, cost=cost,
+                            mode=pg.MODE_CANONICAL, dtype=pg.F32))
+    for l in range(nl):
+        o.set_params(l, Ws[l], bs[l])
+        g.set_params(l, Ws[l], bs[l])
+    return o, g, rng
+
+
+def rel(a, b):
+    a = np.asarray(a, np.float64); b = np.asarray(b, np.float64)
+    return np.max(np.abs(a - b) / (np.abs(b) + 1e-3))
+
+
+CASES = [
+    ("relu_softmax_ragged", [37, 70, 33, 10], [po.RELU, po.RELU, po.SOFTMAX], [0, 0, 0], po.CLASSIFICATION, 53),
+    ("cfg3_like_small", [784, 128, 64, 10], [po.RELU, po.RELU, po.SOFTMAX], [0, 0, 0], po.CLASSIFICATION, 128),
+    ("sigmoid_bce", [6, 9, 4], [po.SIGMOID, po.SIGMOID], [0, 0], po.CLASSIFICATION, 17),
+    ("cfg2_shape_tanh_mse", [32, 64, 64, 1], [po.TANH, po.TANH, po.LINEAR], [0, 0, 1.0], po.REGRESSION, 256),
+    ("one_row", [5, 4, 3], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 1),
+    ("leaky_sigmoidp_kl", [9, 11, 7, 3], [po.LEAKY, po.TANHP, po.SIGMOID], [0.05, 0.1, 0], po.KL, 12),
+]
+
+
+@pytest.mark.parametrize("name,sizes,acts,params,cost,B", CASES)
+def test_training_steps_match_cpu(name, sizes, acts, params, cost, B):
+    print("case", name, flush=True)
+    o, g, rng = build_pair(sizes, acts, params, cost, 0.05, 0.9, 1e-4, 1e-3, 11)
+    steps = 8
+    N = B * steps
+    X = rng.standard_normal((N, sizes[0])).astype(np.float32)
+    if cost == po.REGRESSION:
+        Y = rng.standard_normal((N, sizes[-1])).astype(np.float32)
+    elif cost == po.KL:
+        Y = (rng.random((N, sizes[-1])) * 0.8 + 0.1).astype(np.float32)
+    else:
+        Y = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], N)]
+    g.set_dataset(X, Y)
+    for s in range(steps):
+        mo = o.step(X[s * B:(s + 1) * B], Y[s * B:(s + 1) * B])
+        mg = g.train_step(s * B, B)
+        assert abs(mg.loss - mo.loss) <= 1e-4 * abs(mo.loss) + 1e-6, (s, mg.loss, mo.loss)
+        assert abs(mg.accuracy - mo.accuracy) <= 1e-4 * abs(mo.accuracy) + 1e-4
+        assert mg.correct == mo.correct, s
+    for l in range(len(sizes) - 1):
+        Wo, bo = o.get_params(l)
+        Wg, bg = g.get_params(l)
+        np.testing.assert_allclose(Wg, Wo, rtol=1e-4, atol=2e-6)
+        np.testing.assert_allclose(bg, bo, rtol=1e-4, atol=2e-6)
+    Xt = rng.standard_normal((23, sizes[0])).astype(np.float32)
+    po_out, pg_out = o.forward(Xt), g.forward(Xt)
+    np.testing.assert_allclose(pg_out, po_out, rtol=1e-4, atol=1e-6)
+    if cost == po.CLASSIFICATION:
+        assert np.array_equal(pg_out.argmax(1), po_out.argmax(1))
+    g.close()
+
+
+def test_forward_matches_reference_forward():
+    """Canonical forward with an all-equal bias vector = the reference forward (exact-mode
+    oracle, itself bit-compared with the reference's objects)."""
+    import pyglades as pg
+    rng = np.random.default_rng(4)
+    sizes, acts, params = [7, 9, 8, 4], [po.RELU, po.SIGMOIDP, po.LEAKY], [0, 0.1, 0.05]
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * 0.5).astype(np.float32) for l in range(3)]
+    sb = [0.0, 0.25, -0.125]
+    X = rng.standard_normal((21, 7)).astype(np.float32)
+    Y = rng.random((21, 4)).astype(np.float32)
+    ex = po.ExactNet(po.make_spec(sizes, acts, act_params=params, batch=1, cost=po.REGRESSION))
+    g = pg.Net(pg.make_spec(sizes, acts, act_params=params, cost=pg.REGRESSION, mode=pg.MODE_CANONICAL))
+    for l in range(3):
+        ex.set_weights(l, Ws[l]); ex.set_bias(l, sb[l])
+        g.set_params(l, Ws[l], np.full(sizes[l + 1], sb[l], np.float32))
+    _, preds = ex.epoch(X, Y, train=False)
+    np.testing.assert_allclose(g.forward(X), preds, rtol=1e-4, atol=1e-6)
+    g.close()
+
+
+def test_last_partial_batch_and_bounds():
+    import pyglades as pg
+    o, g, rng = build_pair([10, 12, 3], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 0.1, 0.5, 0, 0, 5)
+    X = rng.standard_normal((25, 10)).astype(np.float32)
+    Y = np.eye(3, dtype=np.float32)[rng.integers(0, 3, 25)]
+    g.set_dataset(X, Y)
+    for r0, b in [(0, 10), (10, 10), (20, 5)]:   # last batch averaged over its true size
+        mo = o.step(X[r0:r0 + b], Y[r0:r0 + b]); mg = g.train_step(r0, b)
+        assert abs(mg.loss - mo.loss) <= 1e-4 * abs(mo.loss)
+    np.testing.assert_allclose(g.get_params(0)[0], o.get_params(0)[0], rtol=1e-4, atol=1e-6)
+    with pytest.raises(pg.GladesHipError):
+        g.train_step(20, 6)
+    g.close()

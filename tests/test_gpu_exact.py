@@ -1,0 +1,153 @@
+"""Exact mode on the GPU (through the C ABI) against the CPU restatement and the fixtures made
+by the reference's own compiled objects.  fp32 bar: 1e-4 relative on predictions, loss,
+accuracy and weights after the full schedule, identical argmax per row."""
+import numpy as np
+import pytest
+
+import pyoracle as po
+from helpers import TRAIN_CASES, load_case
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-4
+
+
+def close(a, b, rtol=RTOL, atol=None):
+    """|a-b| <= rtol*|b| + atol, with atol = rtol * (largest magnitude in b) unless given: an
+    entry that is tiny next to its neighbours is held to the array's scale, not its own."""
+    a = np.asarray(a, np.float64)
+    b = np.asarray(b, np.float64)
+    fin = np.isfinite(b)
+    assert np.array_equal(np.isfinite(a), fin)
+    if atol is None:
+        atol = rtol * (np.abs(b[fin]).max() if fin.any() else 0.0) + 1e-7
+    np.testing.assert_allclose(a[fin], b[fin], rtol=rtol, atol=atol)
+
+
+def gpu_net(c, bias_mode=0):
+    import pyglades as pg
+    spec = pg.make_spec(c["sizes"], [c["spec"].act[l] for l in range(c["nl"])],
+                        lr=[c["spec"].lr[l] for l in range(c["nl"])], mom=[c["spec"].mom[l] for l in range(c["nl"])],
+                        wd1=[c["spec"].wd1[l] for l in range(c["nl"])], wd2=[c["spec"].wd2[l] for l in range(c["nl"])],
+                        act_params=[c["spec"].act_param[l] for l in range(c["nl"])], batch=c["mb"], cost=c["cost"],
+                        mode=pg.MODE_EXACT, bias_mode=bias_mode)
+    net = pg.Net(spec)
+    for l in range(c["nl"]):
+        net.set_params(l, c["W0"][l], c["bias0"][l])
+    net.set_dataset(c["X"], c["Y"])
+    return net
+
+
+@pytest.mark.parametrize("name", TRAIN_CASES)
+def test_fixture_schedule(name):
+    print("case", name, flush=True)
+    c = load_case(name)
+    net = gpu_net(c)
+    ms, preds = net.run_epochs_exact(c["epochs"], train=True, want_preds=True)
+    d = c["d"]
+    assert len(ms) == c["epochs"]
+    loose = name.startswith("cfg2")  # first-layer weights reach ~1e14 there (doubling accumulator)
+    close([m[0] for m in ms], d["epochs"][:, 0])
+    close([m[1] for m in ms], d["epochs"][:, 1])
+    close(preds, d["preds"])
+    for r in range(c["N"]):
+        assert po.lib().go_argmax_ref(np.ascontiguousarray(preds[r]), preds.shape[1]) == \
+            po.lib().go_argmax_ref(np.ascontiguousarray(d["preds"][r]), preds.shape[1])
+    for l in range(c["nl"]):
+        W, b = net.get_params(l)
+        close(W, d[f"W_{l}"], rtol=1e-3 if loose else RTOL)
+        if l >= 1:
+            close(b[0], d["bias"][l])
+    net.close()
+
+
+def test_epoch_by_epoch_equals_one_launch():
+    """Resuming (one launch per epoch) must equal a single multi-epoch launch: all state,
+    including pending delta windows, survives between launches."""
+    c = load_case("window_4_5_3_1")
+    a = gpu_net(c)
+    b = gpu_net(c)
+    ms_a, _ = a.run_epochs_exact(4)
+    ms_b = []
+    for _ in range(4):
+        m, _ = b.run_epochs_exact(1)
+        ms_b += m
+    assert ms_a == ms_b
+    for l in range(c["nl"]):
+        assert np.array_equal(a.get_params(l)[0], b.get_params(l)[0])
+    a.close(); b.close()
+
+
+def test_test_pass_changes_nothing_and_matches_oracle():
+    c = load_case("mixed_5_7_6_4")
+    net = gpu_net(c)
+    ms, preds = net.run_epochs_exact(1, train=False, want_preds=True)
+    o = po.ExactNet(c["spec"])
+    for l in range(c["nl"]):
+        o.set_weights(l, c["W0"][l]); o.set_bias(l, c["bias0"][l])
+    m, opreds = o.epoch(c["X"], c["Y"], train=False)
+    close(preds, opreds)
+    close(ms[0][0], m.loss); close(ms[0][1], m.accuracy)
+    assert ms[0][2] == m.correct
+    for l in range(c["nl"]):
+        assert np.array_equal(net.get_params(l)[0], c["W0"][l])
+    net.close()
+
+
+def test_stop_accuracy_ends_early():
+    c = load_case("iris")
+    net = gpu_net(c)
+    target = float(c["d"]["epochs"][9, 1]) - 1e-3   # reached for the first time in some epoch <= 10
+    first = int(np.argmax(c["d"]["epochs"][:, 1] >= target)) + 1
+    ms, _ = net.run_epochs_exact(c["epochs"], stop_accuracy=target)
+    assert len(ms) == first
+    net.close()
+
+
+def test_closed_form_bias_is_close_but_sequential_is_default():
+    c = load_case("cfg1_shape_4_16_3")
+    seq = gpu_net(c, bias_mode=0)
+    fast = gpu_net(c, bias_mode=1)
+    ms_s, _ = seq.run_epochs_exact(5)
+    ms_f, _ = fast.run_epochs_exact(5)
+    close([m[0] for m in ms_f], [m[0] for m in ms_s], rtol=1e-3)
+    seq.close(); fast.close()
+
+
+@pytest.mark.parametrize("sizes,N,mb", [([1, 1], 1, 1), ([3, 300, 2], 5, 2), ([70, 3, 65, 1], 6, 4), ([2, 2, 2, 2, 2, 2], 9, 20)])
+def test_edge_shapes_against_oracle(sizes, N, mb):
+    """Single node, a layer wider than a wavefront, odd sizes, mb > N, deep narrow."""
+    import pyglades as pg
+    print("shape", sizes, N, mb, flush=True)
+    rng = np.random.default_rng(7)
+    nl = len(sizes) - 1
+    acts = [po.TANH] * nl
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (0.5 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(nl)]
+    X = rng.random((N, sizes[0])).astype(np.float32)
+    Y = rng.random((N, sizes[-1])).astype(np.float32)
+    ospec = po.make_spec(sizes, acts, lr=0.01, mom=0.5, batch=mb, cost=po.REGRESSION)
+    o = po.ExactNet(ospec)
+    net = pg.Net(pg.make_spec(sizes, acts, lr=0.01, mom=0.5, batch=mb, cost=pg.REGRESSION, mode=pg.MODE_EXACT))
+    for l in range(nl):
+        o.set_weights(l, Ws[l]); net.set_params(l, Ws[l], 0.0)
+    net.set_dataset(X, Y)
+    oms = [o.epoch(X, Y)[0] for _ in range(3)]
+    ms, _ = net.run_epochs_exact(3)
+    close([m[0] for m in ms], [m.loss for m in oms])
+    for l in range(nl):
+        close(net.get_params(l)[0], o.get_weights(l))
+    net.close()
+
+
+def test_error_paths():
+    import pyglades as pg
+    with pytest.raises(pg.GladesHipError):   # BATCH_FULL = 0 is "row % 0" in the reference
+        pg.Net(pg.make_spec([2, 2, 1], [0, 0], batch=0, mode=pg.MODE_EXACT))
+    with pytest.raises(pg.GladesHipError):
+        pg.Net(pg.make_spec([2, 0, 1], [0, 0], batch=1, mode=pg.MODE_EXACT))
+    net = pg.Net(pg.make_spec([2, 2, 1], [0, 0], batch=1, mode=pg.MODE_EXACT))
+    with pytest.raises(pg.GladesHipError):   # no dataset yet
+        net.run_epochs_exact(1)
+    with pytest.raises(pg.GladesHipError):   # wrong mode
+        net.train_step(0, 1)
+    net.close()
