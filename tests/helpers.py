@@ -38,3 +38,51 @@ def rel_err(a, b):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return float(np.max(np.abs(a - b) / (np.abs(b) + 1e-6))) if a.size else 0.0
+
+
+def bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, steps, lr, mom, wd2):
+    """numpy statement of the bf16 training pipeline: bf16 weights (rounded from the fp32 master),
+    bf16 activations and deltas, products exact and summed in float64, fp32 logits/softmax,
+    fp32 master + momentum update.  Hidden activations: TANH / RELU (0.046 knee) / SIGMOID;
+    output: SOFTMAX with cross-entropy.  Returns final master weights, biases and losses."""
+    q = po.bf16_round
+    Wm = [w.astype(np.float32).copy() for w in Ws]
+    bm = [b.astype(np.float32).copy() for b in bs]
+    vW = [np.zeros_like(w) for w in Wm]
+    vb = [np.zeros_like(b) for b in bm]
+    L = len(Wm)
+    losses = []
+    for s in range(steps):
+        x, y = X[s * B:(s + 1) * B], Y[s * B:(s + 1) * B]
+        Wh = [q(w) for w in Wm]
+        H = [q(x)]
+        for l in range(L):
+            Z = (H[l].astype(np.float64) @ Wh[l].T.astype(np.float64)).astype(np.float32) + bm[l]
+            if l == L - 1:
+                break
+            if acts[l] == po.TANH:
+                A = np.tanh(Z)
+            elif acts[l] == po.RELU:
+                A = np.where(Z < np.float32(0.046), np.float32(0), Z)
+            else:
+                A = 1.0 / (1.0 + np.exp(-Z))
+            H.append(q(A.astype(np.float32)))
+        E = np.exp(Z - Z.max(1, keepdims=True))
+        P = (E / E.sum(1, keepdims=True)).astype(np.float32)
+        losses.append(float(-(y * np.log(np.maximum(P, 1e-30))).sum(1).mean()))
+        D = q(P - y)
+        for l in range(L - 1, -1, -1):
+            g = (D.T.astype(np.float64) @ H[l].astype(np.float64) / B).astype(np.float32)
+            gb = D.astype(np.float64).mean(0).astype(np.float32)
+            if l > 0:
+                Eb = (D.astype(np.float64) @ Wh[l].astype(np.float64)).astype(np.float32)
+                h = H[l]
+                der = (1 - h * h) if acts[l - 1] == po.TANH else ((h > 0).astype(np.float32) if acts[l - 1] == po.RELU else h * (1 - h))
+                D = q(Eb * der)
+            d = lr * (g + wd2 * Wm[l]) + mom * vW[l]
+            vW[l] = d
+            Wm[l] = Wm[l] - d
+            db = lr * gb + mom * vb[l]
+            vb[l] = db
+            bm[l] = bm[l] - db
+    return Wm, bm, losses
