@@ -1,0 +1,296 @@
+#!/usr/bin/env python3
+"""Benchmark of the dense feed-forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg4|cfg5|cfg3|cfg2|cfg1]
+
+A "step" is one pass of the path over one batch of synthetic input that is already resident in
+HBM when the timed region starts: forward + backward + update (training workloads), forward
+(cfg5), one epoch of sequential rows (cfg1/cfg2, exact mode).  One JSON line is printed.
+
+Default workload cfg4 = BASELINE.json configs[3], the configuration its metric and target are
+quoted on: MLP 4096-4096-4096-4096-4096-1024, ReLU, softmax cross-entropy, batch 8192, bf16
+weights/activations, fp32 accumulation, fp32 master weights, SGD with momentum.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "glades-ml_amd"))
+
+PEAKS = {"bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}  # dense MFMA, TFLOP/s
+HBM_PEAK = 8000.0  # GB/s
+
+WORKLOADS = {
+    "cfg4": dict(desc="bf16 train MLP 4096-4096-4096-4096-4096-1024 ReLU softmax-CE, batch 8192, SGD momentum 0.9, fp32 master",
+                 sizes=[4096, 4096, 4096, 4096, 4096, 1024], batch=8192, rows=262144, dtype="bf16", kind="train"),
+    "cfg5": dict(desc="e4m3 inference MLP 8192-8192-8192-8192-1024 ReLU, batch 16384, per-channel weight / per-row activation scales",
+                 sizes=[8192, 8192, 8192, 8192, 1024], batch=16384, rows=16384, dtype="fp8", kind="infer"),
+    "cfg3": dict(desc="fp32 train MLP 784-1024-1024-10 ReLU softmax-CE, batch 512, SGD lr .05 momentum .9 L2 1e-4",
+                 sizes=[784, 1024, 1024, 10], batch=512, rows=60000, dtype="f32", kind="train"),
+    "cfg2": dict(desc="exact mode MLP 32-64-64-1 tanh/tanh/linear MSE, 10000 rows, mb 256, lr .01 momentum .9",
+                 sizes=[32, 64, 64, 1], batch=256, rows=10000, dtype="f32", kind="exact"),
+    "cfg1": dict(desc="exact mode MLP 4-16-3 sigmoid BCE, 150 rows, mb 150, lr .01 momentum .9",
+                 sizes=[4, 16, 3], batch=150, rows=150, dtype="f32", kind="exact"),
+}
+
+
+def train_flops_per_sample(sizes):
+    w = [sizes[l] * sizes[l + 1] for l in range(len(sizes) - 1)]
+    return 6 * sum(w) - 2 * w[0]  # forward + weight gradient everywhere, back-prop except layer 0
+
+
+def infer_flops_per_sample(sizes):
+    return 2 * sum(sizes[l] * sizes[l + 1] for l in range(len(sizes) - 1))
+
+
+def he_weights(sizes, seed):
+    rng = np.random.default_rng(seed)
+    return [(rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l])))
+            for l in range(len(sizes) - 1)]
+
+
+def hip_timed(net, fn, steps):
+    """Wall time of `steps` calls bracketed by device synchronisation on both sides."""
+    import torch
+    net.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(steps):
+        fn(s)
+    net.sync()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0
+
+
+def kernel_profile(net, fn, steps):
+    """Per-kernel HIP-event timing (events recorded on the stream the kernels run on)."""
+    net.profile(True)
+    net.profile_reset()
+    for s in range(steps):
+        fn(s)
+    net.sync()
+    tab = net.profile_table()
+    net.profile(False)
+    return tab
+
+
+def run_canonical(w, args):
+    import torch
+    import pyglades as pg
+    sizes, B, N = w["sizes"], w["batch"], w["rows"]
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev)
+    g.manual_seed(1234)
+    dt = {"bf16": pg.BF16, "f32": pg.F32, "fp8": pg.FP8_INFER}[w["dtype"]]
+    nl = len(sizes) - 1
+    acts = [pg.RELU] * (nl - 1) + ([pg.SOFTMAX] if w["kind"] == "train" else [pg.RELU])
+    if w["name"] == "cfg3":
+        hyper = dict(lr=0.05, mom=0.9, wd2=1e-4)
+    else:
+        hyper = dict(lr=0.01, mom=0.9, wd2=0.0)
+    spec = pg.make_spec(sizes, acts, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=dt, batch=B, **hyper)
+    net = pg.Net(spec)
+    Ws = he_weights(sizes, 42)
+    for l in range(nl):
+        net.set_params(l, Ws[l])
+    # synthetic table, generated on the device (torch is only the allocator / generator here)
+    if w["name"] == "cfg3":
+        X = torch.rand((N, sizes[0]), device=dev, generator=g, dtype=torch.float32)
+    else:
+        X = torch.randn((N, sizes[0]), device=dev, generator=g, dtype=torch.float32)
+    Y = None
+    if w["kind"] == "train":
+        T = torch.randn((sizes[0], sizes[-1]), device=dev, generator=g, dtype=torch.float32)
+        Y = torch.zeros((N, sizes[-1]), device=dev, dtype=torch.float32)
+        for r in range(0, N, 32768):
+            lab = (X[r:r + 32768] @ T).argmax(1)
+            Y[r:r + 32768].scatter_(1, lab[:, None], 1.0)
+        del T
+    torch.cuda.synchronize()
+    net.set_dataset_device(X.data_ptr(), Y.data_ptr() if Y is not None else 0, N)
+    nb = N // B
+    if w["kind"] == "train":
+        fn = lambda s: net.train_step((s % nb) * B, B, want_metrics=False)  # noqa: E731
+        flops = train_flops_per_sample(sizes)
+    else:
+        net.quantize_fp8(want=False)
+        fn = lambda s: net.forward_resident((s % nb) * B, B)  # noqa: E731
+        flops = infer_flops_per_sample(sizes)
+    for s in range(args.warmup):
+        fn(s)
+    el = hip_timed(net, fn, args.steps)
+    loss = net.last_metrics().loss if w["kind"] == "train" else None
+    prof = kernel_profile(net, fn, min(args.steps, 5))
+    net.close()
+    # dominant kernel + its algorithmic FLOPs per launch
+    gemm_names = {
+        "bf16": {"gemm_bf16_forward": "fwd_hidden", "gemm_bf16_forward_out": "fwd_out", "gemm_bf16_dgrad": "dgrad", "gemm_bf16_wgrad_sgd": "wgrad"},
+        "fp8": {"gemm_fp8_forward": "fwd_hidden", "gemm_fp8_forward_out": "fwd_out"},
+        "f32": {"gemm_f32_forward": "fwd_all", "gemm_f32_dgrad": "dgrad", "gemm_f32_wgrad": "wgrad"},
+    }[w["dtype"]]
+    wl = [sizes[l] * sizes[l + 1] for l in range(nl)]
+    per_step = {"fwd_hidden": 2 * B * sum(wl[:-1]), "fwd_out": 2 * B * wl[-1], "fwd_all": 2 * B * sum(wl),
+                "dgrad": 2 * B * sum(wl[1:]), "wgrad": 2 * B * sum(wl)}
+    psteps = min(args.steps, 5)
+    kern = {}
+    for name, (ms, cnt) in prof.items():
+        kern[name] = dict(total_ms=ms, launches=cnt, avg_ms=ms / max(cnt, 1))
+    dom = max((n for n in kern if n in gemm_names), key=lambda n: kern[n]["total_ms"])
+    fl_launch = per_step[gemm_names[dom]] * psteps / kern[dom]["launches"]
+    ach = fl_launch / (kern[dom]["avg_ms"] * 1e-3) / 1e12
+    peak = PEAKS[w["dtype"]]
+    roof = dict(bound="mfma", kernel=dom, achieved=round(ach, 2), peak=peak, unit="TFLOP/s", frac=round(ach / peak, 4),
+                traffic=None, flop_per_launch=fl_launch, avg_launch_ms=round(kern[dom]["avg_ms"], 4))
+    total_ms = sum(k["total_ms"] for k in kern.values())
+    breakdown = {n: round(k["total_ms"] / psteps, 4) for n, k in sorted(kern.items(), key=lambda kv: -kv[1]["total_ms"])}
+    value = args.steps * B / el
+    step_tflops = flops * B / (el / args.steps) / 1e12
+    extra = dict(step_tflops=round(step_tflops, 2), step_frac_of_peak=round(step_tflops / peak, 4),
+                 kernel_ms_per_step=breakdown, kernel_ms_sum=round(total_ms / psteps, 4), final_loss=loss)
+    return value, el, roof, extra
+
+
+def run_exact(w, args):
+    import pyglades as pg
+    sizes, N, mb = w["sizes"], w["rows"], w["batch"]
+    rng = np.random.default_rng(1234)
+    if w["name"] == "cfg2":
+        t = np.arange(N + 32, dtype=np.float64)
+        f, ph = rng.random(3) * 0.05 + 0.01, rng.random(3) * 6.28
+        sig = sum(np.sin(2 * np.pi * f[k] * t + ph[k]) for k in range(3)) + rng.standard_normal(N + 32) * 0.05
+        sig = (sig - sig.min()) / (sig.max() - sig.min())
+        X = np.stack([sig[i:i + 32] for i in range(N)]).astype(np.float32)
+        Y = sig[32:32 + N, None].astype(np.float32)
+        acts, params, cost = [pg.TANH, pg.TANH, pg.LINEAR], [0, 0, 1.0], pg.REGRESSION
+    else:
+        c = rng.random((3, 4)) * 8
+        lab = np.repeat(np.arange(3), 50)
+        X = (c[lab] + rng.standard_normal((150, 4)) * 0.5).astype(np.float32)
+        X = ((X - X.min(0)) / (X.max(0) - X.min(0)) * 0.98 + 0.01).astype(np.float32)
+        Y = np.where(np.eye(3)[lab] > 0, 0.99, 0.01).astype(np.float32)
+        acts, params, cost = [pg.SIGMOID, pg.SIGMOID], [0, 0], pg.CLASSIFICATION
+    nl = len(sizes) - 1
+    spec = pg.make_spec(sizes, acts, lr=0.01, mom=0.9, act_params=params, batch=mb, cost=cost, mode=pg.MODE_EXACT)
+    net = pg.Net(spec)
+    for l in range(nl):
+        lim = np.sqrt(6.0 / (sizes[l] + sizes[l + 1]))
+        net.set_params(l, rng.uniform(-lim, lim, (sizes[l + 1], sizes[l])).astype(np.float32), 0.0)
+    net.set_dataset(X, Y)
+    for _ in range(args.warmup):
+        net.run_epochs_exact(1)
+    net.sync()
+    t0 = time.perf_counter()
+    ms, _ = net.run_epochs_exact(args.steps)   # one launch, `steps` epochs
+    net.sync()
+    el = time.perf_counter() - t0
+    prof = kernel_profile(net, lambda s: net.run_epochs_exact(1), 3)
+    net.close()
+    value = args.steps * N / el
+    k = prof["exact_epochs"]
+    bytes_per_sample = 4 * (sizes[0] + sizes[-1])
+    ach = bytes_per_sample * N / (k[0] / k[1] * 1e-3) / 1e9
+    roof = dict(bound="hbm", kernel="exact_epochs", achieved=round(ach, 4), peak=HBM_PEAK, unit="GB/s",
+                frac=round(ach / HBM_PEAK, 8), traffic=None, avg_launch_ms=round(k[0] / k[1], 4),
+                note="latency-bound: one persistent workgroup, rows strictly sequential")
+    extra = dict(final_loss=ms[-1][0], final_accuracy=ms[-1][1], flop_per_sample=train_flops_per_sample(sizes))
+    return value, el, roof, extra
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """The CPU restatement (oracle/, kind "port") timed on this host's cores on a bounded sample."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import pyoracle as po
+    sizes = w["sizes"]
+    nl = len(sizes) - 1
+    cores = min(16, os.cpu_count() or 1)
+    rng = np.random.default_rng(7)
+    if w["kind"] == "exact":
+        acts = [po.TANH, po.TANH, po.LINEAR] if w["name"] == "cfg2" else [po.SIGMOID, po.SIGMOID]
+        params = [0, 0, 1.0] if w["name"] == "cfg2" else [0, 0]
+        cost = po.REGRESSION if w["name"] == "cfg2" else po.CLASSIFICATION
+        net = po.ExactNet(po.make_spec(sizes, acts, lr=0.01, mom=0.9, act_params=params, batch=w["batch"], cost=cost))
+        for l in range(nl):
+            net.set_weights(l, (rng.standard_normal((sizes[l + 1], sizes[l])) * 0.1).astype(np.float32))
+        N = w["rows"]
+        X = rng.random((N, sizes[0])).astype(np.float32)
+        Y = (rng.random((N, sizes[-1])) * 0.98 + 0.01).astype(np.float32)
+        ep, t0 = 0, time.perf_counter()
+        with np.errstate(all="ignore"):
+            while time.perf_counter() - t0 < min(budget_s, 5.0):
+                net.epoch(X, Y, want_preds=False)
+                ep += 1
+        el = time.perf_counter() - t0
+        return dict(value=round(ep * N / el, 1), unit="samples/s", cores=1, kind="port",
+                    sample=f"{ep} epochs of {N} rows, exact mode, 1 thread (the reference is single-threaded)")
+    po.lib().go_set_threads(cores)
+    acts = [po.RELU] * (nl - 1) + ([po.SOFTMAX] if w["kind"] == "train" else [po.RELU])
+    net = po.CanonNet(po.make_spec(sizes, acts, lr=0.01, mom=0.9, cost=po.CLASSIFICATION))
+    for l in range(nl):
+        net.set_params(l, (rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l]))))
+    rows = {"cfg4": 256, "cfg5": 256, "cfg3": 512}.get(w["name"], 256)
+    X = rng.standard_normal((rows, sizes[0]), dtype=np.float32)
+    Y = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], rows)]
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        if w["kind"] == "train":
+            net.step(X, Y)
+        else:
+            net.forward(X)
+        reps += 1
+        if time.perf_counter() - t0 > budget_s / 2 or reps >= 50:
+            break
+    el = time.perf_counter() - t0
+    what = "fwd+bwd+update steps" if w["kind"] == "train" else "fp32 forwards"
+    return dict(value=round(reps * rows / el, 1), unit="samples/s", cores=cores, kind="port",
+                sample=f"{reps} {what} of {rows} rows (1/{w['batch'] // rows} of a batch), fp32, {cores} OpenMP threads")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    w = dict(WORKLOADS[args.workload], name=args.workload)
+    if args.steps is None:
+        args.steps = {"cfg4": 40, "cfg5": 40, "cfg3": 200, "cfg2": 5, "cfg1": 200}[args.workload]
+    if args.warmup is None:
+        args.warmup = {"cfg4": 5, "cfg5": 5, "cfg3": 20, "cfg2": 1, "cfg1": 5}[args.workload]
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    if w["kind"] == "exact":
+        value, el, roof, extra = run_exact(w, args)
+        unit_rows = w["rows"]
+    else:
+        value, el, roof, extra = run_canonical(w, args)
+        unit_rows = w["batch"]
+    out = {
+        "metric": "train samples/sec (fwd+bwd+update)" if w["kind"] != "infer" else "infer samples/sec",
+        "value": round(value, 1), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(el / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}", "rows_per_step": unit_rows,
+                   "flop_per_sample": train_flops_per_sample(w["sizes"]) if w["kind"] != "infer" else infer_flops_per_sample(w["sizes"])},
+        "roofline": roof,
+    }
+    out["detail"] = extra
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
