@@ -24,11 +24,16 @@ __device__ __forceinline__ double wave_sum_d(double v)
     return v;
 }
 
-// One wavefront per row, 16 rows per wavefront, 4 wavefronts per workgroup.
 // Output layer of the canonical mode: softmax (if asked), per-sample loss = sum over outputs of
 // the reference's cost (gmath.cpp:272-321 without the 1/dataSize), the reference's accuracy term
 // (network.cpp:541-547), argmax agreement under gmath.cpp:412-455, and delta = dLoss/dz.
-constexpr int kRowsPerWave = 16;
+// One wavefront per row, kRowsPerWave rows per wavefront, 4 wavefronts per workgroup.  A row of
+// up to 64*kRegs outputs is read from memory once and kept in registers (lane j-th value =
+// column j*64 + lane): one exp per element, and the softmax passes cost no extra HBM traffic.
+constexpr int kRowsPerWave = 2;
+constexpr int kRegs = 16;
+
+template <bool kInRegs>
 __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
 {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -41,24 +46,45 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
         if (b >= a.B) break;
         float* p = a.P + (long long)b * a.ldp;
         const float* y = a.Y ? a.Y + (long long)b * a.ldy : nullptr;
+        float reg[kRegs];
         float inv = 1.0f, mx = 0.0f;
+        if (kInRegs) {
+#pragma unroll
+            for (int j = 0; j < kRegs; ++j) {
+                const int o = j * 64 + lane;
+                reg[j] = (o < a.n) ? p[o] : -3.0e38f;
+            }
+        }
         if (softmax) {
             float m = -3.0e38f;
-            for (int o = lane; o < a.n; o += 64) m = fmaxf(m, p[o]);
+            if (kInRegs) {
+#pragma unroll
+                for (int j = 0; j < kRegs; ++j) m = fmaxf(m, reg[j]);
+            } else {
+                for (int o = lane; o < a.n; o += 64) m = fmaxf(m, p[o]);
+            }
             mx = wave_max(m);
             float s = 0.0f;
-            for (int o = lane; o < a.n; o += 64) s += expf(p[o] - mx);
+            if (kInRegs) {
+#pragma unroll
+                for (int j = 0; j < kRegs; ++j) {
+                    const int o = j * 64 + lane;
+                    reg[j] = (o < a.n) ? expf(reg[j] - mx) : 0.0f;
+                    s += reg[j];
+                }
+            } else {
+                for (int o = lane; o < a.n; o += 64) s += expf(p[o] - mx);
+            }
             inv = 1.0f / wave_sum(s);
         }
         float l = 0.0f, ac = 0.0f;
         float bp = 0.0f, by = 0.0f;  // running maxima for the argmax rule (start at 0, strict >)
         int ip = 0x7fffffff, iy = 0x7fffffff;
-        for (int o = lane; o < a.n; o += 64) {
-            float pv = p[o];
+        auto element = [&](int o, float pv) {
             const float yv = y ? y[o] : 0.0f;
             float d;
             if (softmax) {
-                pv = expf(pv - mx) * inv;
+                pv = kInRegs ? pv * inv : expf(pv - mx) * inv;
                 p[o] = pv;
                 if (yv != 0.0f) l += -(yv * logf(fmaxf(pv, 1e-30f)));
                 d = pv - yv;
@@ -71,6 +97,15 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
             if (yv > by) { by = yv; iy = o; }
             if (a.D) a.D[(long long)b * a.n + o] = d;
             if (a.Dbf) a.Dbf[(long long)b * a.n + o] = ghip_f32_to_bf16(d);
+        };
+        if (kInRegs) {
+#pragma unroll
+            for (int j = 0; j < kRegs; ++j) {
+                const int o = j * 64 + lane;
+                if (o < a.n) element(o, reg[j]);
+            }
+        } else {
+            for (int o = lane; o < a.n; o += 64) element(o, p[o]);
         }
         // argmax across lanes: largest value, lowest index on ties; "no element above 0" = none
 #pragma unroll
@@ -130,21 +165,25 @@ bias_update_f32_kernel(const float* __restrict__ D, int B, int n, int ldd, float
     }
 }
 
-// bf16 delta^T [n][B]: one workgroup per channel
+// bf16 delta^T [n][B]: one wavefront per channel, 16-byte loads (B is a multiple of 8)
 __global__ void __launch_bounds__(256)
 bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* __restrict__ bias,
                          float* __restrict__ vb, float lr, float mom)
 {
-    const int o = blockIdx.x;
-    const uint16_t* row = DT + (long long)o * B;
+    const int lane = threadIdx.x & 63;
+    const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (o >= n) return;
+    const uint4* row = reinterpret_cast<const uint4*>(DT + (long long)o * B);
     float s = 0.0f;
-    for (int b = threadIdx.x; b < B; b += 256) s += ghip_bf16_to_f32(row[b]);
+    for (int k = lane; k < (B >> 3); k += 64) {
+        const uint4 q = row[k];
+        const unsigned int wds[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s += __uint_as_float(wds[j] << 16) + __uint_as_float(wds[j] & 0xffff0000u);
+    }
     s = wave_sum(s);
-    __shared__ float red[4];
-    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        const float g = (red[0] + red[1] + red[2] + red[3]) / (float)B;
+    if (lane == 0) {
+        const float g = s / (float)B;
         const float d = lr * g + mom * vb[o];
         vb[o] = d;
         bias[o] = bias[o] - d;
@@ -232,7 +271,9 @@ inline int grid_for(long long n, int cap = 65535 * 4)
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
 {
     const int rows_per_block = 4 * kRowsPerWave;
-    hipLaunchKernelGGL(output_delta_kernel, dim3((a.B + rows_per_block - 1) / rows_per_block), dim3(256), 0, s, a);
+    const dim3 grid((a.B + rows_per_block - 1) / rows_per_block);
+    if (a.n <= 64 * kRegs) hipLaunchKernelGGL(output_delta_kernel<true>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(output_delta_kernel<false>, grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
@@ -254,7 +295,7 @@ hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bi
 hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vb, float lr,
                                   float mom, hipStream_t s)
 {
-    hipLaunchKernelGGL(bias_update_bf16T_kernel, dim3(n), dim3(256), 0, s, DT, n, B, bias, vb, lr, mom);
+    hipLaunchKernelGGL(bias_update_bf16T_kernel, dim3((n + 3) / 4), dim3(256), 0, s, DT, n, B, bias, vb, lr, mom);
     return hipGetLastError();
 }
 

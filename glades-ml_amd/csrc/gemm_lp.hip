@@ -11,11 +11,14 @@
 //             fused with the SGD + momentum + L1/L2 update of the fp32 master weights, which
 //             also writes the bf16 W and W^T used by the next step.
 //
-// Tile: 256 x 256 x 128 bytes of K (64 bf16 / 128 e4m3) per workgroup of 8 wavefronts laid out
-// 2 (M) x 4 (N); each wavefront owns 128 x 64 = 4 x 2 accumulators of 32x32 (128 VGPRs).
-// LDS: two buffers of (256 + 256) rows x 128 B = 128 KiB.  Rows are 128 B, 16-byte chunks are
-// XOR-swizzled with the row index so that both the row-wise stores and the per-lane 16-byte
-// operand reads (32 consecutive rows, same logical chunk) spread over all banks.
+// Tile: 256 x 256 outputs per workgroup of 8 wavefronts laid out 2 (M) x 4 (N); each wavefront owns
+// 128 x 64 = 4 x 2 accumulators of 32x32 (128 VGPRs).  K advances in stages of 64 bytes per row
+// (32 bf16 / 64 e4m3).  LDS holds a ring of 4 stages (4 x 32 KiB) filled by LDS-direct global
+// loads (global_load_lds_dwordx4: no VGPR staging, no ds_write); three stages are in flight while
+// one is consumed, so the s_waitcnt before each barrier only waits for loads issued three stages
+// earlier (the single-stage look-ahead of a plain double buffer left the matrix cores waiting on
+// L2/HBM latency ~30 % of the time).  Rows are 64 B; 16-byte chunks are XOR-swizzled with the row
+// index so that the per-lane 16-byte operand reads spread over all 64 banks.
 // Workgroup ids are remapped so that each XCD (ids congruent mod 8 share an L2) walks a compact
 // block of tiles.
 
@@ -28,19 +31,121 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int TM = 256, TN = 256, TKB = 128, NT = 512;
-constexpr int TILE_BYTES = 256 * TKB;  // one operand tile
+constexpr int TM = 256, TN = 256, NT = 512;
+constexpr int SKB = 128;                 // bytes of K per stage row (64 bf16 / 128 e4m3): one full cache line
+constexpr int STAGE_BYTES = 256 * SKB;   // one operand stage
+constexpr int EPI_PITCH = 528;           // bytes per staged output row: 512 + 16 (keeps 16-byte alignment, rotates banks)
+constexpr int EPI_LDS_BYTES = 256 * EPI_PITCH;  // 132 KiB >= 8 stages
 
-__device__ __forceinline__ int swz(int row, int chunk) { return (row << 7) + (((chunk ^ row) & 7) << 4); }
+// LDS has 64 banks of 4 bytes: a 16-byte-per-lane read is served 16 lanes per clock.  A stage
+// row is 128 B = 32 banks, so row parity picks the bank half and (row >> 1) & 7 rotates the
+// chunk: 16 consecutive rows reading one logical chunk touch 16 distinct (half, chunk) slots.
+__device__ __forceinline__ int swz(int row, int chunk) { return (row << 7) + (((chunk ^ (row >> 1)) & 7) << 4); }
 
-__device__ __forceinline__ float lp_squash(float z, int act, float p) { return ghip_squash<false>(z, act, p); }
+// Activation and its derivative in a branch-free parametric form (filled on the host by
+// resolve_act): the epilogues apply them to 128 accumulators per lane, and a switch over the
+// activation id replicated that often does not fit the instruction cache.
+__device__ __forceinline__ float lp_squash(float z, const GemmLpArgs::ActForm& a)
+{
+    float v = (z < a.thr) ? a.a0 * z + a.b0 : a.a1 * z + a.b1;
+    if (a.trans) v = a.ta * __frcp_rn(1.0f + __expf(-a.tk * z)) + a.tb;
+    v = (z < a.clo) ? a.vlo : v;
+    v = (z > a.chi) ? a.vhi : v;
+    return v;
+}
+__device__ __forceinline__ float lp_act_der(float y, const GemmLpArgs::ActForm& a)
+{
+    const float poly = a.c0 + a.c1 * y + a.c2 * y * y;
+    const float stp = (y > 0.0f) ? a.dhi : a.dlo;
+    return a.step ? stp : poly;
+}
+
+// Operand fragments of one K sub-step for this wavefront: 4 row blocks of A, 2 of B.
+// bf16: 16 bytes per lane per block (K = 16); e4m3: 32 bytes per lane per block (K = 64).
+template <bool FP8> struct Frags { v4i a[4], b[2]; };
+template <> struct Frags<true> { v4i a[4][2], b[2][2]; };
+
+template <bool FP8>
+__device__ __forceinline__ void load_frags(Frags<FP8>& f, const unsigned char* sa, const unsigned char* sb,
+                                           int ks, int wm, int wn, int l31, int lh)
+{
+    if constexpr (!FP8) {
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi) f.a[mi] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, ks * 2 + lh));
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) f.b[ni] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, ks * 2 + lh));
+    } else {
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                f.a[mi][h] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, ks * 4 + lh * 2 + h));
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, ks * 4 + lh * 2 + h));
+    }
+}
+
+template <bool FP8>
+__device__ __forceinline__ void mma_frags(v16f (&acc)[4][2], const Frags<FP8>& f)
+{
+#pragma unroll
+    for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni) {
+            if constexpr (!FP8) {
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi]),
+                                                                      __builtin_bit_cast(bf16x8, f.b[ni]), acc[mi][ni], 0, 0, 0);
+            } else {
+                const v8i av = v8i{f.a[mi][0][0], f.a[mi][0][1], f.a[mi][0][2], f.a[mi][0][3],
+                                   f.a[mi][1][0], f.a[mi][1][1], f.a[mi][1][2], f.a[mi][1][3]};
+                const v8i bv = v8i{f.b[ni][0][0], f.b[ni][0][1], f.b[ni][0][2], f.b[ni][0][3],
+                                   f.b[ni][1][0], f.b[ni][1][1], f.b[ni][1][2], f.b[ni][1][3]};
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+            }
+        }
+}
+
+typedef __attribute__((address_space(3))) unsigned char* lptr_t;
+
+// One operand stage (256 rows x 128 B) is 32 slabs of 8 rows = 1 KiB; a wavefront moves 4 slabs
+// with 4 LDS-direct loads: lane i of a load lands at slab + 16*i, i.e. row i/8, physical chunk
+// i%8, so the lane fetches the logical chunk that the swizzle maps there.  Every load covers
+// whole 128-byte lines (with 64-byte stage rows each line was fetched from L2 twice).
+// The load is issued from inline assembly on purpose: the compiler then keeps no book on it, and
+// the only waits on these loads are the explicit s_waitcnt vmcnt(N) before each barrier (with the
+// builtin it drains all of them, vmcnt(0), in front of LDS reads it cannot tell apart from the
+// stage being filled).  M0 carries the LDS byte address of the slab; loads return in order.
+__device__ __forceinline__ void dma_stage(unsigned char* sdst, const unsigned char* gsrc, long long ldk,
+                                          long long kb, int w, int lane)
+{
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int slab = w * 4 + j;
+        const int row = slab * 8 + (lane >> 3);
+        const int chunk = ((lane & 7) ^ (row >> 1)) & 7;
+        const unsigned char* src = gsrc + (long long)row * ldk + kb + (chunk << 4);
+        const unsigned int dst = (unsigned int)(uintptr_t)((lptr_t)sdst) + slab * 1024;
+        const unsigned int dst_u = __builtin_amdgcn_readfirstlane(dst);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                     :
+                     : "v"(src), "s"(dst_u)
+                     : "memory", "m0");
+    }
+}
 
 template <bool FP8, int EPI>
 __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    unsigned char* sA = lds;                    // [2][TILE_BYTES]
-    unsigned char* sB = lds + 2 * TILE_BYTES;   // [2][TILE_BYTES]
+    // One LDS block: two stages (A then B, 256 rows x 128 B of K each) during the K loop,
+    // then the staging area of the epilogue (256 x 256 bf16 with padded rows).
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[EPI_LDS_BYTES];
+    unsigned char* const sA0 = smem;
+    unsigned char* const sB0 = smem + 1 * STAGE_BYTES;
+    unsigned char* const sA1 = smem + 2 * STAGE_BYTES;
+    unsigned char* const sB1 = smem + 3 * STAGE_BYTES;
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6;
     const int l31 = lane & 31, lh = lane >> 5;
@@ -74,90 +179,101 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
 
-    v4i ra[4], rb[4];
-    int lrow[4], lch[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int c = t + j * NT;
-        lrow[j] = c >> 3;
-        lch[j] = c & 7;
-    }
-    auto gload = [&](int kt) {
-        const long long kb = (long long)kt * TKB;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            ra[j] = *reinterpret_cast<const v4i*>(gA + (long long)lrow[j] * ldk + kb + (lch[j] << 4));
-            rb[j] = *reinterpret_cast<const v4i*>(gB + (long long)lrow[j] * ldk + kb + (lch[j] << 4));
-        }
-    };
-    auto lstore = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            *reinterpret_cast<v4i*>(sA + buf * TILE_BYTES + swz(lrow[j], lch[j])) = ra[j];
-            *reinterpret_cast<v4i*>(sB + buf * TILE_BYTES + swz(lrow[j], lch[j])) = rb[j];
-        }
-    };
+    const int nk = (int)(ldk / SKB);  // stages along K (even, see ghip_gemm_lp_shape_ok)
 
-    const int nk = (int)(ldk / TKB);
-    gload(0);
-    lstore(0);
-    __syncthreads();
+    auto fill = [&](unsigned char* WA, unsigned char* WB, int st) {
+        const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;  // past the end: refetch, never read
+        dma_stage(WA, gA, ldk, kb, w, lane);
+        dma_stage(WB, gB, ldk, kb, w, lane);
+    };
+    fill(sA0, sB0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __builtin_amdgcn_s_barrier();
 
-    for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) gload(kt + 1);
-        const unsigned char* a_base = sA + cur * TILE_BYTES;
-        const unsigned char* b_base = sB + cur * TILE_BYTES;
-        if (!FP8) {
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                v4i af[4], bf[2];
-#pragma unroll
-                for (int mi = 0; mi < 4; ++mi)
-                    af[mi] = *reinterpret_cast<const v4i*>(a_base + swz(wm + mi * 32 + l31, ks * 2 + lh));
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    bf[ni] = *reinterpret_cast<const v4i*>(b_base + swz(wn + ni * 32 + l31, ks * 2 + lh));
-#pragma unroll
-                for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, af[mi]), __builtin_bit_cast(bf16x8, bf[ni]), acc[mi][ni], 0, 0, 0);
-            }
+    Frags<FP8> f0, f1;
+    load_frags<FP8>(f0, sA0, sB0, 0, wm, wn, l31, lh);
+
+    // One stage: reads (RA, RB) = stage s while (WA, WB) is filled with stage s+1 (the buffer of
+    // stage s-1, free since the barrier that ended it).  Sub-steps are software pipelined: each
+    // one first states that its own fragments (requested one MFMA group earlier) have landed, then
+    // requests the next sub-step's fragments, then issues its MFMAs.  The last sub-step waits for
+    // the fill, meets the other wavefronts (bare s_barrier: the explicit counts are exactly what
+    // has to be visible) and requests the first fragments of stage s+1.
+    constexpr int KS = FP8 ? 2 : 4;
+    auto stage = [&](int s, const unsigned char* RA, const unsigned char* RB, unsigned char* WA, unsigned char* WB) {
+        if constexpr (FP8) {
+            fill(WA, WB, s + 1);
+            mma_frags<FP8>(acc, f0);
+            load_frags<FP8>(f0, RA, RB, 1, wm, wn, l31, lh);
+            mma_frags<FP8>(acc, f0);
+            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+            __builtin_amdgcn_s_barrier();
+            load_frags<FP8>(f0, WA, WB, 0, wm, wn, l31, lh);
         } else {
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                v8i af[4], bf[2];
-#pragma unroll
-                for (int mi = 0; mi < 4; ++mi) {
-                    const int row = wm + mi * 32 + l31;
-                    v4i lo = *reinterpret_cast<const v4i*>(a_base + swz(row, ks * 4 + lh * 2));
-                    v4i hi = *reinterpret_cast<const v4i*>(a_base + swz(row, ks * 4 + lh * 2 + 1));
-                    af[mi] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            for (int ks = 0; ks < KS; ++ks) {
+                Frags<FP8>& cur = (ks & 1) ? f1 : f0;
+                Frags<FP8>& nxt = (ks & 1) ? f0 : f1;
+                if (ks + 1 < KS) {
+                    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): cur has landed
+                    load_frags<FP8>(nxt, RA, RB, ks + 1, wm, wn, l31, lh);
+                    if (ks == 0) fill(WA, WB, s + 1);
+                } else {
+                    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+                    __builtin_amdgcn_s_barrier();
+                    load_frags<FP8>(nxt, WA, WB, 0, wm, wn, l31, lh);
                 }
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni) {
-                    const int row = wn + ni * 32 + l31;
-                    v4i lo = *reinterpret_cast<const v4i*>(b_base + swz(row, ks * 4 + lh * 2));
-                    v4i hi = *reinterpret_cast<const v4i*>(b_base + swz(row, ks * 4 + lh * 2 + 1));
-                    bf[ni] = v8i{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                }
-#pragma unroll
-                for (int mi = 0; mi < 4; ++mi)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                            af[mi], bf[ni], acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+                __builtin_amdgcn_sched_barrier(0);
+                mma_frags<FP8>(acc, cur);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        if (kt + 1 < nk) lstore(cur ^ 1);
-        __syncthreads();
+    };
+    for (int s = 0; s < nk; s += 2) {
+        stage(s, sA0, sB0, sA1, sB1);
+        stage(s + 1, sA1, sB1, sA0, sB0);
     }
+    // nothing may still be writing this workgroup's LDS when its wavefronts retire
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
 
     // ---- epilogue.  Accumulator layout of a 32x32 tile: lane -> column lane%32,
-    //      register i -> row 8*(i/4) + 4*(lane/32) + i%4  (4 consecutive rows per register quad)
+    //      register i -> row 8*(i/4) + 4*(lane/32) + i%4  (4 consecutive rows per register quad).
+    //      bf16 results leave through LDS so that global memory only sees 16-byte-per-lane,
+    //      512-byte-per-row stores (direct stores from this layout are 2 bytes per lane, and 8
+    //      bytes per lane with a row-sized stride for the transposed copy).
     const int M = g.M, N = g.N;
+    __builtin_amdgcn_s_barrier();  // every wavefront is done with the ring
+
+    if constexpr (EPI == LP_DGRAD) {
+        // activation tile [256][256] bf16 -> LDS (row pitch 512 B) with LDS-direct loads
+        const unsigned char* aux = (const unsigned char*)g.aux + ((long long)bm * N + bn) * 2;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int slab = w * 16 + j;  // 2 rows per slab
+            const int row = slab * 2 + (lane >> 5);
+            const unsigned char* src = aux + (long long)row * N * 2 + ((lane & 31) << 4);
+            const unsigned int dst = __builtin_amdgcn_readfirstlane((unsigned int)(uintptr_t)((lptr_t)smem) + slab * 1024);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+        }
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = wm + mi * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
+                    const int col = wn + ni * 32 + l31;
+                    const uint16_t hv = *reinterpret_cast<const uint16_t*>(smem + row * 512 + col * 2);
+                    acc[mi][ni][i] *= lp_act_der(ghip_bf16_to_f32(hv), g.ap);
+                }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();
+    }
+
+    constexpr bool kBf16Out = (EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT);
+    uint2 pk[4][2][4];  // bf16 results, 4 consecutive rows packed per entry
 #pragma unroll
     for (int mi = 0; mi < 4; ++mi) {
 #pragma unroll
@@ -169,22 +285,18 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int row0 = bm + wm + mi * 32 + 8 * q + 4 * lh;
-                uint16_t hb[4];
+                uint16_t hb[4] = {0, 0, 0, 0};
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int row = row0 + r;
                     const long long idx = (long long)row * N + col;
                     float v = acc[mi][ni][q * 4 + r];
                     if (EPI == LP_FWD_ACT) {
-                        v = lp_squash(v + cbias, g.act, g.act_param);
-                        hb[r] = ghip_f32_to_bf16(v);
-                        ((uint16_t*)g.out)[idx] = hb[r];
+                        hb[r] = ghip_f32_to_bf16(lp_squash(v + cbias, g.ap));
                     } else if (EPI == LP_FWD_F32) {
-                        ((float*)g.out)[idx] = lp_squash(v + cbias, g.act, g.act_param);
+                        ((float*)g.out)[idx] = lp_squash(v + cbias, g.ap);
                     } else if (EPI == LP_DGRAD) {
-                        v = v * ghip_act_der_canon(ghip_bf16_to_f32(g.aux[idx]), g.act, g.act_param);
                         hb[r] = ghip_f32_to_bf16(v);
-                        ((uint16_t*)g.out)[idx] = hb[r];
                     } else if (EPI == LP_WGRAD_SGD) {
                         const float wv = g.master[idx];
                         const float sg = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : 0.0f);
@@ -194,28 +306,70 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                         const float nw = wv - d;
                         g.master[idx] = nw;
                         hb[r] = ghip_f32_to_bf16(nw);
-                        ((uint16_t*)g.out)[idx] = hb[r];
                     } else if (EPI == LP_FP8_ACT) {
-                        v = lp_squash(__fmul_rn(v, __fmul_rn(g.row_scale[row], cscale)), g.act, g.act_param);
+                        v = lp_squash(__fmul_rn(v, __fmul_rn(g.row_scale[row], cscale)), g.ap);
                         hb[r] = ghip_f32_to_bf16(v);
-                        ((uint16_t*)g.out)[idx] = hb[r];
                         // row amax of the stored (bf16-rounded) values over this wavefront's 32 columns
                         float am = fabsf(ghip_bf16_to_f32(hb[r]));
 #pragma unroll
                         for (int o = 16; o > 0; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
                         if (l31 == 0) atomicMax(&g.row_amax_bits[row], __float_as_uint(am));
                     } else {  // LP_FP8_F32
-                        v = lp_squash(__fmul_rn(v, __fmul_rn(g.row_scale[row], cscale)), g.act, g.act_param);
-                        ((float*)g.out)[idx] = v;
+                        ((float*)g.out)[idx] = lp_squash(__fmul_rn(v, __fmul_rn(g.row_scale[row], cscale)), g.ap);
                     }
                 }
-                if ((EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD) && g.outT) {
-                    uint2 pk;
-                    pk.x = (uint32_t)hb[0] | ((uint32_t)hb[1] << 16);
-                    pk.y = (uint32_t)hb[2] | ((uint32_t)hb[3] << 16);
-                    *reinterpret_cast<uint2*>((uint16_t*)g.outT + (long long)col * M + row0) = pk;
-                }
+                pk[mi][ni][q].x = (uint32_t)hb[0] | ((uint32_t)hb[1] << 16);
+                pk[mi][ni][q].y = (uint32_t)hb[2] | ((uint32_t)hb[3] << 16);
             }
+        }
+    }
+    if constexpr (kBf16Out) {
+        const int lr2 = lane >> 5, lc = (lane & 31) << 4;
+        // transposed copy first: LDS_T[n][m], a lane's 4 consecutive rows are 8 contiguous bytes
+        if ((EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD) && g.outT) {
+#pragma unroll
+            for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int rl = wm + mi * 32 + 8 * q + 4 * lh, cl = wn + ni * 32 + l31;
+                        *reinterpret_cast<uint2*>(smem + cl * EPI_PITCH + rl * 2) = pk[mi][ni][q];
+                    }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();
+            unsigned char* dstT = (unsigned char*)g.outT + ((long long)bn * M + bm) * 2;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int nl = w * 32 + i * 2 + lr2;
+                const v4i val = *reinterpret_cast<const v4i*>(smem + nl * EPI_PITCH + lc);
+                *reinterpret_cast<v4i*>(dstT + (long long)nl * M * 2 + lc) = val;
+            }
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();
+        }
+        // row-major copy: LDS[m][n]
+#pragma unroll
+        for (int mi = 0; mi < 4; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int rl = wm + mi * 32 + 8 * q + 4 * lh, cl = wn + ni * 32 + l31;
+                    unsigned char* d0 = smem + rl * EPI_PITCH + cl * 2;
+                    *reinterpret_cast<uint16_t*>(d0) = (uint16_t)(pk[mi][ni][q].x & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(d0 + EPI_PITCH) = (uint16_t)(pk[mi][ni][q].x >> 16);
+                    *reinterpret_cast<uint16_t*>(d0 + 2 * EPI_PITCH) = (uint16_t)(pk[mi][ni][q].y & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(d0 + 3 * EPI_PITCH) = (uint16_t)(pk[mi][ni][q].y >> 16);
+                }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();
+        unsigned char* dst = (unsigned char*)g.out + ((long long)bm * N + bn) * 2;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int ml = w * 32 + i * 2 + lr2;
+            const v4i val = *reinterpret_cast<const v4i*>(smem + ml * EPI_PITCH + lc);
+            *reinterpret_cast<v4i*>(dst + (long long)ml * N * 2 + lc) = val;
         }
     }
 }
@@ -223,30 +377,44 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 template <bool FP8, int EPI>
 hipError_t launch(const GemmLpArgs& a, hipStream_t s)
 {
-    const size_t lds = 4 * TILE_BYTES;
-    static bool attr_done = false;
-    if (!attr_done) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_lp_kernel<FP8, EPI>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return e;
-        attr_done = true;
-    }
     const int nb = (a.M / TM) * (a.N / TN);
-    hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI>), dim3(nb), dim3(NT), lds, s, a);
+    hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI>), dim3(nb), dim3(NT), 0, s, a);
     return hipGetLastError();
 }
 
 }  // namespace
 
+static void resolve_act(GemmLpArgs& g)
+{
+    GemmLpArgs::ActForm& a = g.ap;
+    const float inf = __builtin_huge_valf(), p = g.act_param;
+    a = GemmLpArgs::ActForm{-inf, 0.f, 0.f, 1.f, 0.f, 1.f, 1.f, 0.f, -inf, 0.f, inf, 0.f, 0, 0, 1.f, 1.f, 1.f, 0.f, 0.f};
+    switch (g.act) {
+    case GHIP_TANH:     a.trans = 1; a.tk = 2.f; a.ta = 2.f; a.tb = -1.f; a.c0 = 1.f; a.c2 = -1.f; break;
+    case GHIP_TANHP:    a.trans = 1; a.tk = 2.f; a.ta = 2.f; a.tb = -1.f; a.c0 = 1.f; a.c2 = -1.f;
+                        a.clo = p - 1.f; a.vlo = -1.f; a.chi = 1.f - p; a.vhi = 1.f; break;
+    case GHIP_SIGMOID:  a.trans = 1; a.c0 = 0.f; a.c1 = 1.f; a.c2 = -1.f; break;
+    case GHIP_SIGMOIDP: a.trans = 1; a.c0 = 0.f; a.c1 = 1.f; a.c2 = -1.f;
+                        a.clo = p; a.vlo = 0.01f; a.chi = 1.f - p; a.vhi = 0.99f; break;
+    case GHIP_RELU:     a.thr = GHIP_OUTLIER; a.a0 = 0.f; a.step = 1; a.dhi = 1.f; a.dlo = 0.f; break;
+    case GHIP_LEAKY:    a.thr = GHIP_OUTLIER; a.a0 = p; a.step = 1; a.dhi = 1.f; a.dlo = p; break;
+    case GHIP_LINEAR:   a.a1 = p; a.c0 = p; break;
+    case GHIP_STEP:     a.thr = p; a.a0 = 0.f; a.a1 = 0.f; a.b1 = 1.f; a.c0 = 0.f; break;
+    default: break;
+    }
+}
+
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8)
 {
-    const int kq = fp8 ? 128 : 64;
+    const int kq = fp8 ? 256 : 128;  // two stages of 128 bytes of K per pass of the main loop
     return M > 0 && N > 0 && K > 0 && (M % TM) == 0 && (N % TN) == 0 && (K % kq) == 0;
 }
 
-hipError_t ghip_gemm_lp(const GemmLpArgs& a, hipStream_t s)
+hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
 {
-    if (!ghip_gemm_lp_shape_ok(a.M, a.N, a.K, a.fp8)) return hipErrorInvalidValue;
+    if (!ghip_gemm_lp_shape_ok(a_.M, a_.N, a_.K, a_.fp8)) return hipErrorInvalidValue;
+    GemmLpArgs a = a_;
+    resolve_act(a);
     if (!a.fp8) {
         switch (a.epilogue) {
         case LP_FWD_ACT: return launch<false, LP_FWD_ACT>(a, s);

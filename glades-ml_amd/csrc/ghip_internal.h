@@ -252,7 +252,15 @@ struct GemmLpArgs {
     void* out; void* outT;            // see LpEpilogue; outT may be NULL
     const float* bias;                // [N] or NULL
     const uint16_t* aux;              // LP_DGRAD: activations bf16 [M][N]
-    int act; float act_param;
+    int act; float act_param;   // resolved into `ap` by ghip_gemm_lp
+    struct ActForm {
+        // forward:  v = z < thr ? a0*z + b0 : a1*z + b1;  if (trans) v = ta / (1 + exp(-tk*z)) + tb;
+        //           v = z < clo ? vlo : v;  v = z > chi ? vhi : v
+        float thr, a0, b0, a1, b1, tk, ta, tb, clo, vlo, chi, vhi;
+        int trans;
+        // derivative in the output a:  step ? (a > 0 ? dhi : dlo) : c0 + c1*a + c2*a*a
+        int step; float dhi, dlo, c0, c1, c2;
+    } ap;
     // LP_WGRAD_SGD
     float* master; float* mom; float lr, momf, wd1, wd2, gscale;
     // fp8
