@@ -807,6 +807,25 @@ int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_o
     return 0;
 }
 
+int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* host_metrics)
+{
+    if (!n || batch < 1 || row0 < 0 || !host_metrics) return fail(GHIP_EINVAL, "bad arguments");
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
+    if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
+    const ghip_net_spec& s = n->spec;
+    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
+    TRY(reserve_batch(n, batch));
+    const int L = s.n_layers;
+    float* P = nullptr;
+    if (s.dtype == GHIP_F32) { TRY(forward_f32(n, n->dX + row0 * s.sizes[0], batch)); P = n->act[L]; }
+    else if (s.dtype == GHIP_BF16) { TRY(refresh_shadows(n)); TRY(forward_bf16(n, n->Xbf + row0 * s.sizes[0], batch)); P = n->logits; }
+    else { TRY(forward_fp8(n, n->Xbf + row0 * s.sizes[0], batch, n->out8)); P = n->out8; }
+    TRY(output_delta_f32(n, P, n->dY + row0 * s.sizes[L], nullptr, nullptr, batch));
+    n->last_batch = batch;
+    return fetch_metrics(n, host_metrics);
+}
+
 int ghip_net_quantize_fp8(ghip_net* n, float* const* host_scales, uint8_t* const* host_codes)
 {
     if (!n) return fail(GHIP_EINVAL, "net is NULL");

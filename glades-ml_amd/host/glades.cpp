@@ -1,0 +1,587 @@
+// Host side of the reference's class API (see glades.h) over the C ABI in include/glades_hip.h.
+// Citations are to the reference tree, "ML/" = "Backend/Machine Learning/".
+#include "glades.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+
+#include "glades_hip.h"
+
+namespace glades {
+
+// ------------------------------------------------------------------ LayerInfo family
+
+LayerInfo::LayerInfo(int newSize)
+    : lSize(newSize), learningRate(0.01f), momentumFactor(0.0f), weightDecay1(0.0f), weightDecay2(0.0f),
+      pDropout(0.0f), activationParam(0.0f), activationType(0)
+{
+}
+
+InputLayerInfo::InputLayerInfo(int newBatchSize, float newLearningRate, float newMomentumFactor,
+                               float newWeightDecay1, float newWeightDecay2, float newPDropout,
+                               int newActivationType, float newActivationParam)
+    : LayerInfo(0), batchSize(newBatchSize)
+{
+    learningRate = newLearningRate; momentumFactor = newMomentumFactor;
+    weightDecay1 = newWeightDecay1; weightDecay2 = newWeightDecay2; pDropout = newPDropout;
+    activationType = newActivationType; activationParam = newActivationParam;
+}
+
+HiddenLayerInfo::HiddenLayerInfo(int newSize, float newLearningRate, float newMomentumFactor,
+                                 float newWeightDecay1, float newWeightDecay2, float newPDropout,
+                                 int newActivationType, float newActivationParam)
+    : LayerInfo(newSize)
+{
+    learningRate = newLearningRate; momentumFactor = newMomentumFactor;
+    weightDecay1 = newWeightDecay1; weightDecay2 = newWeightDecay2; pDropout = newPDropout;
+    activationType = newActivationType; activationParam = newActivationParam;
+}
+
+OutputLayerInfo::OutputLayerInfo(int newSize, int newOutputType) : LayerInfo(newSize), outputType(newOutputType) {}
+
+// ------------------------------------------------------------------ NNInfo
+
+NNInfo::NNInfo(const std::string& newName) : name(newName), inputType(0), inputLayer(NULL), outputLayer(NULL) {}
+
+NNInfo::NNInfo(const std::string& newName, const NNTable& table)
+    : name(newName), inputType(0), inputLayer(NULL), outputLayer(NULL)
+{
+    if (!table.empty() && table[0].size() < 10)
+        printf("[NNINFO] Bad table size: (%d,%d)\n", (int)table.size(), (int)table[0].size());
+    fromTable(newName, table);
+}
+
+NNInfo::NNInfo(const std::string& newName, InputLayerInfo* newInputLayer,
+               const std::vector<HiddenLayerInfo*>& hidden, OutputLayerInfo* newOutputLayer)
+    : name(newName), inputType(0), inputLayer(newInputLayer), outputLayer(newOutputLayer), layers(hidden)
+{
+}
+
+NNInfo::~NNInfo()
+{
+    for (size_t i = 0; i < layers.size(); ++i) delete layers[i];
+    layers.clear();
+    delete inputLayer;
+    delete outputLayer;
+}
+
+int NNInfo::getOutputType() const { return outputLayer ? outputLayer->getOutputType() : 0; }
+float NNInfo::getPInput() const { return inputLayer ? inputLayer->getPDropout() : 0.0f; }
+int NNInfo::getBatchSize() const { return inputLayer ? inputLayer->getBatchSize() : 1; }
+int NNInfo::getHiddenLayerSize(unsigned int i) const { return (i < layers.size() && layers[i]) ? layers[i]->size() : 0; }
+unsigned int NNInfo::getOutputLayerSize() const { return outputLayer ? (unsigned int)outputLayer->size() : 0u; }
+
+// nninfo.cpp:240-373: index 0 = input row, index k = hidden row k-1; defaults when out of range
+#define NN_GETTER(NAME, TYPE, DEFAULT, INPUT_EXPR, HIDDEN_EXPR)          \
+    TYPE NNInfo::NAME(unsigned int index) const                          \
+    {                                                                    \
+        if (index > layers.size()) return DEFAULT;                       \
+        if (index == 0) return inputLayer ? (INPUT_EXPR) : (DEFAULT);    \
+        if (!layers[index - 1]) return DEFAULT;                          \
+        return layers[index - 1]->HIDDEN_EXPR;                           \
+    }
+NN_GETTER(getLearningRate, float, 0.01f, inputLayer->getLearningRate(), getLearningRate())
+NN_GETTER(getMomentumFactor, float, 0.0f, inputLayer->getMomentumFactor(), getMomentumFactor())
+NN_GETTER(getWeightDecay1, float, 0.0f, inputLayer->getWeightDecay1(), getWeightDecay1())
+// the reference returns the input row's weightDecay1 here (nninfo.cpp:305-306)
+NN_GETTER(getWeightDecay2, float, 0.0f, inputLayer->getWeightDecay1(), getWeightDecay2())
+NN_GETTER(getPDropout, float, 1.0f, inputLayer->getPDropout(), getPDropout())
+NN_GETTER(getActivationType, int, 0, inputLayer->getActivationType(), getActivationType())
+NN_GETTER(getActivationParam, float, 0.0f, inputLayer->getActivationParam(), getActivationParam())
+#undef NN_GETTER
+
+void NNInfo::setOutputType(int v) { if (outputLayer) outputLayer->setOutputType(v); }
+void NNInfo::setOutputSize(int v) { if (outputLayer) outputLayer->setSize(v); }
+void NNInfo::setBatchSize(int v) { if (inputLayer) inputLayer->setBatchSize(v); }
+void NNInfo::setLearningRate(unsigned int index, float v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setLearningRate(v); }
+    else if (layers[index - 1]) layers[index - 1]->setLearningRate(v);
+}
+void NNInfo::setMomentumFactor(unsigned int index, float v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setMomentumFactor(v); }
+    else if (layers[index - 1]) layers[index - 1]->setMomentumFactor(v);
+}
+void NNInfo::setActivationType(unsigned int index, int v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setActivationType(v); }
+    else if (layers[index - 1]) layers[index - 1]->setActivationType(v);
+}
+void NNInfo::setActivationParam(unsigned int index, float v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setActivationParam(v); }
+    else if (layers[index - 1]) layers[index - 1]->setActivationParam(v);
+}
+void NNInfo::addHiddenLayer(HiddenLayerInfo* l) { if (l) layers.push_back(l); }
+
+NNTable NNInfo::toTable() const
+{
+    NNTable t;
+    if (!inputLayer || !outputLayer) return t;
+    std::vector<float> r(10, -1.0f);
+    r[COL_SIZE] = -1.0f; r[COL_BATCH_SIZE] = (float)inputLayer->getBatchSize();
+    r[COL_LEARNING_RATE] = inputLayer->getLearningRate(); r[COL_MOMENTUM_FACTOR] = inputLayer->getMomentumFactor();
+    r[COL_WEIGHT_DECAY1] = inputLayer->getWeightDecay1(); r[COL_WEIGHT_DECAY2] = inputLayer->getWeightDecay2();
+    r[COL_PDROPOUT] = inputLayer->getPDropout(); r[COL_ACTIVATION_TYPE] = (float)inputLayer->getActivationType();
+    r[COL_ACTIVATION_PARAM] = inputLayer->getActivationParam(); r[COL_OUTPUT_TYPE] = -1.0f;
+    t.push_back(r);
+    for (size_t i = 0; i < layers.size(); ++i) {
+        const HiddenLayerInfo* h = layers[i];
+        r[COL_SIZE] = (float)h->size(); r[COL_BATCH_SIZE] = (float)inputLayer->getBatchSize();
+        r[COL_LEARNING_RATE] = h->getLearningRate(); r[COL_MOMENTUM_FACTOR] = h->getMomentumFactor();
+        r[COL_WEIGHT_DECAY1] = h->getWeightDecay1(); r[COL_WEIGHT_DECAY2] = h->getWeightDecay2();
+        r[COL_PDROPOUT] = h->getPDropout(); r[COL_ACTIVATION_TYPE] = (float)h->getActivationType();
+        r[COL_ACTIVATION_PARAM] = h->getActivationParam(); r[COL_OUTPUT_TYPE] = -1.0f;
+        t.push_back(r);
+    }
+    std::vector<float> o(10, -1.0f);
+    o[COL_SIZE] = (float)outputLayer->size(); o[COL_BATCH_SIZE] = (float)inputLayer->getBatchSize();
+    o[COL_OUTPUT_TYPE] = (float)outputLayer->getOutputType();
+    t.push_back(o);
+    return t;
+}
+
+// nninfo.cpp:738-785: first row = input row (batch size read there), last row = output row
+bool NNInfo::fromTable(const std::string& netName, const NNTable& t)
+{
+    if (t.size() < 2) return false;
+    for (size_t i = 0; i < t.size(); ++i)
+        if (t[i].size() < 10) return false;
+    name = netName;
+    for (size_t i = 0; i < layers.size(); ++i) delete layers[i];
+    layers.clear();
+    delete inputLayer; inputLayer = NULL;
+    delete outputLayer; outputLayer = NULL;
+    for (size_t i = 0; i < t.size(); ++i) {
+        const std::vector<float>& r = t[i];
+        if (i == 0)
+            inputLayer = new InputLayerInfo((int)r[COL_BATCH_SIZE], r[COL_LEARNING_RATE], r[COL_MOMENTUM_FACTOR],
+                                            r[COL_WEIGHT_DECAY1], r[COL_WEIGHT_DECAY2], r[COL_PDROPOUT],
+                                            (int)r[COL_ACTIVATION_TYPE], r[COL_ACTIVATION_PARAM]);
+        else if (i == t.size() - 1)
+            outputLayer = new OutputLayerInfo((int)r[COL_SIZE], (int)r[COL_OUTPUT_TYPE]);
+        else
+            layers.push_back(new HiddenLayerInfo((int)r[COL_SIZE], r[COL_LEARNING_RATE], r[COL_MOMENTUM_FACTOR],
+                                                 r[COL_WEIGHT_DECAY1], r[COL_WEIGHT_DECAY2], r[COL_PDROPOUT],
+                                                 (int)r[COL_ACTIVATION_TYPE], r[COL_ACTIVATION_PARAM]));
+    }
+    return true;
+}
+
+bool NNInfo::loadFile(const std::string& path)
+{
+    FILE* f = fopen(path.c_str(), "r");
+    if (!f) return false;
+    NNTable t;
+    char line[1024];
+    bool first = true;
+    while (fgets(line, sizeof(line), f)) {
+        if (first) { first = false; if (strncmp(line, "Size", 4) == 0) continue; }
+        std::vector<float> r;
+        for (char* tok = strtok(line, ",\r\n"); tok; tok = strtok(NULL, ",\r\n")) r.push_back((float)atof(tok));
+        if (r.size() >= 10) t.push_back(r);
+    }
+    fclose(f);
+    std::string base = path;
+    size_t slash = base.find_last_of('/');
+    if (slash != std::string::npos) base = base.substr(slash + 1);
+    return fromTable(base, t);
+}
+
+bool NNInfo::saveFile(const std::string& path) const
+{
+    NNTable t = toTable();
+    if (t.empty()) return false;
+    FILE* f = fopen(path.c_str(), "w");
+    if (!f) return false;
+    fprintf(f, "Size,batchSize,learningRate,momentumFactor,weightDecay1,weightDecay2,pDropout,activationType,activationParam,outputType");
+    for (size_t i = 0; i < t.size(); ++i) {
+        const std::vector<float>& r = t[i];
+        fprintf(f, "\n%d,%d,%f,%f,%f,%f,%f,%d,%f,%d", (int)r[0], (int)r[1], r[2], r[3], r[4], r[5], r[6], (int)r[7], r[8], (int)r[9]);
+    }
+    fclose(f);
+    return true;
+}
+
+// ------------------------------------------------------------------ Terminator
+
+Terminator::Terminator() : timestamp(0), epoch(0), accuracy(0.0f) {}
+
+bool Terminator::triggered(int64_t cTimestamp, int64_t cEpoch, float cAccuracy) const
+{
+    if ((timestamp > 0l) && (cTimestamp % timestamp == 0)) return true;
+    if ((epoch > 0l) && (cEpoch % epoch == 0)) return true;
+    if ((accuracy > 0.0f) && (cAccuracy >= accuracy)) return true;
+    return false;
+}
+
+// ------------------------------------------------------------------ DataInput
+
+void DataInput::denseTrain(std::vector<float>& X, std::vector<float>& Y, unsigned int& nOut) const
+{
+    const unsigned int n = getTrainSize(), f = getFeatureCount();
+    nOut = n ? (unsigned int)getTrainExpectedRow(0).size() : 0;
+    X.resize((size_t)n * f);
+    Y.resize((size_t)n * nOut);
+    for (unsigned int r = 0; r < n; ++r) {
+        std::vector<float> xr = getTrainRow(r), yr = getTrainExpectedRow(r);
+        for (unsigned int c = 0; c < f; ++c) X[(size_t)r * f + c] = c < xr.size() ? xr[c] : 0.0f;
+        for (unsigned int c = 0; c < nOut; ++c) Y[(size_t)r * nOut + c] = c < yr.size() ? yr[c] : 0.0f;
+    }
+}
+
+DenseInput::DenseInput(const float* x, const float* y, unsigned int nRows, unsigned int nFeatures, unsigned int nOutputs)
+    : X(x, x + (size_t)nRows * nFeatures), Y(y, y + (size_t)nRows * nOutputs), rows(nRows), feats(nFeatures), outs(nOutputs)
+{
+    featureIsCategorical.assign(nFeatures, false);
+}
+std::vector<float> DenseInput::getTrainRow(unsigned int i) const
+{
+    if (i >= rows) return std::vector<float>();
+    return std::vector<float>(X.begin() + (size_t)i * feats, X.begin() + (size_t)(i + 1) * feats);
+}
+std::vector<float> DenseInput::getTrainExpectedRow(unsigned int i) const
+{
+    if (i >= rows) return std::vector<float>();
+    return std::vector<float>(Y.begin() + (size_t)i * outs, Y.begin() + (size_t)(i + 1) * outs);
+}
+void DenseInput::denseTrain(std::vector<float>& x, std::vector<float>& y, unsigned int& nOut) const
+{
+    x = X; y = Y; nOut = outs;
+}
+
+// ------------------------------------------------------------------ weight sampler
+
+// ML/GMath/gmath.cpp:355-405 (Acklam's inverse normal CDF; log/sqrt on float arguments are the
+// float overloads there, the rational part is evaluated in double)
+static float norm_inv_CDF(float x)
+{
+    const double a1 = -39.69683028665376, a2 = 220.9460984245205, a3 = -275.9285104469687,
+                 a4 = 138.3577518672690, a5 = -30.66479806614716, a6 = 2.506628277459239;
+    const double b1 = -54.47609879822406, b2 = 161.5858368580409, b3 = -155.6989798598866,
+                 b4 = 66.80131188771972, b5 = -13.280681552885721;
+    const double c1 = -0.007784894002430293, c2 = -0.3223964580411365, c3 = -2.400758277161838,
+                 c4 = -2.549732539343734, c5 = 4.374664141464968, c6 = 2.938163982698783;
+    const double d1 = 0.007784695709041462, d2 = 0.3224671290700398, d3 = 2.445134137142996,
+                 d4 = 3.754408661907416;
+    float p_low = 0.02452;
+    float p_high = 1 - p_low;
+    if (x < p_low) {
+        double q = sqrtf(-2 * logf(x));
+        return (float)((((((c1 * q + c2) * q + c3) * q + c4) * q + c5) * q + c6) / ((((d1 * q + d2) * q + d3) * q + d4) * q + 1));
+    } else if (x < p_high) {
+        double q = x - 0.5;
+        double r = q * q;
+        return (float)(((((((a1 * r + a2) * r + a3) * r + a4) * r + a5) * r + a6) * q) /
+                       (((((b1 * r + b2) * r + b3) * r + b4) * r + b5) * r + 1));
+    }
+    double q = sqrtf(-2 * logf(1 - x));
+    return (float)(-(((((c1 * q + c2) * q + c3) * q + c4) * q + c5) * q + c6) / ((((d1 * q + d2) * q + d3) * q + d4) * q + 1));
+}
+
+static float normal_pdf(float z) { return (float)((1 / sqrt(6.2831853)) * expf(-(z * z) / 2)); }
+
+void xavierLayer(int fanIn, int nOut, int activationType, float* W)
+{
+    const unsigned int num_layers = 2048;
+    static float zigg[2049];
+    float normal_CDF = 1.0;
+    for (unsigned int i = 1; i < num_layers; i++) {
+        normal_CDF = normal_CDF - (1 / ((float)num_layers * 2));
+        zigg[i] = norm_inv_CDF(normal_CDF);
+    }
+    zigg[0] = zigg[1];
+    zigg[num_layers] = 0;
+    float std_dev = (activationType != GMath::RELU) ? sqrtf(1 / (float)fanIn) : sqrtf(2 / (float)fanIn);
+    for (int o = 0; o < nOut; ++o)
+        for (int e = 0; e < fanIn; ++e) {
+            bool accepted = false;
+            float x = 0.0f;
+            while (!accepted) {
+                int layer = rand() % 2048;
+                x = rand() / (RAND_MAX / zigg[layer]);
+                if (layer == 0) continue;
+                else if (x < zigg[layer + 1]) accepted = true;
+                else if (x > zigg[layer + 1]) {
+                    float randU = rand() / RAND_MAX;  // integer division, as the reference writes it
+                    float y = normal_pdf(zigg[layer]) + randU * (normal_pdf(zigg[layer - 1] - normal_pdf(zigg[layer])));
+                    if (y < normal_pdf(x)) accepted = true;
+                }
+            }
+            W[(size_t)o * fanIn + e] = x * std_dev;
+        }
+}
+
+// ------------------------------------------------------------------ NNetwork
+
+static int64_t g_next_id = 1;
+
+NNetwork::NNetwork()
+    : di(NULL), skeleton(NULL), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
+      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallCorrect(0),
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
+{
+}
+
+NNetwork::NNetwork(NNInfo* newNNInfo)
+    : di(NULL), skeleton(newNNInfo), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
+      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallCorrect(0),
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
+{
+}
+
+NNetwork::~NNetwork() { clean(); }
+
+void NNetwork::clean()
+{
+    if (dev) ghip_net_destroy(dev);
+    dev = NULL;
+    di = NULL;  // borrowed, like the skeleton (network.cpp:745-762)
+}
+
+std::string NNetwork::getName() const { return skeleton ? skeleton->getName() : std::string(); }
+
+bool NNetwork::load(const std::string& path)
+{
+    NNInfo* info = new NNInfo("");
+    if (!info->loadFile(path)) { delete info; return false; }
+    skeleton = info;  // like the reference, the loaded skeleton is never freed by the network
+    return true;
+}
+
+bool NNetwork::save(const std::string& path) const { return skeleton ? skeleton->saveFile(path) : false; }
+
+void NNetwork::train(DataInput* d) { run(d, RUN_TRAIN); }
+void NNetwork::test(DataInput* d) { run(d, RUN_TEST); }
+
+bool NNetwork::setWeights(unsigned int layer, const std::vector<float>& W)
+{
+    if (!skeleton || layer > (unsigned int)skeleton->numHiddenLayers()) return false;
+    if (dev) {
+        if (ghip_net_set_params(dev, (int)layer, W.data(), NULL, 0) != 0) { lastError = ghip_last_error(); return false; }
+        return true;
+    }
+    if (initW.size() <= layer) initW.resize(layer + 1);
+    initW[layer] = W;
+    return true;
+}
+
+bool NNetwork::setBias(unsigned int layer, const std::vector<float>& bias)
+{
+    if (!skeleton || layer > (unsigned int)skeleton->numHiddenLayers()) return false;
+    if (initB.size() <= layer) initB.resize(layer + 1);
+    initB[layer] = bias;
+    return true;
+}
+
+std::vector<float> NNetwork::getWeights(unsigned int layer)
+{
+    std::vector<float> W;
+    if (!dev || !skeleton || layer > (unsigned int)skeleton->numHiddenLayers()) return W;
+    const int ni = layer == 0 ? (int)nFeat : skeleton->getHiddenLayerSize(layer - 1);
+    const int no = layer == (unsigned int)skeleton->numHiddenLayers() ? (int)nOut : skeleton->getHiddenLayerSize(layer);
+    W.resize((size_t)ni * no);
+    if (ghip_net_get_params(dev, (int)layer, W.data(), NULL, 0) != 0) { lastError = ghip_last_error(); W.clear(); }
+    return W;
+}
+
+std::vector<float> NNetwork::getBias(unsigned int layer)
+{
+    std::vector<float> b;
+    if (!dev || !skeleton || layer > (unsigned int)skeleton->numHiddenLayers()) return b;
+    const int no = layer == (unsigned int)skeleton->numHiddenLayers() ? (int)nOut : skeleton->getHiddenLayerSize(layer);
+    b.resize(mode == MODE_EXACT ? 1 : (size_t)no);
+    if (ghip_net_get_params(dev, (int)layer, NULL, b.data(), (int)b.size()) != 0) { lastError = ghip_last_error(); b.clear(); }
+    return b;
+}
+
+// LayerBuilder::build (ML/State/LayerBuilder.cpp:54-267): table to the device, weights sampled
+// in the reference's order (hidden layers, then the output layer, node by node) unless injected.
+bool NNetwork::build()
+{
+    std::vector<float> X, Y;
+    di->denseTrain(X, Y, nOut);
+    nRows = di->getTrainSize();
+    nFeat = di->getFeatureCount();
+    const int H = skeleton->numHiddenLayers();
+    if (H + 1 > GHIP_MAX_LAYERS) { lastError = "too many layers"; return false; }
+    if (nOut != skeleton->getOutputLayerSize()) { lastError = "expected rows do not match the output layer size"; return false; }
+    ghip_net_spec s;
+    memset(&s, 0, sizeof(s));
+    s.n_layers = H + 1;
+    s.sizes[0] = (int)nFeat;
+    for (int i = 0; i < H; ++i) s.sizes[i + 1] = skeleton->getHiddenLayerSize(i);
+    s.sizes[H + 1] = (int)nOut;
+    for (int l = 0; l <= H; ++l) {
+        s.lr[l] = skeleton->getLearningRate(l); s.mom[l] = skeleton->getMomentumFactor(l);
+        s.wd1[l] = skeleton->getWeightDecay1(l); s.wd2[l] = skeleton->getWeightDecay2(l);
+        s.act[l] = skeleton->getActivationType(l); s.act_param[l] = skeleton->getActivationParam(l);
+        if (skeleton->getPDropout(l) != 0.0f) { lastError = "dropout is not supported on this path"; return false; }
+    }
+    s.batch = skeleton->getBatchSize();
+    s.cost = skeleton->getOutputType();
+    s.mode = mode == MODE_EXACT ? GHIP_MODE_EXACT : GHIP_MODE_CANONICAL;
+    s.dtype = dtype == DTYPE_BF16 ? GHIP_BF16 : GHIP_F32;
+    s.bias_mode = biasMode;
+    if (ghip_net_create(&s, &dev) != 0) { lastError = ghip_last_error(); dev = NULL; return false; }
+    for (int l = 0; l <= H; ++l) {
+        const int ni = s.sizes[l], no = s.sizes[l + 1];
+        std::vector<float> W;
+        if ((size_t)l < initW.size() && initW[l].size() == (size_t)ni * no) {
+            W = initW[l];
+        } else {
+            W.resize((size_t)ni * no);
+            // the output layer is scaled by the activation type of index H-1 (LayerBuilder.cpp:243-265)
+            const int at = skeleton->getActivationType(l < H ? l : (H > 0 ? H - 1 : 0));
+            xavierLayer(ni, no, at, W.data());
+        }
+        const float* bp = NULL;
+        int bl = 0;
+        if ((size_t)l < initB.size() && !initB[l].empty()) { bp = initB[l].data(); bl = (int)initB[l].size(); }
+        if (ghip_net_set_params(dev, l, W.data(), bp, bl) != 0) { lastError = ghip_last_error(); return false; }
+    }
+    if (ghip_net_set_dataset(dev, X.data(), Y.data(), (int64_t)nRows) != 0) { lastError = ghip_last_error(); return false; }
+    return true;
+}
+
+// NNetwork::run (ML/Networks/network.cpp:114-397)
+void NNetwork::run(DataInput* newDataInput, int runType)
+{
+    if (!skeleton) return;
+    if (!newDataInput) return;
+    di = newDataInput;
+    if ((di->getTrainSize() <= 0) || (di->getFeatureCount() <= 0)) return;
+    if (epochs == 0 && !dev) {
+        if (!build()) {
+            if (dev) ghip_net_destroy(dev);
+            dev = NULL;
+            return;
+        }
+    }
+    if (!dev) return;
+    minibatchSize = skeleton->getBatchSize();
+    if (runType == RUN_TRAIN) printf("[NN] Training...\n");
+    else if (runType == RUN_TEST) printf("[NN] Testing...\n");
+
+    const bool want_preds = (size_t)nRows * nOut <= (1u << 20);
+    std::vector<float> preds(want_preds ? (size_t)nRows * nOut : 0);
+    std::vector<float> Ylast = di->getTrainExpectedRow(nRows - 1);
+    running = true;
+    while (running) {
+        if (mode == MODE_EXACT) {
+            // several epochs per launch where the stop conditions allow it: up to the next epoch
+            // multiple, 1 when a wall-clock condition has to be polled every epoch
+            int chunk = 16;
+            if (runType == RUN_TEST || terminator.getTimestamp() > 0) chunk = 1;
+            else if (terminator.getEpoch() > 0) {
+                const int64_t e = terminator.getEpoch();
+                int64_t left = e - ((int64_t)epochs % e);
+                chunk = (int)(left < 4096 ? left : 4096);
+            }
+            std::vector<ghip_metrics> ms(chunk);
+            int ran = 0;
+            if (ghip_net_run_epochs_exact(dev, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran,
+                                          want_preds ? preds.data() : NULL) != 0) {
+                lastError = ghip_last_error();
+                break;
+            }
+            if (ran <= 0) break;
+            epochs += ran;
+            overallTotalError = ms[ran - 1].loss;
+            overallTotalAccuracy = ms[ran - 1].accuracy;
+            overallCorrect = ms[ran - 1].correct;
+        } else {
+            // canonical mode: batches [k*mb, (k+1)*mb), the last one averaged over its true size
+            const int mb = minibatchSize > 0 ? minibatchSize : (int)nRows;
+            double loss = 0.0, acc = 0.0;
+            int64_t correct = 0;
+            bool failed = false;
+            for (unsigned int r0 = 0; r0 < nRows && !failed; r0 += mb) {
+                const int b = (int)((nRows - r0) < (unsigned int)mb ? (nRows - r0) : (unsigned int)mb);
+                ghip_metrics m;
+                int rc = (runType == RUN_TRAIN) ? ghip_net_train_step(dev, r0, b, &m) : ghip_net_eval_resident(dev, r0, b, &m);
+                if (rc != 0) { lastError = ghip_last_error(); failed = true; break; }
+                loss += (double)m.loss * b; acc += (double)m.accuracy * b; correct += m.correct;
+            }
+            if (failed) break;
+            ++epochs;
+            overallTotalError = (float)(loss / nRows);
+            overallTotalAccuracy = (float)(acc / nRows);
+            overallCorrect = correct;
+        }
+        if (runType == RUN_TRAIN) {
+            printf("\33[2K[NN] %d\t%f%%\r", epochs, overallTotalAccuracy);
+            fflush(stdout);
+        }
+        if (terminator.triggered(time(NULL), epochs, overallTotalAccuracy)) break;
+        if (runType == RUN_TEST) break;
+    }
+    if (want_preds && mode == MODE_EXACT) {
+        results.clear();  // the reference's list holds the last row's (expected, predicted) pairs
+        for (unsigned int o = 0; o < nOut; ++o) {
+            results.push_back(o < Ylast.size() ? Ylast[o] : 0.0f);
+            results.push_back(preds[(size_t)(nRows - 1) * nOut + o]);
+        }
+    }
+    if (runType == RUN_TRAIN) printf("\n");
+    else if (runType == RUN_TEST) printf("[NN] %s Accuracy: %f%%\n", skeleton->getName().c_str(), overallTotalAccuracy);
+    running = false;
+}
+
+// ------------------------------------------------------------------ facade (ML/main.cpp:51-243)
+
+void init() { ghip_init(0); }
+
+MetaNetwork* train(NNetwork* net, DataInput* d)
+{
+    if (!net || !d) return NULL;
+    MetaNetwork* m = new MetaNetwork(net->getName());
+    m->addSubnet(net);
+    return train(m, d);
+}
+
+MetaNetwork* train(NNInfo* info, DataInput* d)
+{
+    if (!info || !d) return NULL;
+    return train(new NNetwork(info), d);
+}
+
+MetaNetwork* train(MetaNetwork* m, DataInput* d)
+{
+    if (!m || !d) return NULL;
+    for (unsigned int i = 0; i < m->size(); ++i)
+        if (m->getSubnets()[i]) m->getSubnets()[i]->train(d);
+    return m;
+}
+
+MetaNetwork* test(NNetwork* net, DataInput* d)
+{
+    if (!net || !d) return NULL;
+    MetaNetwork* m = new MetaNetwork(net->getName());
+    m->addSubnet(net);
+    return test(m, d);
+}
+
+MetaNetwork* test(NNInfo* info, DataInput* d)
+{
+    if (!info || !d) return NULL;
+    return test(new NNetwork(info), d);
+}
+
+MetaNetwork* test(MetaNetwork* m, DataInput* d)
+{
+    if (!m || !d) return NULL;
+    for (unsigned int i = 0; i < m->size(); ++i)
+        if (m->getSubnets()[i]) m->getSubnets()[i]->test(d);
+    return m;
+}
+
+}  // namespace glades

@@ -1,0 +1,307 @@
+// glades.h -- the reference's C++ network/training API for the dense feed-forward path, backed
+// by the gfx950 library behind include/glades_hip.h.
+//
+// Same class names, method names, argument order and error behaviour (silent early returns,
+// NULL / false; nothing throws) as the reference, with std types where the reference uses the
+// shmea containers (GString -> std::string, GList -> std::vector<float>, GTable -> rows of
+// floats).  Citations are to the reference tree, "ML/" = "Backend/Machine Learning/".
+//
+//   GMath constants        ML/GMath/gmath.h:35-54
+//   LayerInfo family       ML/Structure/{layerinfo,inputlayerinfo,hiddenlayerinfo,outputlayerinfo}.h
+//   NNInfo                 ML/Structure/nninfo.h:41-127 (index-shifted getters: nninfo.cpp:240-373)
+//   Terminator             ML/State/Terminator.h:27-51
+//   DataInput              ML/DataObjects/DataInput.h:26-50
+//   NNetwork               ML/Networks/network.h:59-141
+//   MetaNetwork            ML/Networks/metanetwork.h:44-64
+//   glades::init/train/test  ML/main.h:44-54
+#ifndef GLADES_AMD_HOST_H
+#define GLADES_AMD_HOST_H
+
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+struct ghip_net;
+
+namespace glades {
+
+class GMath
+{
+public:
+    static constexpr float INLIER = 0.954f;
+    static constexpr float OUTLIER = 0.046f;
+    static const int REGRESSION = 0, CLASSIFICATION = 1, KL = 2;
+    static const int TANH = 0, TANHP = 1, SIGMOID = 2, SIGMOIDP = 3, LINEAR = 4, RELU = 5, LEAKY = 6, STEP = 7;
+    static const int SOFTMAX = 8;  // extension: canonical mode output layer only
+    static const int MINMAX = 0, ZSCORE = 1;
+};
+
+class LayerInfo
+{
+protected:
+    int lSize;
+    float learningRate, momentumFactor, weightDecay1, weightDecay2, pDropout, activationParam;
+    int activationType;
+
+public:
+    explicit LayerInfo(int newSize);
+    virtual ~LayerInfo() {}
+    int size() const { return lSize; }
+    float getLearningRate() const { return learningRate; }
+    float getMomentumFactor() const { return momentumFactor; }
+    float getWeightDecay1() const { return weightDecay1; }
+    float getWeightDecay2() const { return weightDecay2; }
+    float getPDropout() const { return pDropout; }
+    int getActivationType() const { return activationType; }
+    float getActivationParam() const { return activationParam; }
+    void setSize(int v) { lSize = v; }
+    void setLearningRate(float v) { learningRate = v; }
+    void setMomentumFactor(float v) { momentumFactor = v; }
+    void setWeightDecay1(float v) { weightDecay1 = v; }
+    void setWeightDecay2(float v) { weightDecay2 = v; }
+    void setPDropout(float v) { pDropout = v; }
+    void setActivationType(int v) { activationType = v; }
+    void setActivationParam(float v) { activationParam = v; }
+};
+
+class InputLayerInfo : public LayerInfo
+{
+    int batchSize;
+
+public:
+    // argument order of inputlayerinfo.cpp:29-32
+    InputLayerInfo(int newBatchSize, float newLearningRate, float newMomentumFactor, float newWeightDecay1,
+                   float newWeightDecay2, float newPDropout, int newActivationType, float newActivationParam);
+    int getBatchSize() const { return batchSize; }
+    void setBatchSize(int v) { batchSize = v; }
+};
+
+class HiddenLayerInfo : public LayerInfo
+{
+public:
+    // argument order of hiddenlayerinfo.cpp:31-34
+    HiddenLayerInfo(int newSize, float newLearningRate, float newMomentumFactor, float newWeightDecay1,
+                    float newWeightDecay2, float newPDropout, int newActivationType, float newActivationParam);
+};
+
+class OutputLayerInfo : public LayerInfo
+{
+    int outputType;
+
+public:
+    OutputLayerInfo(int newSize, int newOutputType);
+    int getOutputType() const { return outputType; }
+    void setOutputType(int v) { outputType = v; }
+};
+
+// One row of the 10-column table the reference stores a network skeleton in
+// (nninfo.h:69-78: Size,batchSize,learningRate,momentumFactor,weightDecay1,weightDecay2,pDropout,
+//  activationType,activationParam,outputType).
+typedef std::vector<std::vector<float> > NNTable;
+
+class NNInfo
+{
+    std::string name;
+    int inputType;
+    InputLayerInfo* inputLayer;
+    OutputLayerInfo* outputLayer;
+    std::vector<HiddenLayerInfo*> layers;
+
+public:
+    static const int BATCH_FULL = 0;
+    static const int BATCH_STOCHASTIC = 1;
+    static const int COL_SIZE = 0, COL_BATCH_SIZE = 1, COL_LEARNING_RATE = 2, COL_MOMENTUM_FACTOR = 3,
+                     COL_WEIGHT_DECAY1 = 4, COL_WEIGHT_DECAY2 = 5, COL_PDROPOUT = 6, COL_ACTIVATION_TYPE = 7,
+                     COL_ACTIVATION_PARAM = 8, COL_OUTPUT_TYPE = 9;
+
+    explicit NNInfo(const std::string& newName);
+    NNInfo(const std::string& newName, const NNTable& table);  // nninfo.cpp:70-82,738-785
+    NNInfo(const std::string& newName, InputLayerInfo*, const std::vector<HiddenLayerInfo*>&, OutputLayerInfo*);
+    ~NNInfo();  // owns and deletes its LayerInfos (nninfo.cpp:88-104)
+
+    std::string getName() const { return name; }
+    int getInputType() const { return inputType; }
+    int getOutputType() const;
+    float getPInput() const;
+    int getBatchSize() const;
+    InputLayerInfo* getInputLayer() const { return inputLayer; }
+    std::vector<HiddenLayerInfo*> getLayers() const { return layers; }
+    int numHiddenLayers() const { return (int)layers.size(); }
+    int getHiddenLayerSize(unsigned int) const;
+    unsigned int getOutputLayerSize() const;
+    // index 0 reads the input row, index k >= 1 the hidden row k-1 (nninfo.cpp:240-373);
+    // getWeightDecay2(0) returns the input row's weightDecay1, as the reference does (:305-306)
+    float getLearningRate(unsigned int) const;
+    float getMomentumFactor(unsigned int) const;
+    float getWeightDecay1(unsigned int) const;
+    float getWeightDecay2(unsigned int) const;
+    float getPDropout(unsigned int) const;
+    int getActivationType(unsigned int) const;
+    float getActivationParam(unsigned int) const;
+
+    void setName(const std::string& v) { name = v; }
+    void setOutputType(int);
+    void setOutputSize(int);
+    void setBatchSize(int);
+    void setLearningRate(unsigned int, float);
+    void setMomentumFactor(unsigned int, float);
+    void setActivationType(unsigned int, int);
+    void setActivationParam(unsigned int, float);
+    void addHiddenLayer(HiddenLayerInfo*);
+
+    NNTable toTable() const;
+    bool fromTable(const std::string& netName, const NNTable& table);
+    // CSV form of the table as the reference's fixtures hold it (header line + rows)
+    bool loadFile(const std::string& path);
+    bool saveFile(const std::string& path) const;
+};
+
+class Terminator
+{
+    int64_t timestamp, epoch;
+    float accuracy;
+
+public:
+    Terminator();
+    int64_t getTimestamp() const { return timestamp; }
+    int64_t getEpoch() const { return epoch; }
+    float getAccuracy() const { return accuracy; }
+    void setTimestamp(int64_t v) { timestamp = v; }
+    void setEpoch(int64_t v) { epoch = v; }
+    void setAccuracy(float v) { accuracy = v; }
+    bool triggered(int64_t cTimestamp, int64_t cEpoch, float cAccuracy) const;  // Terminator.cpp:63-78
+};
+
+class DataInput
+{
+public:
+    static const int CSV = 0, IMAGE = 1, TEXT = 2;
+    std::vector<bool> featureIsCategorical;
+    virtual ~DataInput() {}
+    virtual void import(std::string) = 0;
+    virtual std::vector<float> getTrainRow(unsigned int) const = 0;
+    virtual std::vector<float> getTrainExpectedRow(unsigned int) const = 0;
+    virtual std::vector<float> getTestRow(unsigned int) const = 0;
+    virtual std::vector<float> getTestExpectedRow(unsigned int) const = 0;
+    virtual unsigned int getTrainSize() const = 0;
+    virtual unsigned int getTestSize() const = 0;
+    virtual unsigned int getFeatureCount() const = 0;
+    virtual int getType() const = 0;
+    // dense views; the default builds them from the row getters
+    virtual void denseTrain(std::vector<float>& X, std::vector<float>& Y, unsigned int& nOut) const;
+};
+
+// In-memory table (no counterpart class in the reference; plays the role NumberInput's
+// trainTable / trainExpectedTable play after import)
+class DenseInput : public DataInput
+{
+    std::vector<float> X, Y;
+    unsigned int rows, feats, outs;
+
+public:
+    DenseInput(const float* x, const float* y, unsigned int nRows, unsigned int nFeatures, unsigned int nOutputs);
+    void import(std::string) {}
+    std::vector<float> getTrainRow(unsigned int) const;
+    std::vector<float> getTrainExpectedRow(unsigned int) const;
+    std::vector<float> getTestRow(unsigned int i) const { return getTrainRow(i); }
+    std::vector<float> getTestExpectedRow(unsigned int i) const { return getTrainExpectedRow(i); }
+    unsigned int getTrainSize() const { return rows; }
+    unsigned int getTestSize() const { return 0; }
+    unsigned int getFeatureCount() const { return feats; }
+    int getType() const { return CSV; }
+    void denseTrain(std::vector<float>& x, std::vector<float>& y, unsigned int& nOut) const;
+};
+
+class MetaNetwork;
+
+class NNetwork
+{
+    friend class MetaNetwork;
+    DataInput* di;
+    NNInfo* skeleton;
+    ghip_net* dev;
+    volatile bool running;
+    int netType, epochs, mode, dtype, biasMode;
+    float overallTotalError, overallTotalAccuracy;
+    int64_t overallCorrect;
+    int minibatchSize;
+    int64_t id;
+    std::vector<float> results;                 // (expected, predicted) pairs of the last row
+    std::vector<std::vector<float> > initW;     // weights injected before the first run
+    std::vector<std::vector<float> > initB;
+    unsigned int nRows, nFeat, nOut;
+    std::string lastError;
+
+    void run(DataInput*, int);
+    bool build();
+    void clean();
+
+public:
+    static const int TYPE_DFF = 0, TYPE_RNN = 1;
+    static const int RUN_TRAIN = 0, RUN_TEST = 1, RUN_VALIDATE = 2;
+    static const int MODE_EXACT = 0, MODE_CANONICAL = 1;      // extension
+    static const int DTYPE_F32 = 0, DTYPE_BF16 = 1;           // extension (canonical mode)
+
+    Terminator terminator;
+
+    NNetwork();
+    explicit NNetwork(NNInfo*);
+    virtual ~NNetwork();
+    bool getRunning() const { return running; }
+    int getEpochs() const { return epochs; }
+    void stop() { running = false; }
+
+    bool load(const std::string& path);  // reads an NNInfo table file (network.cpp:701-712)
+    bool save(const std::string& path) const;
+
+    void train(DataInput*);
+    void test(DataInput*);
+
+    int64_t getID() const { return id; }
+    std::string getName() const;
+    NNInfo* getNNInfo() { return skeleton; }
+    float getAccuracy() const { return overallTotalAccuracy; }
+    std::vector<float> getResults() const { return results; }
+
+    // ---- absent from the reference (its loss has no getter and its weights are not reachable)
+    float getLoss() const { return overallTotalError; }
+    int64_t getCorrect() const { return overallCorrect; }
+    void setMode(int newMode, int newDtype = DTYPE_F32) { mode = newMode; dtype = newDtype; }
+    void setSequentialBias(bool faithful) { biasMode = faithful ? 0 : 1; }
+    // layer = weight layer 0..numHiddenLayers(); W is [n_out][n_in] row-major
+    bool setWeights(unsigned int layer, const std::vector<float>& W);
+    bool setBias(unsigned int layer, const std::vector<float>& bias);  // 1 value (exact) or n_out
+    std::vector<float> getWeights(unsigned int layer);
+    std::vector<float> getBias(unsigned int layer);
+    std::string getLastError() const { return lastError; }
+};
+
+class MetaNetwork
+{
+    std::string name;
+    std::vector<NNetwork*> subnets;
+
+public:
+    explicit MetaNetwork(const std::string& newName) : name(newName) {}
+    std::string getName() const { return name; }
+    void addSubnet(NNetwork* n) { if (n) subnets.push_back(n); }
+    const std::vector<NNetwork*>& getSubnets() const { return subnets; }
+    unsigned int size() const { return (unsigned int)subnets.size(); }
+};
+
+void init();
+// ML/main.cpp:82-243: wrap in a MetaNetwork the caller owns, run every subnet on the same data
+MetaNetwork* train(NNInfo*, DataInput*);
+MetaNetwork* train(NNetwork*, DataInput*);
+MetaNetwork* train(MetaNetwork*, DataInput*);
+MetaNetwork* test(NNInfo*, DataInput*);
+MetaNetwork* test(NNetwork*, DataInput*);
+MetaNetwork* test(MetaNetwork*, DataInput*);
+
+// The reference's weight sampler (ML/State/layer.cpp:196-217, ML/State/node.cpp:241-276): draws
+// from libc rand(), so srand(seed) reproduces the reference's initial weights for a layer.
+void xavierLayer(int fanIn, int nOut, int activationType, float* W);
+
+}  // namespace glades
+#endif

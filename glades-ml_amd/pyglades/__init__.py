@@ -21,7 +21,7 @@ BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
 EXPORTS = [
     "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact",
-    "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident",
+    "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
     "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
     "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
 ]
@@ -77,6 +77,7 @@ def load():
             "ghip_net_last_metrics": (i, [vp, C.POINTER(Metrics)]),
             "ghip_net_forward": (i, [vp, vp, i, vp]),
             "ghip_net_forward_resident": (i, [vp, i64, i, vp]),
+            "ghip_net_eval_resident": (i, [vp, i64, i, C.POINTER(Metrics)]),
             "ghip_net_quantize_fp8": (i, [vp, vp, vp]),
             "ghip_net_sync": (i, [vp]),
             "ghip_net_profile": (i, [vp, i]),
@@ -211,6 +212,11 @@ class Net:
 
     def forward_resident(self, row0, batch, out_ptr=None):
         _check(self.lib.ghip_net_forward_resident(self.h, row0, batch, C.c_void_p(out_ptr) if out_ptr else None))
+
+    def eval_resident(self, row0, batch):
+        m = Metrics()
+        _check(self.lib.ghip_net_eval_resident(self.h, row0, batch, C.byref(m)))
+        return m
 
     def quantize_fp8(self, want=True):
         if not want:

@@ -137,6 +137,10 @@ int ghip_net_forward(ghip_net* net, const float* host_X, int batch, float* host_
  * dev_out (fp32, batch x sizes[n_layers], may be NULL) receives a device-to-device copy. */
 int ghip_net_forward_resident(ghip_net* net, int64_t row0, int batch, float* dev_out);
 
+/* Canonical mode RUN_TEST pass (network.cpp:109-112,372-373) on rows [row0,row0+batch) of the
+ * resident table: forward and metrics, no parameter changes. */
+int ghip_net_eval_resident(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);
+
 /* GHIP_FP8_INFER: quantises the current fp32 weights to e4m3 with one fp32 scale per output
  * channel (scale = amax(row)/448).  host_scales[l] (may be NULL) receives sizes[l+1] scales and
  * host_codes[l] (may be NULL) the sizes[l+1]*sizes[l] code bytes.  No reference counterpart (the
