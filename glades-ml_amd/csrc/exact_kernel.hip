@@ -9,7 +9,7 @@
 //   edge update  one lane per edge (delta push, window sum, conditional apply)
 //   back-prop    one lane per input node, outputs visited in ascending order with the
 //                reference's doubling accumulator  e <- e + (e + d*w)   (network.cpp:660-662)
-//   bias, loss   one designated lane, in the reference's visiting order
+//   bias, loss   one wavefront / one designated lane, in the reference's visiting order
 // Every fp32 operation is written with explicit round-to-nearest intrinsics so that nothing is
 // contracted into an FMA or re-associated: the arithmetic order is the reference's.
 //
@@ -22,6 +22,23 @@
 namespace {
 
 constexpr int kPrefetch = 4;  // values per lane of the next row held in registers
+
+// The reference updates the scalar layer bias once per (input, output) pair (network.cpp:654-656):
+// bias -= lr*d[o] for o = 0..n_out-1, repeated n_in times -- one dependent chain of n_in*n_out fp32
+// subtractions whose rounding order must be kept.  The n_out values sit in NP registers (padded
+// with zeros: b - 0 is exact), so a step is a single subtract with no memory access.
+template <int NP>
+__device__ __forceinline__ float bias_chain(float b, const float* bs, int no, int ni)
+{
+    float x[NP];
+#pragma unroll
+    for (int k = 0; k < NP; ++k) x[k] = (k < no) ? bs[k] : 0.0f;
+    for (int i = 0; i < ni; ++i) {
+#pragma unroll
+        for (int k = 0; k < NP; ++k) b = __fsub_rn(b, x[k]);
+    }
+    return b;
+}
 
 template <bool kLds>
 __global__ void __launch_bounds__(1024)
@@ -124,7 +141,7 @@ exact_kernel(ExactLaunch p)
                 for (int o = tid; o < no; o += T) {
                     const float* w = Wl + o * ld;
                     float z = 0.0f;
-#pragma unroll 8
+#pragma unroll 16
                     for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
                     if (l != 0) z = __fadd_rn(z, bl);
                     aout[o] = ghip_squash<true>(z, act, par);
@@ -141,7 +158,7 @@ exact_kernel(ExactLaunch p)
                 int ip = -1, iy = -1;
                 for (int o = 0; o < nout; ++o) {
                     const float pr = pred[o], ex = sy[o];
-                    tot_err = __fadd_rn(tot_err, ghip_cost<true>(ex, pr, data_size, p.cost));
+                    tot_err = __fadd_rn(tot_err, ghip_cost<false>(ex, pr, data_size, p.cost));
                     tot_acc = __fadd_rn(tot_acc, ghip_accuracy_term(pr, ex));
                     if (pr > mp) { mp = pr; ip = o; }
                     if (ex > my) { my = ex; iy = o; }
@@ -201,19 +218,28 @@ exact_kernel(ExactLaunch p)
                         }
                     }
                     // ---- scalar bias of the in-layer (network.cpp:654-656)
-                    if (tid == serial && l != 0) {
+                    // The n_in*n_out subtractions are one dependent chain; it runs in the last
+                    // wavefront with the lr*d values held in registers (bias_chain below).
+                    if ((tid >> 6) == (T >> 6) - 1 && l != 0) {
                         float b = sbias[l];
                         if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
-                            for (int i = 0; i < ni; ++i) {
+                            if (no <= 4) b = bias_chain<4>(b, bs, no, ni);
+                            else if (no <= 8) b = bias_chain<8>(b, bs, no, ni);
+                            else if (no <= 16) b = bias_chain<16>(b, bs, no, ni);
+                            else if (no <= 32) b = bias_chain<32>(b, bs, no, ni);
+                            else if (no <= 64) b = bias_chain<64>(b, bs, no, ni);
+                            else {
+                                for (int i = 0; i < ni; ++i) {
 #pragma unroll 8
-                                for (int o = 0; o < no; ++o) b = __fsub_rn(b, bs[o]);
+                                    for (int o = 0; o < no; ++o) b = __fsub_rn(b, bs[o]);
+                                }
                             }
                         } else {
                             float s = 0.0f;
                             for (int o = 0; o < no; ++o) s = __fadd_rn(s, bs[o]);
                             b = __fsub_rn(b, __fmul_rn((float)ni, s));
                         }
-                        sbias[l] = b;
+                        if (tid == serial) sbias[l] = b;
                     }
                     __syncthreads();
                     // ---- error partials of the in-layer with the UPDATED weights
@@ -225,7 +251,7 @@ exact_kernel(ExactLaunch p)
                         const float lrn = p.lr[l - 1];
                         for (int i = tid; i < ni; i += T) {
                             float e = 0.0f;
-#pragma unroll 8
+#pragma unroll 16
                             for (int o = 0; o < no; ++o)
                                 e = __fadd_rn(e, __fadd_rn(e, __fmul_rn(dl[o], Wl[o * ld + i])));
                             // the reference always passes 0.01 here (network.cpp:617-618)

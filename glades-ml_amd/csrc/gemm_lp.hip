@@ -12,13 +12,13 @@
 //             also writes the bf16 W and W^T used by the next step.
 //
 // Tile: 256 x 256 outputs per workgroup of 8 wavefronts laid out 2 (M) x 4 (N); each wavefront owns
-// 128 x 64 = 4 x 2 accumulators of 32x32 (128 VGPRs).  K advances in stages of 64 bytes per row
-// (32 bf16 / 64 e4m3).  LDS holds a ring of 4 stages (4 x 32 KiB) filled by LDS-direct global
-// loads (global_load_lds_dwordx4: no VGPR staging, no ds_write); three stages are in flight while
-// one is consumed, so the s_waitcnt before each barrier only waits for loads issued three stages
-// earlier (the single-stage look-ahead of a plain double buffer left the matrix cores waiting on
-// L2/HBM latency ~30 % of the time).  Rows are 64 B; 16-byte chunks are XOR-swizzled with the row
-// index so that the per-lane 16-byte operand reads spread over all 64 banks.
+// 128 x 64 = 4 x 2 accumulators of 32x32 (128 VGPRs).  K advances in stages of 128 bytes per row
+// (64 bf16 / 128 e4m3: whole cache lines).  LDS holds two stages (2 x 64 KiB) filled by LDS-direct
+// global loads (global_load_lds_dwordx4: no VGPR staging, no ds_write): stage s+1 is in flight
+// while stage s is consumed.  (A ring of four 64-byte-row stages with three in flight was
+// measured too: same loop time, because every 128-byte line then travels from L2 twice.)
+// 16-byte chunks are XOR-swizzled with the row index so that the per-lane 16-byte operand reads
+// spread over all 64 banks.
 // Workgroup ids are remapped so that each XCD (ids congruent mod 8 share an L2) walks a compact
 // block of tiles.
 
