@@ -26,6 +26,15 @@ sys.path.insert(0, os.path.join(ROOT, "glades-ml_amd"))
 PEAKS = {"bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}  # dense MFMA, TFLOP/s
 HBM_PEAK = 8000.0  # GB/s
 
+# HBM bytes per launch of a workload's dominant kernel, from two `rocprofv3 --pmc` runs of this
+# script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch averaged over the kernel's launches), each
+# scaled by what the same counter reads for the 1 GiB copy of `--workload copy`
+# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); profiles/gemm_bf16_cfg4_pmc.md has the runs.
+# A workload / kernel pair that was not measured reports null.
+MEASURED_TRAFFIC_BYTES = {
+    ("cfg4", "gemm_bf16_wgrad_sgd"): int((233040.23 * 2.000 + 167116.8 * 1.000) * 1024),
+}
+
 WORKLOADS = {
     "cfg4": dict(desc="bf16 train MLP 4096-4096-4096-4096-4096-1024 ReLU softmax-CE, batch 8192, SGD momentum 0.9, fp32 master",
                  sizes=[4096, 4096, 4096, 4096, 4096, 1024], batch=8192, rows=262144, dtype="bf16", kind="train"),
@@ -146,7 +155,8 @@ def run_canonical(w, args):
     ach = fl_launch / (kern[dom]["avg_ms"] * 1e-3) / 1e12
     peak = PEAKS[w["dtype"]]
     roof = dict(bound="mfma", kernel=dom, achieved=round(ach, 2), peak=peak, unit="TFLOP/s", frac=round(ach / peak, 4),
-                traffic=None, flop_per_launch=fl_launch, avg_launch_ms=round(kern[dom]["avg_ms"], 4))
+                traffic=MEASURED_TRAFFIC_BYTES.get((w["name"], dom)), flop_per_launch=fl_launch,
+                avg_launch_ms=round(kern[dom]["avg_ms"], 4))
     total_ms = sum(k["total_ms"] for k in kern.values())
     breakdown = {n: round(k["total_ms"] / psteps, 4) for n, k in sorted(kern.items(), key=lambda kv: -kv[1]["total_ms"])}
     value = args.steps * B / el
@@ -256,12 +266,27 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS) + ["copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "copy":
+        # calibration target for the FETCH_SIZE / WRITE_SIZE counters: a plain device-to-device copy
+        # of a known size (1 GiB read + 1 GiB written per launch)
+        import torch
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps or 10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        print(json.dumps({"workload": "copy", "bytes_read_per_launch": src.numel() * 4, "bytes_written_per_launch": src.numel() * 4,
+                          "launches": args.steps or 10, "GBps": 2 * src.numel() * 4 * (args.steps or 10) / el / 1e9}))
+        return
     w = dict(WORKLOADS[args.workload], name=args.workload)
     if args.steps is None:
         args.steps = {"cfg4": 40, "cfg5": 40, "cfg3": 200, "cfg2": 5, "cfg1": 200}[args.workload]
