@@ -11,14 +11,16 @@
 //             fused with the SGD + momentum + L1/L2 update of the fp32 master weights, which
 //             also writes the bf16 W and W^T used by the next step.
 //
-// Tile: 256 x 256 outputs per workgroup of 8 wavefronts laid out 2 (M) x 4 (N); each wavefront owns
-// 128 x 64 = 4 x 2 accumulators of 32x32 (128 VGPRs).  K advances in stages of 128 bytes per row
-// (64 bf16 / 128 e4m3: whole cache lines).  LDS holds two stages (2 x 64 KiB) filled by LDS-direct
-// global loads (global_load_lds_dwordx4: no VGPR staging, no ds_write): stage s+1 is in flight
-// while stage s is consumed.  (A ring of four 64-byte-row stages with three in flight was
-// measured too: same loop time, because every 128-byte line then travels from L2 twice.)
-// 16-byte chunks are XOR-swizzled with the row index so that the per-lane 16-byte operand reads
-// spread over all 64 banks.
+// Tile: a workgroup of 8 wavefronts laid out 2 (M) x 4 (N); each wavefront owns MI x NI
+// accumulators of 32x32.  MI = 4, NI = 2 gives the 256 x 256 tile (128 x 64 per wavefront, 128
+// accumulator VGPRs) used whenever it fills the 256 CUs; MI = 2, NI = 1 gives a 128 x 128 tile for
+// the products that would otherwise leave most CUs idle (the 1024-wide output layer).
+// K advances in stages of 128 bytes per row (64 bf16 / 128 e4m3: whole cache lines).  LDS holds
+// two stages filled by LDS-direct global loads (global_load_lds_dwordx4: no VGPR staging, no
+// ds_write): stage s+1 is in flight while stage s is consumed.  (A ring of four 64-byte-row stages
+// with three in flight was measured too: same loop time, because every 128-byte line then travels
+// from L2 twice.)  16-byte chunks are XOR-swizzled with the row index so that the per-lane
+// 16-byte operand reads spread over all 64 banks.
 // Workgroup ids are remapped so that each XCD (ids congruent mod 8 share an L2) walks a compact
 // block of tiles.
 
@@ -31,11 +33,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 
-constexpr int TM = 256, TN = 256, NT = 512;
-constexpr int SKB = 128;                 // bytes of K per stage row (64 bf16 / 128 e4m3): one full cache line
-constexpr int STAGE_BYTES = 256 * SKB;   // one operand stage
-constexpr int EPI_PITCH = 528;           // bytes per staged output row: 512 + 16 (keeps 16-byte alignment, rotates banks)
-constexpr int EPI_LDS_BYTES = 256 * EPI_PITCH;  // 132 KiB >= 8 stages
+constexpr int NT = 512;
+constexpr int SKB = 128;  // bytes of K per stage row (64 bf16 / 128 e4m3): one full cache line
 
 // LDS has 64 banks of 4 bytes: a 16-byte-per-lane read is served 16 lanes per clock.  A stage
 // row is 128 B = 32 banks, so row parity picks the bank half and (row >> 1) & 7 rotates the
@@ -43,7 +42,7 @@ constexpr int EPI_LDS_BYTES = 256 * EPI_PITCH;  // 132 KiB >= 8 stages
 __device__ __forceinline__ int swz(int row, int chunk) { return (row << 7) + (((chunk ^ (row >> 1)) & 7) << 4); }
 
 // Activation and its derivative in a branch-free parametric form (filled on the host by
-// resolve_act): the epilogues apply them to 128 accumulators per lane, and a switch over the
+// resolve_act): the epilogues apply them to up to 128 accumulators per lane, and a switch over the
 // activation id replicated that often does not fit the instruction cache.
 __device__ __forceinline__ float lp_squash(float z, const GemmLpArgs::ActForm& a)
 {
@@ -60,44 +59,37 @@ __device__ __forceinline__ float lp_act_der(float y, const GemmLpArgs::ActForm& 
     return a.step ? stp : poly;
 }
 
-// Operand fragments of one K sub-step for this wavefront: 4 row blocks of A, 2 of B.
+// Operand fragments of one K sub-step for this wavefront: MI row blocks of A, NI of B.
 // bf16: 16 bytes per lane per block (K = 16); e4m3: 32 bytes per lane per block (K = 64).
-template <bool FP8> struct Frags { v4i a[4], b[2]; };
-template <> struct Frags<true> { v4i a[4][2], b[2][2]; };
+template <bool FP8, int MI, int NI> struct Frags { v4i a[MI][FP8 ? 2 : 1], b[NI][FP8 ? 2 : 1]; };
 
-template <bool FP8>
-__device__ __forceinline__ void load_frags(Frags<FP8>& f, const unsigned char* sa, const unsigned char* sb,
+template <bool FP8, int MI, int NI>
+__device__ __forceinline__ void load_frags(Frags<FP8, MI, NI>& f, const unsigned char* sa, const unsigned char* sb,
                                            int ks, int wm, int wn, int l31, int lh)
 {
-    if constexpr (!FP8) {
+    constexpr int H = FP8 ? 2 : 1;
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi) f.a[mi] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, ks * 2 + lh));
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) f.b[ni] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, ks * 2 + lh));
-    } else {
+        for (int h = 0; h < H; ++h)
+            f.a[mi][h] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, (ks * 2 + lh) * H + h));
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+    for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-                f.a[mi][h] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, ks * 4 + lh * 2 + h));
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-            for (int h = 0; h < 2; ++h)
-                f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, ks * 4 + lh * 2 + h));
-    }
+        for (int h = 0; h < H; ++h)
+            f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, (ks * 2 + lh) * H + h));
 }
 
-template <bool FP8>
-__device__ __forceinline__ void mma_frags(v16f (&acc)[4][2], const Frags<FP8>& f)
+template <bool FP8, int MI, int NI>
+__device__ __forceinline__ void mma_frags(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f)
 {
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
+        for (int ni = 0; ni < NI; ++ni) {
             if constexpr (!FP8) {
-                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi]),
-                                                                      __builtin_bit_cast(bf16x8, f.b[ni]), acc[mi][ni], 0, 0, 0);
+                acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, f.a[mi][0]),
+                                                                      __builtin_bit_cast(bf16x8, f.b[ni][0]), acc[mi][ni], 0, 0, 0);
             } else {
                 const v8i av = v8i{f.a[mi][0][0], f.a[mi][0][1], f.a[mi][0][2], f.a[mi][0][3],
                                    f.a[mi][1][0], f.a[mi][1][1], f.a[mi][1][2], f.a[mi][1][3]};
@@ -110,42 +102,51 @@ __device__ __forceinline__ void mma_frags(v16f (&acc)[4][2], const Frags<FP8>& f
 
 typedef __attribute__((address_space(3))) unsigned char* lptr_t;
 
-// One operand stage (256 rows x 128 B) is 32 slabs of 8 rows = 1 KiB; a wavefront moves 4 slabs
-// with 4 LDS-direct loads: lane i of a load lands at slab + 16*i, i.e. row i/8, physical chunk
-// i%8, so the lane fetches the logical chunk that the swizzle maps there.  Every load covers
-// whole 128-byte lines (with 64-byte stage rows each line was fetched from L2 twice).
-// The load is issued from inline assembly on purpose: the compiler then keeps no book on it, and
-// the only waits on these loads are the explicit s_waitcnt vmcnt(N) before each barrier (with the
-// builtin it drains all of them, vmcnt(0), in front of LDS reads it cannot tell apart from the
-// stage being filled).  M0 carries the LDS byte address of the slab; loads return in order.
+// LDS-direct load of one 1 KiB slab: lane i's 16 bytes land at lds_slab + 16*i.
+// Issued from inline assembly on purpose: the compiler then keeps no book on it, and the only
+// waits on these loads are the explicit s_waitcnt vmcnt(N) before the barriers (with the builtin
+// it drains all of them, vmcnt(0), in front of LDS reads it cannot tell apart from the stage
+// being filled).  M0 carries the LDS byte address of the slab; loads return in order.
+__device__ __forceinline__ void lds_direct_16(const unsigned char* src, unsigned int lds_slab)
+{
+    const unsigned int dst_u = __builtin_amdgcn_readfirstlane(lds_slab);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst_u) : "memory", "m0");
+}
+
+// One operand stage (ROWS rows x 128 B) is ROWS/8 slabs of 8 rows = 1 KiB; a wavefront moves
+// ROWS/64 slabs: lane i of a load lands at row i/8, physical chunk i%8 of its slab, so the lane
+// fetches the logical chunk that the swizzle maps there.  Every load covers whole 128-byte lines.
+template <int ROWS>
 __device__ __forceinline__ void dma_stage(unsigned char* sdst, const unsigned char* gsrc, long long ldk,
                                           long long kb, int w, int lane)
 {
+    constexpr int PER_WAVE = ROWS / 64;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int slab = w * 4 + j;
+    for (int j = 0; j < PER_WAVE; ++j) {
+        const int slab = w * PER_WAVE + j;
         const int row = slab * 8 + (lane >> 3);
         const int chunk = ((lane & 7) ^ (row >> 1)) & 7;
-        const unsigned char* src = gsrc + (long long)row * ldk + kb + (chunk << 4);
-        const unsigned int dst = (unsigned int)(uintptr_t)((lptr_t)sdst) + slab * 1024;
-        const unsigned int dst_u = __builtin_amdgcn_readfirstlane(dst);
-        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                     :
-                     : "v"(src), "s"(dst_u)
-                     : "memory", "m0");
+        lds_direct_16(gsrc + (long long)row * ldk + kb + (chunk << 4), (unsigned int)(uintptr_t)((lptr_t)sdst) + slab * 1024);
     }
 }
 
-template <bool FP8, int EPI>
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+
+template <bool FP8, int EPI, int MI, int NI>
 __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 {
-    // One LDS block: two stages (A then B, 256 rows x 128 B of K each) during the K loop,
-    // then the staging area of the epilogue (256 x 256 bf16 with padded rows).
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[EPI_LDS_BYTES];
+    constexpr int TM = 64 * MI, TN = 128 * NI;       // tile
+    constexpr int WM = 32 * MI, WN = 32 * NI;        // per wavefront
+    constexpr int A_BYTES = TM * SKB, B_BYTES = TN * SKB;
+    constexpr int PITCH = 2 * TN + 16;               // staged bf16 output row [TM][TN]: +16 rotates banks, keeps alignment
+    constexpr int PITCH_T = 2 * TM + 16;             // staged transposed row [TN][TM]
+    constexpr int LDS_BYTES = cmax(2 * (A_BYTES + B_BYTES), cmax(TM * PITCH, TN * PITCH_T));
+    // One LDS block: two stages (A then B) during the K loop, then the staging area of the epilogue.
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
     unsigned char* const sA0 = smem;
-    unsigned char* const sB0 = smem + 1 * STAGE_BYTES;
-    unsigned char* const sA1 = smem + 2 * STAGE_BYTES;
-    unsigned char* const sB1 = smem + 3 * STAGE_BYTES;
+    unsigned char* const sB0 = sA0 + A_BYTES;
+    unsigned char* const sA1 = sB0 + B_BYTES;
+    unsigned char* const sB1 = sA1 + A_BYTES;
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6;
     const int l31 = lane & 31, lh = lane >> 5;
@@ -169,13 +170,13 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     const unsigned char* gA = (const unsigned char*)g.A + (long long)bm * ldk;
     const unsigned char* gB = (const unsigned char*)g.B + (long long)bn * ldk;
 
-    const int wm = (w >> 2) * 128, wn = (w & 3) * 64;
+    const int wm = (w >> 2) * WM, wn = (w & 3) * WN;
 
-    v16f acc[4][2];
+    v16f acc[MI][NI];
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi)
+    for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni)
+        for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
 
@@ -183,48 +184,51 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 
     auto fill = [&](unsigned char* WA, unsigned char* WB, int st) {
         const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;  // past the end: refetch, never read
-        dma_stage(WA, gA, ldk, kb, w, lane);
-        dma_stage(WB, gB, ldk, kb, w, lane);
+        dma_stage<TM>(WA, gA, ldk, kb, w, lane);
+        dma_stage<TN>(WB, gB, ldk, kb, w, lane);
     };
     fill(sA0, sB0, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
     __builtin_amdgcn_s_barrier();
 
-    Frags<FP8> f0, f1;
-    load_frags<FP8>(f0, sA0, sB0, 0, wm, wn, l31, lh);
+    typedef Frags<FP8, MI, NI> F;
+    F f0, f1;
+    load_frags<FP8, MI, NI>(f0, sA0, sB0, 0, wm, wn, l31, lh);
 
     // One stage: reads (RA, RB) = stage s while (WA, WB) is filled with stage s+1 (the buffer of
     // stage s-1, free since the barrier that ended it).  Sub-steps are software pipelined: each
     // one first states that its own fragments (requested one MFMA group earlier) have landed, then
     // requests the next sub-step's fragments, then issues its MFMAs.  The last sub-step waits for
     // the fill, meets the other wavefronts (bare s_barrier: the explicit counts are exactly what
-    // has to be visible) and requests the first fragments of stage s+1.
+    // has to be visible) and requests the first fragments of stage s+1.  The 256 x 256 e4m3 tile
+    // has no registers left for a second fragment set and runs its two sub-steps in sequence.
     constexpr int KS = FP8 ? 2 : 4;
+    constexpr bool kDouble = !(FP8 && MI * NI > 2);
     auto stage = [&](int s, const unsigned char* RA, const unsigned char* RB, unsigned char* WA, unsigned char* WB) {
-        if constexpr (FP8) {
+        if constexpr (!kDouble) {
             fill(WA, WB, s + 1);
-            mma_frags<FP8>(acc, f0);
-            load_frags<FP8>(f0, RA, RB, 1, wm, wn, l31, lh);
-            mma_frags<FP8>(acc, f0);
+            mma_frags<FP8, MI, NI>(acc, f0);
+            load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
+            mma_frags<FP8, MI, NI>(acc, f0);
             __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
-            load_frags<FP8>(f0, WA, WB, 0, wm, wn, l31, lh);
+            load_frags<FP8, MI, NI>(f0, WA, WB, 0, wm, wn, l31, lh);
         } else {
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
-                Frags<FP8>& cur = (ks & 1) ? f1 : f0;
-                Frags<FP8>& nxt = (ks & 1) ? f0 : f1;
+                F& cur = (ks & 1) ? f1 : f0;
+                F& nxt = (ks & 1) ? f0 : f1;
                 if (ks + 1 < KS) {
                     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): cur has landed
-                    load_frags<FP8>(nxt, RA, RB, ks + 1, wm, wn, l31, lh);
+                    load_frags<FP8, MI, NI>(nxt, RA, RB, ks + 1, wm, wn, l31, lh);
                     if (ks == 0) fill(WA, WB, s + 1);
                 } else {
                     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
                     __builtin_amdgcn_s_barrier();
-                    load_frags<FP8>(nxt, WA, WB, 0, wm, wn, l31, lh);
+                    load_frags<FP8, MI, NI>(nxt, WA, WB, 0, wm, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                mma_frags<FP8>(acc, cur);
+                mma_frags<FP8, MI, NI>(acc, cur);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -238,34 +242,35 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 
     // ---- epilogue.  Accumulator layout of a 32x32 tile: lane -> column lane%32,
     //      register i -> row 8*(i/4) + 4*(lane/32) + i%4  (4 consecutive rows per register quad).
-    //      bf16 results leave through LDS so that global memory only sees 16-byte-per-lane,
-    //      512-byte-per-row stores (direct stores from this layout are 2 bytes per lane, and 8
-    //      bytes per lane with a row-sized stride for the transposed copy).
+    //      bf16 results leave through LDS so that global memory only sees 16-byte-per-lane stores
+    //      of whole tile rows (direct stores from this layout are 2 bytes per lane, and 8 bytes per
+    //      lane with a row-sized stride for the transposed copy).
     const int M = g.M, N = g.N;
     __builtin_amdgcn_s_barrier();  // every wavefront is done with the ring
 
     if constexpr (EPI == LP_DGRAD) {
-        // activation tile [256][256] bf16 -> LDS (row pitch 512 B) with LDS-direct loads
+        // activation tile [TM][TN] bf16 -> LDS (row pitch 2*TN bytes) with LDS-direct loads
+        constexpr int LPR = TN / 8;         // lanes per tile row (16 bytes each)
+        constexpr int RPS = 64 / LPR;       // rows per 1 KiB slab
+        constexpr int PER_WAVE = TM / RPS / 8;
         const unsigned char* aux = (const unsigned char*)g.aux + ((long long)bm * N + bn) * 2;
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-            const int slab = w * 16 + j;  // 2 rows per slab
-            const int row = slab * 2 + (lane >> 5);
-            const unsigned char* src = aux + (long long)row * N * 2 + ((lane & 31) << 4);
-            const unsigned int dst = __builtin_amdgcn_readfirstlane((unsigned int)(uintptr_t)((lptr_t)smem) + slab * 1024);
-            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+        for (int j = 0; j < PER_WAVE; ++j) {
+            const int slab = w * PER_WAVE + j;
+            const int row = slab * RPS + lane / LPR;
+            lds_direct_16(aux + (long long)row * N * 2 + ((lane % LPR) << 4), (unsigned int)(uintptr_t)((lptr_t)smem) + slab * 1024);
         }
         __builtin_amdgcn_s_waitcnt(0x0070);
         __builtin_amdgcn_s_barrier();
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+        for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+            for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int row = wm + mi * 32 + 8 * (i >> 2) + 4 * lh + (i & 3);
                     const int col = wn + ni * 32 + l31;
-                    const uint16_t hv = *reinterpret_cast<const uint16_t*>(smem + row * 512 + col * 2);
+                    const uint16_t hv = *reinterpret_cast<const uint16_t*>(smem + row * (2 * TN) + col * 2);
                     acc[mi][ni][i] *= lp_act_der(ghip_bf16_to_f32(hv), g.ap);
                 }
         __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -273,11 +278,11 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     }
 
     constexpr bool kBf16Out = (EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT);
-    uint2 pk[4][2][4];  // bf16 results, 4 consecutive rows packed per entry
+    uint2 pk[MI][NI][4];  // bf16 results, 4 consecutive rows packed per entry
 #pragma unroll
-    for (int mi = 0; mi < 4; ++mi) {
+    for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
+        for (int ni = 0; ni < NI; ++ni) {
             const int col = bn + wn + ni * 32 + l31;
             float cbias = 0.0f, cscale = 1.0f;
             if (EPI == LP_FWD_ACT || EPI == LP_FWD_F32) cbias = g.bias ? g.bias[col] : 0.0f;
@@ -324,25 +329,26 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         }
     }
     if constexpr (kBf16Out) {
-        const int lr2 = lane >> 5, lc = (lane & 31) << 4;
         // transposed copy first: LDS_T[n][m], a lane's 4 consecutive rows are 8 contiguous bytes
         if ((EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD) && g.outT) {
 #pragma unroll
-            for (int mi = 0; mi < 4; ++mi)
+            for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
+                for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int rl = wm + mi * 32 + 8 * q + 4 * lh, cl = wn + ni * 32 + l31;
-                        *reinterpret_cast<uint2*>(smem + cl * EPI_PITCH + rl * 2) = pk[mi][ni][q];
+                        *reinterpret_cast<uint2*>(smem + cl * PITCH_T + rl * 2) = pk[mi][ni][q];
                     }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_s_barrier();
+            constexpr int LPR = TM / 8, RPI = 64 / LPR;   // lanes per transposed row, rows per instruction
             unsigned char* dstT = (unsigned char*)g.outT + ((long long)bn * M + bm) * 2;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int nl = w * 32 + i * 2 + lr2;
-                const v4i val = *reinterpret_cast<const v4i*>(smem + nl * EPI_PITCH + lc);
+            for (int i = 0; i < (TN / 8) / RPI; ++i) {
+                const int nl = w * (TN / 8) + i * RPI + lane / LPR;
+                const int lc = (lane % LPR) << 4;
+                const v4i val = *reinterpret_cast<const v4i*>(smem + nl * PITCH_T + lc);
                 *reinterpret_cast<v4i*>(dstT + (long long)nl * M * 2 + lc) = val;
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -350,41 +356,50 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         }
         // row-major copy: LDS[m][n]
 #pragma unroll
-        for (int mi = 0; mi < 4; ++mi)
+        for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+            for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int rl = wm + mi * 32 + 8 * q + 4 * lh, cl = wn + ni * 32 + l31;
-                    unsigned char* d0 = smem + rl * EPI_PITCH + cl * 2;
+                    unsigned char* d0 = smem + rl * PITCH + cl * 2;
                     *reinterpret_cast<uint16_t*>(d0) = (uint16_t)(pk[mi][ni][q].x & 0xffffu);
-                    *reinterpret_cast<uint16_t*>(d0 + EPI_PITCH) = (uint16_t)(pk[mi][ni][q].x >> 16);
-                    *reinterpret_cast<uint16_t*>(d0 + 2 * EPI_PITCH) = (uint16_t)(pk[mi][ni][q].y & 0xffffu);
-                    *reinterpret_cast<uint16_t*>(d0 + 3 * EPI_PITCH) = (uint16_t)(pk[mi][ni][q].y >> 16);
+                    *reinterpret_cast<uint16_t*>(d0 + PITCH) = (uint16_t)(pk[mi][ni][q].x >> 16);
+                    *reinterpret_cast<uint16_t*>(d0 + 2 * PITCH) = (uint16_t)(pk[mi][ni][q].y & 0xffffu);
+                    *reinterpret_cast<uint16_t*>(d0 + 3 * PITCH) = (uint16_t)(pk[mi][ni][q].y >> 16);
                 }
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_s_barrier();
+        constexpr int LPR = TN / 8, RPI = 64 / LPR;
         unsigned char* dst = (unsigned char*)g.out + ((long long)bm * N + bn) * 2;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            const int ml = w * 32 + i * 2 + lr2;
-            const v4i val = *reinterpret_cast<const v4i*>(smem + ml * EPI_PITCH + lc);
+        for (int i = 0; i < (TM / 8) / RPI; ++i) {
+            const int ml = w * (TM / 8) + i * RPI + lane / LPR;
+            const int lc = (lane % LPR) << 4;
+            const v4i val = *reinterpret_cast<const v4i*>(smem + ml * PITCH + lc);
             *reinterpret_cast<v4i*>(dst + (long long)ml * N * 2 + lc) = val;
         }
     }
 }
 
+// 256 x 256 tiles when they give every CU at least one workgroup, else 128 x 128.
+constexpr int kCUs = 256;
+inline bool use_small_tile(int M, int N) { return (long long)(M / 256) * (N / 256) < kCUs; }
+
 template <bool FP8, int EPI>
 hipError_t launch(const GemmLpArgs& a, hipStream_t s)
 {
-    const int nb = (a.M / TM) * (a.N / TN);
-    hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI>), dim3(nb), dim3(NT), 0, s, a);
+    if (use_small_tile(a.M, a.N)) {
+        const int nb = (a.M / 128) * (a.N / 128);
+        hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI, 2, 1>), dim3(nb), dim3(NT), 0, s, a);
+    } else {
+        const int nb = (a.M / 256) * (a.N / 256);
+        hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI, 4, 2>), dim3(nb), dim3(NT), 0, s, a);
+    }
     return hipGetLastError();
 }
 
-}  // namespace
-
-static void resolve_act(GemmLpArgs& g)
+void resolve_act(GemmLpArgs& g)
 {
     GemmLpArgs::ActForm& a = g.ap;
     const float inf = __builtin_huge_valf(), p = g.act_param;
@@ -404,10 +419,12 @@ static void resolve_act(GemmLpArgs& g)
     }
 }
 
+}  // namespace
+
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8)
 {
     const int kq = fp8 ? 256 : 128;  // two stages of 128 bytes of K per pass of the main loop
-    return M > 0 && N > 0 && K > 0 && (M % TM) == 0 && (N % TN) == 0 && (K % kq) == 0;
+    return M > 0 && N > 0 && K > 0 && (M % 256) == 0 && (N % 256) == 0 && (K % kq) == 0;
 }
 
 hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)

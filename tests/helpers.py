@@ -40,12 +40,13 @@ def rel_err(a, b):
     return float(np.max(np.abs(a - b) / (np.abs(b) + 1e-6))) if a.size else 0.0
 
 
-def bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, steps, lr, mom, wd2):
+def bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, steps, lr, mom, wd2, wide=True):
     """numpy statement of the bf16 training pipeline: bf16 weights (rounded from the fp32 master),
     bf16 activations and deltas, products exact and summed in float64, fp32 logits/softmax,
     fp32 master + momentum update.  Hidden activations: TANH / RELU (0.046 knee) / SIGMOID;
     output: SOFTMAX with cross-entropy.  Returns final master weights, biases and losses."""
     q = po.bf16_round
+    mm = np.float64 if wide else np.float32   # accumulation type of the matrix products
     Wm = [w.astype(np.float32).copy() for w in Ws]
     bm = [b.astype(np.float32).copy() for b in bs]
     vW = [np.zeros_like(w) for w in Wm]
@@ -57,7 +58,7 @@ def bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, steps, lr, mom, wd2):
         Wh = [q(w) for w in Wm]
         H = [q(x)]
         for l in range(L):
-            Z = (H[l].astype(np.float64) @ Wh[l].T.astype(np.float64)).astype(np.float32) + bm[l]
+            Z = (H[l].astype(mm) @ Wh[l].T.astype(mm)).astype(np.float32) + bm[l]
             if l == L - 1:
                 break
             if acts[l] == po.TANH:
@@ -72,10 +73,10 @@ def bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, steps, lr, mom, wd2):
         losses.append(float(-(y * np.log(np.maximum(P, 1e-30))).sum(1).mean()))
         D = q(P - y)
         for l in range(L - 1, -1, -1):
-            g = (D.T.astype(np.float64) @ H[l].astype(np.float64) / B).astype(np.float32)
+            g = (D.T.astype(mm) @ H[l].astype(mm) / B).astype(np.float32)
             gb = D.astype(np.float64).mean(0).astype(np.float32)
             if l > 0:
-                Eb = (D.astype(np.float64) @ Wh[l].astype(np.float64)).astype(np.float32)
+                Eb = (D.astype(mm) @ Wh[l].astype(mm)).astype(np.float32)
                 h = H[l]
                 der = (1 - h * h) if acts[l - 1] == po.TANH else ((h > 0).astype(np.float32) if acts[l - 1] == po.RELU else h * (1 - h))
                 D = q(Eb * der)

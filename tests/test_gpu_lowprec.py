@@ -130,3 +130,34 @@ def test_lowprec_shape_rules():
     with pytest.raises(pg.GladesHipError):   # not quantised yet
         g.forward(np.zeros((256, 256), np.float32))
     g.close()
+
+
+def test_bf16_step_at_full_tile_size():
+    """Layers of 4096 with a batch of 4096 give 256 tiles of 256 x 256 per product, which is where
+    the library switches from its 128 x 128 to its 256 x 256 tile (every smaller case above runs
+    the small one).  One training step against the numpy statement of the bf16 pipeline (float32
+    matmuls here: 137 GFLOP each): loss 1e-3, update within 1e-2 of its Frobenius norm."""
+    import pyglades as pg
+    from helpers import bf16_pipeline_steps
+    print("bf16 full-size tile", flush=True)
+    rng = np.random.default_rng(11)
+    sizes, acts = [4096, 4096, 4096], [po.RELU, po.SOFTMAX]
+    B = 4096
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l]))) for l in range(2)]
+    bs = [np.zeros(sizes[l + 1], np.float32) for l in range(2)]
+    X = rng.standard_normal((B, 4096), dtype=np.float32)
+    Y = np.eye(4096, dtype=np.float32)[rng.integers(0, 4096, B)]
+    lr = 0.5
+    g = pg.Net(pg.make_spec(sizes, acts, lr=lr, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=pg.BF16))
+    for l in range(2):
+        g.set_params(l, Ws[l], bs[l])
+    g.set_dataset(X, Y)
+    loss = g.train_step(0, B).loss
+    Wm, bm, ref_losses = bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, 1, lr, 0.0, 0.0, wide=False)
+    assert abs(loss - ref_losses[0]) <= 1e-3 * abs(ref_losses[0]), (loss, ref_losses)
+    for l in range(2):
+        Wg, bg = g.get_params(l)
+        fro = np.linalg.norm(Wg - Wm[l]) / np.linalg.norm(Wm[l] - Ws[l])
+        print("layer", l, "update error vs pipeline statement", fro, flush=True)
+        assert fro <= 1e-2, (l, fro)
+    g.close()
