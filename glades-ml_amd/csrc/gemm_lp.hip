@@ -44,9 +44,11 @@ __device__ __forceinline__ int swz(int row, int chunk) { return (row << 7) + (((
 // Activation and its derivative in a branch-free parametric form (filled on the host by
 // resolve_act): the epilogues apply them to up to 128 accumulators per lane, and a switch over the
 // activation id replicated that often does not fit the instruction cache.
+template <bool PLAIN>
 __device__ __forceinline__ float lp_squash(float z, const GemmLpArgs::ActForm& a)
 {
     float v = (z < a.thr) ? a.a0 * z + a.b0 : a.a1 * z + a.b1;
+    if (PLAIN) return v;
     if (a.trans) v = a.ta * __frcp_rn(1.0f + __expf(-a.tk * z)) + a.tb;
     v = (z < a.clo) ? a.vlo : v;
     v = (z > a.chi) ? a.vhi : v;
@@ -80,8 +82,35 @@ __device__ __forceinline__ void load_frags(Frags<FP8, MI, NI>& f, const unsigned
             f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, (ks * 2 + lh) * H + h));
 }
 
-template <bool FP8, int MI, int NI>
-__device__ __forceinline__ void mma_frags(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f)
+typedef __attribute__((address_space(3))) unsigned char* lptr_t;
+
+// LDS-direct load of one 1 KiB slab: lane i's 16 bytes land at lds_slab + 16*i.
+// Issued from inline assembly on purpose: the compiler then keeps no book on it, and the only
+// waits on these loads are the explicit s_waitcnt vmcnt(N) before the barriers (with the builtin
+// it drains all of them, vmcnt(0), in front of LDS reads it cannot tell apart from the stage
+// being filled).  M0 carries the LDS byte address of the slab; loads return in order.
+__device__ __forceinline__ void lds_direct_16(const unsigned char* src, unsigned int lds_slab)
+{
+    const unsigned int dst_u = __builtin_amdgcn_readfirstlane(lds_slab);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst_u) : "memory", "m0");
+}
+// The same with a wavefront-uniform base address and a 32-bit per-lane byte offset: the main loop
+// advances the base with scalar arithmetic and keeps one offset register per operand and slab parity.
+__device__ __forceinline__ void lds_direct_16s(const unsigned char* sbase, unsigned int voff, unsigned int lds_slab)
+{
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_slab) : "memory", "m0");
+}
+
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
+template <int V> struct IC { static constexpr int value = V; };
+
+// MFMAs of one K sub-step with the LDS-direct loads of the running fill spread between them:
+// `before` MFMAs of the fill's span have been issued before this group; after MFMA number m of
+// the span, loads number ceil(m * NDMA / SPAN) .. ceil((m + 1) * NDMA / SPAN) - 1 go out.  A
+// wavefront that issues its loads back to back stalls on the address unit (16 clocks per load,
+// shared by the 8 wavefronts), and the matrix pipe of its SIMD idles with it.
+template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, typename Dma>
+__device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma)
 {
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -97,40 +126,18 @@ __device__ __forceinline__ void mma_frags(v16f (&acc)[MI][NI], const Frags<FP8, 
                                    f.b[ni][1][0], f.b[ni][1][1], f.b[ni][1][2], f.b[ni][1][3]};
                 acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
             }
+            if constexpr (NDMA > 0) {
+                const int m = BEFORE + mi * NI + ni;
+                const int lo = (m * NDMA + SPAN - 1) / SPAN, hi = ((m + 1) * NDMA + SPAN - 1) / SPAN;
+                if (m < SPAN && hi > lo) {
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int d = lo; d < hi; ++d) dma(d);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         }
 }
-
-typedef __attribute__((address_space(3))) unsigned char* lptr_t;
-
-// LDS-direct load of one 1 KiB slab: lane i's 16 bytes land at lds_slab + 16*i.
-// Issued from inline assembly on purpose: the compiler then keeps no book on it, and the only
-// waits on these loads are the explicit s_waitcnt vmcnt(N) before the barriers (with the builtin
-// it drains all of them, vmcnt(0), in front of LDS reads it cannot tell apart from the stage
-// being filled).  M0 carries the LDS byte address of the slab; loads return in order.
-__device__ __forceinline__ void lds_direct_16(const unsigned char* src, unsigned int lds_slab)
-{
-    const unsigned int dst_u = __builtin_amdgcn_readfirstlane(lds_slab);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst_u) : "memory", "m0");
-}
-
-// One operand stage (ROWS rows x 128 B) is ROWS/8 slabs of 8 rows = 1 KiB; a wavefront moves
-// ROWS/64 slabs: lane i of a load lands at row i/8, physical chunk i%8 of its slab, so the lane
-// fetches the logical chunk that the swizzle maps there.  Every load covers whole 128-byte lines.
-template <int ROWS>
-__device__ __forceinline__ void dma_stage(unsigned char* sdst, const unsigned char* gsrc, long long ldk,
-                                          long long kb, int w, int lane)
-{
-    constexpr int PER_WAVE = ROWS / 64;
-#pragma unroll
-    for (int j = 0; j < PER_WAVE; ++j) {
-        const int slab = w * PER_WAVE + j;
-        const int row = slab * 8 + (lane >> 3);
-        const int chunk = ((lane & 7) ^ (row >> 1)) & 7;
-        lds_direct_16(gsrc + (long long)row * ldk + kb + (chunk << 4), (unsigned int)(uintptr_t)((lptr_t)sdst) + slab * 1024);
-    }
-}
-
-constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
 template <bool FP8, int EPI, int MI, int NI>
 __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
@@ -138,15 +145,13 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     constexpr int TM = 64 * MI, TN = 128 * NI;       // tile
     constexpr int WM = 32 * MI, WN = 32 * NI;        // per wavefront
     constexpr int A_BYTES = TM * SKB, B_BYTES = TN * SKB;
+    constexpr int SLOT = cmax(A_BYTES, B_BYTES);     // one operand stage
+    constexpr int NSLOT = 5;
     constexpr int PITCH = 2 * TN + 16;               // staged bf16 output row [TM][TN]: +16 rotates banks, keeps alignment
     constexpr int PITCH_T = 2 * TM + 16;             // staged transposed row [TN][TM]
-    constexpr int LDS_BYTES = cmax(2 * (A_BYTES + B_BYTES), cmax(TM * PITCH, TN * PITCH_T));
-    // One LDS block: two stages (A then B) during the K loop, then the staging area of the epilogue.
+    constexpr int LDS_BYTES = cmax(NSLOT * SLOT, cmax(TM * PITCH, TN * PITCH_T));
+    // One LDS block: a ring of five operand stages during the K loop, then the staging area of the epilogue.
     __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
-    unsigned char* const sA0 = smem;
-    unsigned char* const sB0 = sA0 + A_BYTES;
-    unsigned char* const sA1 = sB0 + B_BYTES;
-    unsigned char* const sB1 = sA1 + A_BYTES;
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6;
     const int l31 = lane & 31, lh = lane >> 5;
@@ -166,9 +171,12 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     const int tn = (id % per_group) / gsize;
     const int bm = tm * TM, bn = tn * TN;
 
-    const long long ldk = FP8 ? (long long)g.K : (long long)g.K * 2;  // row pitch in bytes
-    const unsigned char* gA = (const unsigned char*)g.A + (long long)bm * ldk;
-    const unsigned char* gB = (const unsigned char*)g.B + (long long)bn * ldk;
+    constexpr int ES = FP8 ? 1 : 2;                                   // bytes per operand element
+    const long long ldk = (long long)g.K * ES;                        // bytes of K per row
+    const long long lda = (long long)(g.lda ? g.lda : g.K) * ES;      // row pitches in bytes
+    const long long ldb = (long long)(g.ldb ? g.ldb : g.K) * ES;
+    const unsigned char* gA = (const unsigned char*)g.A + (long long)bm * lda;
+    const unsigned char* gB = (const unsigned char*)g.B + (long long)bn * ldb;
 
     const int wm = (w >> 2) * WM, wn = (w & 3) * WN;
 
@@ -180,40 +188,80 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[mi][ni][i] = 0.0f;
 
-    const int nk = (int)(ldk / SKB);  // stages along K (even, see ghip_gemm_lp_shape_ok)
+    const int nk = (int)(ldk / SKB);  // stages along K
 
-    auto fill = [&](unsigned char* WA, unsigned char* WB, int st) {
+    // ---- operand stages.  Stage j of A is TM rows x 128 B, of B TN rows x 128 B; both are
+    // sequences of 1 KiB slabs of 8 rows, one LDS-direct load each: lane i lands at row i/8,
+    // physical chunk i%8 of its slab, so it fetches the logical chunk that the swizzle maps there
+    // (every load covers whole 128-byte lines).  A wavefront moves PWA + PWB slabs per stage.
+    // The ring holds the half-stages A0 B0 A1 B1 ... in slots 0 1 2 3 4 0 1 ...: while stage j is
+    // consumed, B(j+1) and then A(j+2) are requested into the two slots stage j-1 has left, so A
+    // has two stages of lead and B one, and the wait that ends stage j leaves the A loads in flight.
+    constexpr int PWA = TM / 64, PWB = TN / 64, NDMA = PWA + PWB;
+    static_assert(PWA % 2 == 0 && PWB % 2 == 0 && PWA < 8, "slab parity and the vmcnt immediate assume this");
+    const int ws = __builtin_amdgcn_readfirstlane(w);
+    const unsigned int smem_u = (unsigned int)(uintptr_t)((lptr_t)smem);
+    unsigned int voffA[2], voffB[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {  // slab parity decides bit 2 of (row >> 1)
+        const unsigned int chunk = ((lane & 7) ^ (p * 4 + (lane >> 4))) & 7;
+        voffA[p] = (unsigned int)(lane >> 3) * (unsigned int)lda + (chunk << 4);
+        voffB[p] = (unsigned int)(lane >> 3) * (unsigned int)ldb + (chunk << 4);
+    }
+    const unsigned char* const gAw = gA + (long long)(ws * PWA * 8) * lda;
+    const unsigned char* const gBw = gB + (long long)(ws * PWB * 8) * ldb;
+    auto dmaA = [&](int slot, int st, int jj) {
         const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;  // past the end: refetch, never read
-        dma_stage<TM>(WA, gA, ldk, kb, w, lane);
-        dma_stage<TN>(WB, gB, ldk, kb, w, lane);
+        lds_direct_16s(gAw + (long long)(jj * 8) * lda + kb, voffA[jj & 1], smem_u + slot * SLOT + (ws * PWA + jj) * 1024);
     };
-    fill(sA0, sB0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    auto dmaB = [&](int slot, int st, int jj) {
+        const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;
+        lds_direct_16s(gBw + (long long)(jj * 8) * ldb + kb, voffB[jj & 1], smem_u + slot * SLOT + (ws * PWB + jj) * 1024);
+    };
+#pragma unroll
+    for (int jj = 0; jj < PWA; ++jj) dmaA(0, 0, jj);
+#pragma unroll
+    for (int jj = 0; jj < PWB; ++jj) dmaB(1, 0, jj);
+#pragma unroll
+    for (int jj = 0; jj < PWA; ++jj) dmaA(2, 1, jj);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | PWA);  // vmcnt(PWA): A0 and B0 have landed
     __builtin_amdgcn_s_barrier();
 
     typedef Frags<FP8, MI, NI> F;
     F f0, f1;
-    load_frags<FP8, MI, NI>(f0, sA0, sB0, 0, wm, wn, l31, lh);
+    load_frags<FP8, MI, NI>(f0, smem, smem + SLOT, 0, wm, wn, l31, lh);
 
-    // One stage: reads (RA, RB) = stage s while (WA, WB) is filled with stage s+1 (the buffer of
-    // stage s-1, free since the barrier that ended it).  Sub-steps are software pipelined: each
-    // one first states that its own fragments (requested one MFMA group earlier) have landed, then
-    // requests the next sub-step's fragments, then issues its MFMAs.  The last sub-step waits for
-    // the fill, meets the other wavefronts (bare s_barrier: the explicit counts are exactly what
-    // has to be visible) and requests the first fragments of stage s+1.  The 256 x 256 e4m3 tile
-    // has no registers left for a second fragment set and runs its two sub-steps in sequence.
+    // One stage (P = j mod 5 fixes the slots at compile time).  Sub-steps are software pipelined:
+    // each one first states that its own fragments (requested one MFMA group earlier) have landed,
+    // then requests the next sub-step's fragments, then issues its MFMAs with the fill's loads
+    // between them.  The last sub-step waits for B(j+1), meets the other wavefronts (bare
+    // s_barrier: the explicit counts are exactly what has to be visible) and requests the first
+    // fragments of stage j+1.  The 256 x 256 e4m3 tile has no registers left for a second fragment
+    // set and runs its two sub-steps in sequence.
     constexpr int KS = FP8 ? 2 : 4;
-    constexpr bool kDouble = !(FP8 && MI * NI > 2);
-    auto stage = [&](int s, const unsigned char* RA, const unsigned char* RB, unsigned char* WA, unsigned char* WB) {
+    constexpr int G = MI * NI;
+    constexpr bool kDouble = !(FP8 && G > 2);
+    auto stage = [&](auto Pc, int j) {
+        constexpr int P = decltype(Pc)::value;
+        const unsigned char* const RA = smem + ((2 * P) % NSLOT) * SLOT;
+        const unsigned char* const RB = smem + ((2 * P + 1) % NSLOT) * SLOT;
+        const unsigned char* const NA = smem + ((2 * P + 2) % NSLOT) * SLOT;
+        const unsigned char* const NB = smem + ((2 * P + 3) % NSLOT) * SLOT;
+        auto dma = [&](int d) {
+            if (d < PWB) dmaB((2 * P + 3) % NSLOT, j + 1, d);
+            else dmaA((2 * P + 4) % NSLOT, j + 2, d - PWB);
+        };
+        auto none = [](int) {};
         if constexpr (!kDouble) {
-            fill(WA, WB, s + 1);
-            mma_frags<FP8, MI, NI>(acc, f0);
+            constexpr int SPAN = 2 * G;
+            mma_group<FP8, MI, NI, SPAN, NDMA, 0>(acc, f0, dma);
             load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
-            mma_frags<FP8, MI, NI>(acc, f0);
-            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+            mma_group<FP8, MI, NI, SPAN, NDMA, G>(acc, f0, dma);
+            __builtin_amdgcn_s_waitcnt(0x0070 | PWA);  // vmcnt(PWA) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
-            load_frags<FP8, MI, NI>(f0, WA, WB, 0, wm, wn, l31, lh);
+            load_frags<FP8, MI, NI>(f0, NA, NB, 0, wm, wn, l31, lh);
         } else {
+            constexpr int SPAN = (KS - 1) * G;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 F& cur = (ks & 1) ? f1 : f0;
@@ -221,21 +269,26 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                 if (ks + 1 < KS) {
                     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): cur has landed
                     load_frags<FP8, MI, NI>(nxt, RA, RB, ks + 1, wm, wn, l31, lh);
-                    if (ks == 0) fill(WA, WB, s + 1);
                 } else {
-                    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+                    __builtin_amdgcn_s_waitcnt(0x0070 | PWA);  // vmcnt(PWA) lgkmcnt(0)
                     __builtin_amdgcn_s_barrier();
-                    load_frags<FP8, MI, NI>(nxt, WA, WB, 0, wm, wn, l31, lh);
+                    load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                mma_frags<FP8, MI, NI>(acc, cur);
+                if (ks == 0) mma_group<FP8, MI, NI, SPAN, NDMA, 0>(acc, cur, dma);
+                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, NDMA, G>(acc, cur, dma);
+                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, NDMA, 2 * G>(acc, cur, dma);
+                else mma_group<FP8, MI, NI, 1, 0, 0>(acc, cur, none);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
-    for (int s = 0; s < nk; s += 2) {
-        stage(s, sA0, sB0, sA1, sB1);
-        stage(s + 1, sA1, sB1, sA0, sB0);
+    for (int j = 0;;) {
+        stage(IC<0>{}, j); if (++j == nk) break;
+        stage(IC<1>{}, j); if (++j == nk) break;
+        stage(IC<2>{}, j); if (++j == nk) break;
+        stage(IC<3>{}, j); if (++j == nk) break;
+        stage(IC<4>{}, j); if (++j == nk) break;
     }
     // nothing may still be writing this workgroup's LDS when its wavefronts retire
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
@@ -278,56 +331,64 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     }
 
     constexpr bool kBf16Out = (EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT);
+    constexpr bool kFwd = (EPI == LP_FWD_ACT || EPI == LP_FWD_F32), kF8 = (EPI == LP_FP8_ACT || EPI == LP_FP8_F32);
     uint2 pk[MI][NI][4];  // bf16 results, 4 consecutive rows packed per entry
+    float cbias[NI], cscale[NI];
 #pragma unroll
-    for (int mi = 0; mi < MI; ++mi) {
+    for (int ni = 0; ni < NI; ++ni) {
+        const int col = bn + wn + ni * 32 + l31;
+        cbias[ni] = (kFwd && g.bias) ? g.bias[col] : 0.0f;
+        cscale[ni] = kF8 ? g.col_scale[col] : 1.0f;
+    }
+    // Two copies of the element loop, chosen once per launch: piecewise-linear activations
+    // (ReLU, leaky, linear, step) take four instructions per element, the general form a dozen.
+    auto finish = [&](auto plain_c) {
+        constexpr bool PLAIN = decltype(plain_c)::value;
 #pragma unroll
-        for (int ni = 0; ni < NI; ++ni) {
-            const int col = bn + wn + ni * 32 + l31;
-            float cbias = 0.0f, cscale = 1.0f;
-            if (EPI == LP_FWD_ACT || EPI == LP_FWD_F32) cbias = g.bias ? g.bias[col] : 0.0f;
-            if (EPI == LP_FP8_ACT || EPI == LP_FP8_F32) cscale = g.col_scale[col];
+        for (int mi = 0; mi < MI; ++mi) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int row0 = bm + wm + mi * 32 + 8 * q + 4 * lh;
-                uint16_t hb[4] = {0, 0, 0, 0};
+                float rs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+                if constexpr (kF8) {
+                    const float4 r4 = *reinterpret_cast<const float4*>(g.row_scale + row0);
+                    rs[0] = r4.x; rs[1] = r4.y; rs[2] = r4.z; rs[3] = r4.w;
+                }
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int row = row0 + r;
-                    const long long idx = (long long)row * N + col;
-                    float v = acc[mi][ni][q * 4 + r];
-                    if (EPI == LP_FWD_ACT) {
-                        hb[r] = ghip_f32_to_bf16(lp_squash(v + cbias, g.ap));
-                    } else if (EPI == LP_FWD_F32) {
-                        ((float*)g.out)[idx] = lp_squash(v + cbias, g.ap);
-                    } else if (EPI == LP_DGRAD) {
-                        hb[r] = ghip_f32_to_bf16(v);
-                    } else if (EPI == LP_WGRAD_SGD) {
-                        const float wv = g.master[idx];
-                        const float sg = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : 0.0f);
-                        const float gr = v * g.gscale + g.wd1 * sg + g.wd2 * wv;
-                        const float d = g.lr * gr + g.momf * g.mom[idx];
-                        g.mom[idx] = d;
-                        const float nw = wv - d;
-                        g.master[idx] = nw;
-                        hb[r] = ghip_f32_to_bf16(nw);
-                    } else if (EPI == LP_FP8_ACT) {
-                        v = lp_squash(__fmul_rn(v, __fmul_rn(g.row_scale[row], cscale)), g.ap);
-                        hb[r] = ghip_f32_to_bf16(v);
-                        // row amax of the stored (bf16-rounded) values over this wavefront's 32 columns
-                        float am = fabsf(ghip_bf16_to_f32(hb[r]));
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int col = bn + wn + ni * 32 + l31;
+                    float o[4];
 #pragma unroll
-                        for (int o = 16; o > 0; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
-                        if (l31 == 0) atomicMax(&g.row_amax_bits[row], __float_as_uint(am));
-                    } else {  // LP_FP8_F32
-                        ((float*)g.out)[idx] = lp_squash(__fmul_rn(v, __fmul_rn(g.row_scale[row], cscale)), g.ap);
+                    for (int r = 0; r < 4; ++r) {
+                        const long long idx = (long long)(row0 + r) * N + col;
+                        const float v = acc[mi][ni][q * 4 + r];
+                        if constexpr (kFwd) {
+                            o[r] = lp_squash<PLAIN>(v + cbias[ni], g.ap);
+                        } else if constexpr (kF8) {
+                            o[r] = lp_squash<PLAIN>(__fmul_rn(v, __fmul_rn(rs[r], cscale[ni])), g.ap);
+                        } else if constexpr (EPI == LP_WGRAD_SGD) {
+                            const float wv = g.master[idx];
+                            const float sg = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : 0.0f);
+                            const float gr = v * g.gscale + g.wd1 * sg + g.wd2 * wv;
+                            const float d = g.lr * gr + g.momf * g.mom[idx];
+                            g.mom[idx] = d;
+                            o[r] = wv - d;
+                            g.master[idx] = o[r];
+                        } else {
+                            o[r] = v;
+                        }
+                        if constexpr (EPI == LP_FWD_F32 || EPI == LP_FP8_F32) ((float*)g.out)[idx] = o[r];
+                    }
+                    if constexpr (kBf16Out) {
+                        pk[mi][ni][q].x = ghip_f32x2_to_bf16x2(o[0], o[1]);
+                        pk[mi][ni][q].y = ghip_f32x2_to_bf16x2(o[2], o[3]);
                     }
                 }
-                pk[mi][ni][q].x = (uint32_t)hb[0] | ((uint32_t)hb[1] << 16);
-                pk[mi][ni][q].y = (uint32_t)hb[2] | ((uint32_t)hb[3] << 16);
             }
         }
-    }
+    };
+    if ((kFwd || kF8) && !g.ap.plain) finish(IC<0>{});
+    else finish(IC<1>{});
     if constexpr (kBf16Out) {
         // transposed copy first: LDS_T[n][m], a lane's 4 consecutive rows are 8 contiguous bytes
         if ((EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD) && g.outT) {
@@ -378,6 +439,24 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             const int lc = (lane % LPR) << 4;
             const v4i val = *reinterpret_cast<const v4i*>(smem + ml * PITCH + lc);
             *reinterpret_cast<v4i*>(dst + (long long)ml * N * 2 + lc) = val;
+            if constexpr (EPI == LP_FP8_ACT) {
+                // row amax of the stored values for the next layer's per-row scale: bf16 magnitudes
+                // order like their bit patterns, so the maximum is taken on 15-bit integers
+                unsigned int am = 0;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const unsigned int u = (unsigned int)val[d];
+                    const unsigned int lo = u & 0x7fffu, hi = (u >> 16) & 0x7fffu;
+                    am = am > lo ? am : lo;
+                    am = am > hi ? am : hi;
+                }
+#pragma unroll
+                for (int o = LPR / 2; o > 0; o >>= 1) {
+                    const unsigned int other = (unsigned int)__shfl_xor((int)am, o, 64);
+                    am = am > other ? am : other;
+                }
+                if (lane % LPR == 0) atomicMax(&g.row_amax_bits[bm + ml], am << 16);
+            }
         }
     }
 }
@@ -403,7 +482,7 @@ void resolve_act(GemmLpArgs& g)
 {
     GemmLpArgs::ActForm& a = g.ap;
     const float inf = __builtin_huge_valf(), p = g.act_param;
-    a = GemmLpArgs::ActForm{-inf, 0.f, 0.f, 1.f, 0.f, 1.f, 1.f, 0.f, -inf, 0.f, inf, 0.f, 0, 0, 1.f, 1.f, 1.f, 0.f, 0.f};
+    a = GemmLpArgs::ActForm{-inf, 0.f, 0.f, 1.f, 0.f, 1.f, 1.f, 0.f, -inf, 0.f, inf, 0.f, 0, 0, 0, 1.f, 1.f, 1.f, 0.f, 0.f};
     switch (g.act) {
     case GHIP_TANH:     a.trans = 1; a.tk = 2.f; a.ta = 2.f; a.tb = -1.f; a.c0 = 1.f; a.c2 = -1.f; break;
     case GHIP_TANHP:    a.trans = 1; a.tk = 2.f; a.ta = 2.f; a.tb = -1.f; a.c0 = 1.f; a.c2 = -1.f;
@@ -417,6 +496,7 @@ void resolve_act(GemmLpArgs& g)
     case GHIP_STEP:     a.thr = p; a.a0 = 0.f; a.a1 = 0.f; a.b1 = 1.f; a.c0 = 0.f; break;
     default: break;
     }
+    a.plain = (!a.trans && a.clo == -inf && a.chi == inf) ? 1 : 0;
 }
 
 }  // namespace

@@ -133,6 +133,14 @@ __device__ __forceinline__ uint16_t ghip_f32_to_bf16(float x)
     u += 0x7fffu + ((u >> 16) & 1u);
     return (uint16_t)(u >> 16);
 }
+// two at once with the hardware conversion (round to nearest even): low half = a, high half = b
+__device__ __forceinline__ uint32_t ghip_f32x2_to_bf16x2(float a, float b)
+{
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    const f32x2_t v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 __device__ __forceinline__ float ghip_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 
 // OCP e4m3 (finite only) encode, round-to-nearest-even, saturating at 448.
@@ -247,6 +255,7 @@ enum LpEpilogue {
 struct GemmLpArgs {
     const void* A; const void* B;    // [M][K], [N][K], K contiguous; bf16 or e4m3
     int M, N, K;
+    int lda, ldb;                     // row pitches of A and B in elements (0: K)
     int fp8;                          // 0: bf16 operands, 1: e4m3 operands
     int epilogue;
     void* out; void* outT;            // see LpEpilogue; outT may be NULL
@@ -258,6 +267,7 @@ struct GemmLpArgs {
         //           v = z < clo ? vlo : v;  v = z > chi ? vhi : v
         float thr, a0, b0, a1, b1, tk, ta, tb, clo, vlo, chi, vhi;
         int trans;
+        int plain;  // no transcendental part and no clamps: the first line is the whole activation
         // derivative in the output a:  step ? (a > 0 ? dhi : dlo) : c0 + c1*a + c2*a*a
         int step; float dhi, dlo, c0, c1, c2;
     } ap;
