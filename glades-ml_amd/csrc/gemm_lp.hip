@@ -241,6 +241,34 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     constexpr int KS = FP8 ? 2 : 4;
     constexpr int G = MI * NI;
     constexpr bool kDouble = !(FP8 && G > 2);
+    // Tiles whose epilogue reads more memory get it moving while the K loop leaves HBM idle:
+    // weight-gradient tiles end with a read-modify-write of the fp32 master weights and momentum
+    // (2 x TN x 4 bytes per tile row, bound by HBM), back-propagation tiles read the bf16
+    // activations (TN x 2 bytes per row).  Every stage of the last PF_N each wavefront touches one
+    // dword of 8 of those 128-byte lines, which are then in the memory-side cache (or L2) when the
+    // epilogue asks for them.  The touch goes out between the B and the A loads of the fill, so the
+    // wait that ends a stage (which only needs B) leaves it in flight like the A loads; its result
+    // is never used.
+    constexpr bool kTouch = (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
+    constexpr int PF_ES = (EPI == LP_WGRAD_SGD) ? 4 : 2;         // bytes per element of the touched arrays
+    constexpr int PF_ARRAYS = (EPI == LP_WGRAD_SGD) ? 2 : 1;
+    constexpr int PF_LPR = TN * PF_ES / 128;                     // lines per tile row
+    constexpr int PF_PER = TM * PF_LPR;                          // lines per array
+    constexpr int PF_N = PF_ARRAYS * PF_PER / 64;                // stages needed: 64 lines per stage and workgroup
+    constexpr int PF_LEAD = 2;
+    int pfreg = 0;
+    const int pf_j0 = nk - PF_N - PF_LEAD > 0 ? nk - PF_N - PF_LEAD : 0;
+    auto touch = [&](int j) {
+        int i = j - pf_j0;
+        i = i < 0 ? 0 : (i >= PF_N ? PF_N - 1 : i);  // outside the window: repeat a touched line
+        const int line = (i * 8 + ws) * 8 + (lane & 7);
+        const int within = line % PF_PER;
+        const unsigned char* base = (EPI == LP_DGRAD) ? (const unsigned char*)g.aux
+                                  : (line < PF_PER) ? (const unsigned char*)g.master : (const unsigned char*)g.mom;
+        const unsigned char* src = base + ((long long)(bm + within / PF_LPR) * g.N + bn) * PF_ES + (within % PF_LPR) * 128;
+        if (lane < 8) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
+    };
+    constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0);  // loads a stage's closing wait leaves in flight
     auto stage = [&](auto Pc, int j) {
         constexpr int P = decltype(Pc)::value;
         const unsigned char* const RA = smem + ((2 * P) % NSLOT) * SLOT;
@@ -248,8 +276,9 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         const unsigned char* const NA = smem + ((2 * P + 2) % NSLOT) * SLOT;
         const unsigned char* const NB = smem + ((2 * P + 3) % NSLOT) * SLOT;
         auto dma = [&](int d) {
-            if (d < PWB) dmaB((2 * P + 3) % NSLOT, j + 1, d);
-            else dmaA((2 * P + 4) % NSLOT, j + 2, d - PWB);
+            if (d < PWB) { dmaB((2 * P + 3) % NSLOT, j + 1, d); return; }
+            if (kTouch && d == PWB) touch(j);
+            dmaA((2 * P + 4) % NSLOT, j + 2, d - PWB);
         };
         auto none = [](int) {};
         if constexpr (!kDouble) {
@@ -257,7 +286,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             mma_group<FP8, MI, NI, SPAN, NDMA, 0>(acc, f0, dma);
             load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
             mma_group<FP8, MI, NI, SPAN, NDMA, G>(acc, f0, dma);
-            __builtin_amdgcn_s_waitcnt(0x0070 | PWA);  // vmcnt(PWA) lgkmcnt(0)
+            __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
             load_frags<FP8, MI, NI>(f0, NA, NB, 0, wm, wn, l31, lh);
         } else {
@@ -270,7 +299,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): cur has landed
                     load_frags<FP8, MI, NI>(nxt, RA, RB, ks + 1, wm, wn, l31, lh);
                 } else {
-                    __builtin_amdgcn_s_waitcnt(0x0070 | PWA);  // vmcnt(PWA) lgkmcnt(0)
+                    __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
                     __builtin_amdgcn_s_barrier();
                     load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
                 }
@@ -292,6 +321,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     }
     // nothing may still be writing this workgroup's LDS when its wavefronts retire
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    asm volatile("" : : "v"(pfreg));  // the touches' destination stays reserved up to here
 
     // ---- epilogue.  Accumulator layout of a 32x32 tile: lane -> column lane%32,
     //      register i -> row 8*(i/4) + 4*(lane/32) + i%4  (4 consecutive rows per register quad).
