@@ -80,6 +80,7 @@ struct ghip_net {
     uint16_t* HT[GHIP_MAX_LAYERS + 1] = {};
     uint16_t* D[GHIP_MAX_LAYERS + 1] = {};
     uint16_t* DT[GHIP_MAX_LAYERS + 1] = {};
+    float* csum[GHIP_MAX_LAYERS + 1] = {};  // per-tile-row column sums of D[l] (bias gradient partials)
     float* logits = nullptr;
     bool shadow_dirty = true;
     // fp8
@@ -283,7 +284,7 @@ void free_batch_buffers(ghip_net* n)
     for (int l = 0; l <= GHIP_MAX_LAYERS; ++l) {
         dfree(n->act[l]); dfree(n->dlt[l]);
         if (l > 0) dfree(n->H[l]);
-        dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]);
+        dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]); dfree(n->csum[l]);
     }
     dfree(n->stageX); dfree(n->logits);
     dfree(n->Aq[0]); dfree(n->Aq[1]); dfree(n->ascale[0]); dfree(n->ascale[1]);
@@ -316,6 +317,7 @@ int reserve_batch(ghip_net* n, int B)
             }
             TRY(dalloc(&n->D[l], (size_t)B * s.sizes[l]));
             TRY(dalloc(&n->DT[l], (size_t)B * s.sizes[l]));
+            if (l < L) TRY(dalloc(&n->csum[l], (size_t)((B + 127) / 128) * s.sizes[l]));
         }
         TRY(dalloc(&n->logits, (size_t)B * s.sizes[L]));
     } else {
@@ -461,11 +463,15 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
         if (l > 0) {
             memset(&g, 0, sizeof(g));
             g.A = n->D[l + 1]; g.B = n->WhT[l]; g.M = B; g.N = ni; g.K = no;
-            g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.aux = n->H[l];
+            g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.aux = n->H[l]; g.colsum = n->csum[l];
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1];
             LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));
         }
-        LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+        if (l + 1 < L)  // D[l+1] came from a back-propagation product, which left its column sums
+            LAUNCH(n, "bias_update_bf16", ghip_bias_update_partials(n->csum[l + 1], B / ghip_gemm_lp_tile_m(B, no), no, B, n->b[l], n->vb[l],
+                                                                    s.lr[l], s.mom[l], n->stream));
+        else
+            LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
         memset(&g, 0, sizeof(g));
         g.A = n->DT[l + 1]; g.B = n->HT[l]; g.M = no; g.N = ni; g.K = B;
         g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l];
@@ -748,7 +754,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
             DeltaArgs a;
             memset(&a, 0, sizeof(a));
             a.P = n->act[L]; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
-            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc;
+            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc; a.store_p = 1;
             LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
         }
         *result = n->act[L];
@@ -759,7 +765,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
             DeltaArgs a;
             memset(&a, 0, sizeof(a));
             a.P = n->logits; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
-            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc;
+            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc; a.store_p = 1;
             LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
         }
         *result = n->logits;

@@ -85,7 +85,7 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
             float d;
             if (softmax) {
                 pv = kInRegs ? pv * inv : expf(pv - mx) * inv;
-                p[o] = pv;
+                if (a.store_p) p[o] = pv;
                 if (yv != 0.0f) l += -(yv * logf(fmaxf(pv, 1e-30f)));
                 d = pv - yv;
             } else {
@@ -118,6 +118,104 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
         loss += (double)wave_sum(l);
         accs += (double)wave_sum(ac);
         if (ip == iy) corr += 1.0;
+    }
+    __shared__ double red[4][3];
+    if (lane == 0) { red[w][0] = loss; red[w][1] = accs; red[w][2] = corr; }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        double v = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
+        atomicAdd(&a.acc[threadIdx.x], v);
+    }
+}
+
+// The same for rows whose length is a multiple of 4 and at most 256 * Q: one row per wavefront,
+// lane l owns columns 4*(j*64 + l) .. +3 for j < Q.  The row's outputs and targets are requested
+// together as 16-byte loads before anything is computed (one memory round trip per row), deltas
+// leave as 16-byte (fp32) or 8-byte (bf16) stores.
+template <int Q>
+__global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
+{
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int b = blockIdx.x * 4 + w;
+    double loss = 0.0, accs = 0.0, corr = 0.0;
+    const bool softmax = a.act == GHIP_SOFTMAX;
+    const bool sig_bce = (a.act == GHIP_SIGMOID || a.act == GHIP_SIGMOIDP) && a.cost == GHIP_CLASSIFICATION;
+    if (b < a.B) {
+        float* p = a.P + (long long)b * a.ldp;
+        const float* y = a.Y ? a.Y + (long long)b * a.ldy : nullptr;
+        float4 pr[Q], yr[Q];
+#pragma unroll
+        for (int j = 0; j < Q; ++j) {
+            const int o = (j * 64 + lane) * 4;
+            pr[j] = (o < a.n) ? *reinterpret_cast<const float4*>(p + o) : make_float4(-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f);
+        }
+#pragma unroll
+        for (int j = 0; j < Q; ++j) {
+            const int o = (j * 64 + lane) * 4;
+            yr[j] = (y && o < a.n) ? *reinterpret_cast<const float4*>(y + o) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        float inv = 1.0f;
+        if (softmax) {
+            float m = -3.0e38f;
+#pragma unroll
+            for (int j = 0; j < Q; ++j) m = fmaxf(fmaxf(m, fmaxf(pr[j].x, pr[j].y)), fmaxf(pr[j].z, pr[j].w));
+            const float mx = wave_max(m);
+            float s = 0.0f;
+#pragma unroll
+            for (int j = 0; j < Q; ++j) {
+                const bool ok = (j * 64 + lane) * 4 < a.n;
+                pr[j].x = ok ? expf(pr[j].x - mx) : 0.0f; pr[j].y = ok ? expf(pr[j].y - mx) : 0.0f;
+                pr[j].z = ok ? expf(pr[j].z - mx) : 0.0f; pr[j].w = ok ? expf(pr[j].w - mx) : 0.0f;
+                s += (pr[j].x + pr[j].y) + (pr[j].z + pr[j].w);
+            }
+            inv = 1.0f / wave_sum(s);
+        }
+        float l = 0.0f, ac = 0.0f;
+        float bp = 0.0f, by = 0.0f;  // running maxima for the argmax rule (start at 0, strict >)
+        int ip = 0x7fffffff, iy = 0x7fffffff;
+        auto element = [&](int o, float& pv, float yv) -> float {
+            float d;
+            if (softmax) {
+                pv = pv * inv;
+                if (yv != 0.0f) l += -(yv * logf(fmaxf(pv, 1e-30f)));
+                d = pv - yv;
+            } else {
+                l += ghip_cost<false>(yv, pv, 1.0f, a.cost);
+                d = sig_bce ? (pv - yv) : ghip_cost_der(yv, pv, a.cost) * ghip_act_der_canon(pv, a.act, a.act_param);
+            }
+            ac += ghip_accuracy_term(pv, yv);
+            if (pv > bp) { bp = pv; ip = o; }
+            if (yv > by) { by = yv; iy = o; }
+            return d;
+        };
+#pragma unroll
+        for (int j = 0; j < Q; ++j) {
+            const int o = (j * 64 + lane) * 4;
+            if (o < a.n) {
+                float4 d;
+                d.x = element(o, pr[j].x, yr[j].x); d.y = element(o + 1, pr[j].y, yr[j].y);
+                d.z = element(o + 2, pr[j].z, yr[j].z); d.w = element(o + 3, pr[j].w, yr[j].w);
+                if (a.store_p) *reinterpret_cast<float4*>(p + o) = pr[j];
+                if (a.D) *reinterpret_cast<float4*>(a.D + (long long)b * a.n + o) = d;
+                if (a.Dbf) {
+                    uint2 h;
+                    h.x = (uint32_t)ghip_f32_to_bf16(d.x) | ((uint32_t)ghip_f32_to_bf16(d.y) << 16);
+                    h.y = (uint32_t)ghip_f32_to_bf16(d.z) | ((uint32_t)ghip_f32_to_bf16(d.w) << 16);
+                    *reinterpret_cast<uint2*>(a.Dbf + (long long)b * a.n + o) = h;
+                }
+            }
+        }
+        // argmax across lanes: largest value, lowest index on ties; "no element above 0" = none
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            float ov = __shfl_xor(bp, o, 64); int oi = __shfl_xor(ip, o, 64);
+            if (ov > bp || (ov == bp && oi < ip)) { bp = ov; ip = oi; }
+            ov = __shfl_xor(by, o, 64); oi = __shfl_xor(iy, o, 64);
+            if (ov > by || (ov == by && oi < iy)) { by = ov; iy = oi; }
+        }
+        loss = (double)wave_sum(l);
+        accs = (double)wave_sum(ac);
+        if (ip == iy) corr = 1.0;
     }
     __shared__ double red[4][3];
     if (lane == 0) { red[w][0] = loss; red[w][1] = accs; red[w][2] = corr; }
@@ -174,20 +272,44 @@ bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* _
     const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (o >= n) return;
     const uint4* row = reinterpret_cast<const uint4*>(DT + (long long)o * B);
-    float s = 0.0f;
-    for (int k = lane; k < (B >> 3); k += 64) {
-        const uint4 q = row[k];
-        const unsigned int wds[4] = {q.x, q.y, q.z, q.w};
+    float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int nq = B >> 3;
+    for (int k0 = 0; k0 < nq; k0 += 256) {  // four independent 16-byte loads in flight per lane
+        uint4 q[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) s += __uint_as_float(wds[j] << 16) + __uint_as_float(wds[j] & 0xffff0000u);
+        for (int u = 0; u < 4; ++u) {
+            const int k = k0 + u * 64 + lane;
+            q[u] = (k < nq) ? row[k] : make_uint4(0u, 0u, 0u, 0u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const unsigned int wds[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) s4[u] += __uint_as_float(wds[j] << 16) + __uint_as_float(wds[j] & 0xffff0000u);
+        }
     }
-    s = wave_sum(s);
+    float s = wave_sum((s4[0] + s4[1]) + (s4[2] + s4[3]));
     if (lane == 0) {
         const float g = s / (float)B;
         const float d = lr * g + mom * vb[o];
         vb[o] = d;
         bias[o] = bias[o] - d;
     }
+}
+
+// bias update from per-tile-row partial column sums [tiles][n]: a thread per channel adds them in order
+__global__ void __launch_bounds__(256)
+bias_update_partials_kernel(const float* __restrict__ part, int tiles, int n, int B, float* __restrict__ bias,
+                            float* __restrict__ vb, float lr, float mom)
+{
+    const int o = blockIdx.x * 256 + threadIdx.x;
+    if (o >= n) return;
+    float s = 0.0f;
+    for (int k = 0; k < tiles; ++k) s += part[(long long)k * n + o];
+    const float g = s / (float)B;
+    const float d = lr * g + mom * vb[o];
+    vb[o] = d;
+    bias[o] = bias[o] - d;
 }
 
 template <typename T>
@@ -223,6 +345,34 @@ convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ ds
             const int c = c0 + j, r = r0 + tx;
             if (r < rows && c < cols) dstT[(long long)c * rows + r] = tile[tx][j];
         }
+    }
+}
+
+// bf16 transposition with 16-byte global accesses: a 64 x 64 tile enters LDS row by row (8 lanes
+// per source row) and leaves column by column (each lane gathers 8 values of one source column).
+// rows and cols are multiples of 64 here; other shapes take the kernel above.
+__global__ void __launch_bounds__(256)
+bf16_transpose64_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dstT, int rows, int cols)
+{
+    __shared__ uint16_t tile[64][64 + 2];  // 33 dwords per row: column walks rotate over the banks
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const int sub = threadIdx.x & 7, line = threadIdx.x >> 3;  // 8 lanes per 128-byte line, 32 lines per pass
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int r = line + 32 * h;
+        const uint4 v = *reinterpret_cast<const uint4*>(src + (long long)(r0 + r) * cols + c0 + sub * 8);
+        uint32_t* t32 = reinterpret_cast<uint32_t*>(&tile[r][sub * 8]);
+        t32[0] = v.x; t32[1] = v.y; t32[2] = v.z; t32[3] = v.w;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int c = line + 32 * h;  // source column = destination row
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            o[k] = (uint32_t)tile[sub * 8 + 2 * k][c] | ((uint32_t)tile[sub * 8 + 2 * k + 1][c] << 16);
+        *reinterpret_cast<uint4*>(dstT + (long long)(c0 + c) * rows + r0 + sub * 8) = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 
@@ -270,6 +420,16 @@ inline int grid_for(long long n, int cap = 65535 * 4)
 
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
 {
+    const bool vec_ok = (a.n % 4) == 0 && a.n <= 2048 && (a.ldp % 4) == 0 && (!a.Y || (a.ldy % 4) == 0) &&
+                        ((uintptr_t)a.P % 16) == 0 && ((uintptr_t)a.Y % 16) == 0 && ((uintptr_t)a.D % 16) == 0 && ((uintptr_t)a.Dbf % 8) == 0;
+    if (vec_ok) {
+        const dim3 grid4((a.B + 3) / 4);
+        if (a.n <= 256) hipLaunchKernelGGL(output_delta_vec4_kernel<1>, grid4, dim3(256), 0, s, a);
+        else if (a.n <= 512) hipLaunchKernelGGL(output_delta_vec4_kernel<2>, grid4, dim3(256), 0, s, a);
+        else if (a.n <= 1024) hipLaunchKernelGGL(output_delta_vec4_kernel<4>, grid4, dim3(256), 0, s, a);
+        else hipLaunchKernelGGL(output_delta_vec4_kernel<8>, grid4, dim3(256), 0, s, a);
+        return hipGetLastError();
+    }
     const int rows_per_block = 4 * kRowsPerWave;
     const dim3 grid((a.B + rows_per_block - 1) / rows_per_block);
     if (a.n <= 64 * kRegs) hipLaunchKernelGGL(output_delta_kernel<true>, grid, dim3(256), 0, s, a);
@@ -299,6 +459,13 @@ hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias,
     return hipGetLastError();
 }
 
+hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B, float* bias, float* vb, float lr,
+                                     float mom, hipStream_t s)
+{
+    hipLaunchKernelGGL(bias_update_partials_kernel, dim3((n + 255) / 256), dim3(256), 0, s, part, tiles, n, B, bias, vb, lr, mom);
+    return hipGetLastError();
+}
+
 hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s)
 {
     hipLaunchKernelGGL(fill_kernel<float>, dim3(grid_for(n, 2048)), dim3(256), 0, s, p, n, v);
@@ -325,6 +492,10 @@ hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, 
 hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s)
 {
     dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    if ((rows % 64) == 0 && (cols % 64) == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)dstT % 16) == 0) {
+        hipLaunchKernelGGL(bf16_transpose64_kernel, grid, dim3(256), 0, s, src, dstT, rows, cols);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols);
     return hipGetLastError();
 }

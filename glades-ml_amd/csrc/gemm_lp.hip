@@ -419,6 +419,24 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     };
     if ((kFwd || kF8) && !g.ap.plain) finish(IC<0>{});
     else finish(IC<1>{});
+    // back-propagation also leaves the column sums of the deltas it stores (the bias gradient of
+    // the layer below), per tile row so that the caller adds them in a fixed order
+    float csum[NI];
+    if constexpr (EPI == LP_DGRAD) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ++ni) {
+            float s = 0.0f;
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const uint2 v = pk[mi][ni][q];
+                    s += (__uint_as_float(v.x << 16) + __uint_as_float(v.x & 0xffff0000u)) +
+                         (__uint_as_float(v.y << 16) + __uint_as_float(v.y & 0xffff0000u));
+                }
+            csum[ni] = s + __shfl_xor(s, 32, 64);
+        }
+    }
     if constexpr (kBf16Out) {
         // transposed copy first: LDS_T[n][m], a lane's 4 consecutive rows are 8 contiguous bytes
         if ((EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD) && g.outT) {
@@ -489,6 +507,19 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             }
         }
     }
+    if constexpr (EPI == LP_DGRAD) {
+        if (g.colsum) {
+            float* red = reinterpret_cast<float*>(smem);  // [2][TN]: one row per wavefront row
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();  // the staged tile has been read
+            if (lh == 0)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) red[(w >> 2) * TN + wn + ni * 32 + l31] = csum[ni];
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();
+            if (t < TN) g.colsum[(long long)tm * N + bn + t] = red[t] + red[TN + t];
+        }
+    }
 }
 
 // 256 x 256 tiles when they give every CU at least one workgroup, else 128 x 128.
@@ -530,6 +561,8 @@ void resolve_act(GemmLpArgs& g)
 }
 
 }  // namespace
+
+int ghip_gemm_lp_tile_m(int M, int N) { return use_small_tile(M, N) ? 128 : 256; }
 
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8)
 {

@@ -229,6 +229,7 @@ struct DeltaArgs {
     int B, n, ldp, ldy;
     int act; float act_param; int cost;
     double* acc;
+    int store_p;   // write the activated outputs (softmax probabilities) back into P
 };
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s);
 
@@ -261,6 +262,7 @@ struct GemmLpArgs {
     void* out; void* outT;            // see LpEpilogue; outT may be NULL
     const float* bias;                // [N] or NULL
     const uint16_t* aux;              // LP_DGRAD: activations bf16 [M][N]
+    float* colsum;                    // LP_DGRAD: if set, [M / tile_m][N] column sums of the stored deltas per tile row
     int act; float act_param;   // resolved into `ap` by ghip_gemm_lp
     struct ActForm {
         // forward:  v = z < thr ? a0*z + b0 : a1*z + b1;  if (trans) v = ta / (1 + exp(-tk*z)) + tb;
@@ -278,12 +280,16 @@ struct GemmLpArgs {
 };
 hipError_t ghip_gemm_lp(const GemmLpArgs& a, hipStream_t s);
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8);
+int ghip_gemm_lp_tile_m(int M, int N);  // rows per tile the launcher picks for this product
 
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
 hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s);
 // bias update from bf16 delta^T [n][B] rows (contiguous): gb[o] = sum_b
 hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vbias, float lr,
                                   float mom, hipStream_t s);
+// the same from per-tile-row partial column sums [tiles][n] (written by the LP_DGRAD epilogue)
+hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B, float* bias, float* vbias, float lr,
+                                     float mom, hipStream_t s);
 // per-row e4m3 quantisation: src fp32/bf16 [rows][cols]; scale = amax/448 (1 if row is zero).
 // amax_bits: if non-NULL the row amax is taken from there (uint bits of a non-negative float)
 // instead of being reduced from the row.
