@@ -409,7 +409,15 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                         }
                         if constexpr (EPI == LP_FWD_F32 || EPI == LP_FP8_F32) ((float*)g.out)[idx] = o[r];
                     }
-                    if constexpr (kBf16Out) {
+                    if constexpr (EPI == LP_FP8_ACT) {
+                        // single output: straight into the row-major staging area
+                        const unsigned int p01 = ghip_f32x2_to_bf16x2(o[0], o[1]), p23 = ghip_f32x2_to_bf16x2(o[2], o[3]);
+                        unsigned char* d0 = smem + (wm + mi * 32 + 8 * q + 4 * lh) * PITCH + (wn + ni * 32 + l31) * 2;
+                        *reinterpret_cast<uint16_t*>(d0) = (uint16_t)(p01 & 0xffffu);
+                        *reinterpret_cast<uint16_t*>(d0 + PITCH) = (uint16_t)(p01 >> 16);
+                        *reinterpret_cast<uint16_t*>(d0 + 2 * PITCH) = (uint16_t)(p23 & 0xffffu);
+                        *reinterpret_cast<uint16_t*>(d0 + 3 * PITCH) = (uint16_t)(p23 >> 16);
+                    } else if constexpr (kBf16Out) {
                         pk[mi][ni][q].x = ghip_f32x2_to_bf16x2(o[0], o[1]);
                         pk[mi][ni][q].y = ghip_f32x2_to_bf16x2(o[2], o[3]);
                     }
@@ -464,6 +472,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             __builtin_amdgcn_s_barrier();
         }
         // row-major copy: LDS[m][n]
+        if constexpr (EPI != LP_FP8_ACT)
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -479,10 +488,11 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                 }
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_s_barrier();
-        constexpr int LPR = TN / 8, RPI = 64 / LPR;
+        constexpr int LPR = TN / 8, RPI = 64 / LPR, NIT = (TM / 8) / RPI;
         unsigned char* dst = (unsigned char*)g.out + ((long long)bm * N + bn) * 2;
+        unsigned int am[NIT];
 #pragma unroll
-        for (int i = 0; i < (TM / 8) / RPI; ++i) {
+        for (int i = 0; i < NIT; ++i) {
             const int ml = w * (TM / 8) + i * RPI + lane / LPR;
             const int lc = (lane % LPR) << 4;
             const v4i val = *reinterpret_cast<const v4i*>(smem + ml * PITCH + lc);
@@ -490,21 +500,29 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             if constexpr (EPI == LP_FP8_ACT) {
                 // row amax of the stored values for the next layer's per-row scale: bf16 magnitudes
                 // order like their bit patterns, so the maximum is taken on 15-bit integers
-                unsigned int am = 0;
+                unsigned int m = 0;
 #pragma unroll
                 for (int d = 0; d < 4; ++d) {
                     const unsigned int u = (unsigned int)val[d];
                     const unsigned int lo = u & 0x7fffu, hi = (u >> 16) & 0x7fffu;
-                    am = am > lo ? am : lo;
-                    am = am > hi ? am : hi;
+                    m = m > lo ? m : lo;
+                    m = m > hi ? m : hi;
                 }
-#pragma unroll
-                for (int o = LPR / 2; o > 0; o >>= 1) {
-                    const unsigned int other = (unsigned int)__shfl_xor((int)am, o, 64);
-                    am = am > other ? am : other;
-                }
-                if (lane % LPR == 0) atomicMax(&g.row_amax_bits[bm + ml], am << 16);
+                am[i] = m;
             }
+        }
+        if constexpr (EPI == LP_FP8_ACT) {
+            // the NIT reductions side by side, so that their cross-lane steps overlap
+#pragma unroll
+            for (int o = LPR / 2; o > 0; o >>= 1)
+#pragma unroll
+                for (int i = 0; i < NIT; ++i) {
+                    const unsigned int other = (unsigned int)__shfl_xor((int)am[i], o, 64);
+                    am[i] = am[i] > other ? am[i] : other;
+                }
+            if (lane % LPR == 0)
+#pragma unroll
+                for (int i = 0; i < NIT; ++i) atomicMax(&g.row_amax_bits[bm + w * (TM / 8) + i * RPI + lane / LPR], am[i] << 16);
         }
     }
     if constexpr (EPI == LP_DGRAD) {
