@@ -26,13 +26,16 @@ sys.path.insert(0, os.path.join(ROOT, "glades-ml_amd"))
 PEAKS = {"bf16": 2500.0, "fp8": 5000.0, "f32": 157.3}  # dense MFMA, TFLOP/s
 HBM_PEAK = 8000.0  # GB/s
 
-# HBM bytes per launch of a workload's dominant kernel, from two `rocprofv3 --pmc` runs of this
+# Memory bytes per launch of a workload's dominant kernel, from two `rocprofv3 --pmc` runs of this
 # script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch averaged over the kernel's launches), each
 # scaled by what the same counter reads for the 1 GiB copy of `--workload copy`
-# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); profiles/gemm_bf16_cfg4_pmc.md has the runs.
+# (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); profiles/gemm_lowprec_pmc.md has the runs.  The
+# counters sit between L2 and the fabric, so lines re-fetched from the memory-side cache count again.
 # A workload / kernel pair that was not measured reports null.
 MEASURED_TRAFFIC_BYTES = {
-    ("cfg4", "gemm_bf16_wgrad_sgd"): int((233040.23 * 2.000 + 167116.8 * 1.000) * 1024),
+    # mean over the step's 5 launches: 4 x (329294.5 x 2 + 196608) KiB and 1 x (126595.3 x 2 + 49152) KiB
+    ("cfg4", "gemm_bf16_wgrad_sgd"): int((4 * (329294.5 * 2.000 + 196608.0) + (126595.26 * 2.000 + 49152.0)) / 5 * 1024),
+    ("cfg5", "gemm_fp8_forward"): int((789038.85 * 2.000 + 270336.0 * 1.000) * 1024),
 }
 
 WORKLOADS = {

@@ -298,14 +298,21 @@ bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* _
 }
 
 // bias update from per-tile-row partial column sums [tiles][n]: a thread per channel adds them in order
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 bias_update_partials_kernel(const float* __restrict__ part, int tiles, int n, int B, float* __restrict__ bias,
                             float* __restrict__ vb, float lr, float mom)
 {
-    const int o = blockIdx.x * 256 + threadIdx.x;
+    const int o = blockIdx.x * 64 + threadIdx.x;
     if (o >= n) return;
     float s = 0.0f;
-    for (int k = 0; k < tiles; ++k) s += part[(long long)k * n + o];
+    int k = 0;
+    for (; k + 8 <= tiles; k += 8) {  // eight independent loads in flight, added in a fixed order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = part[(long long)(k + u) * n + o];
+        s += ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]));
+    }
+    for (; k < tiles; ++k) s += part[(long long)k * n + o];
     const float g = s / (float)B;
     const float d = lr * g + mom * vb[o];
     vb[o] = d;
@@ -540,7 +547,7 @@ hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias,
 hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B, float* bias, float* vb, float lr,
                                      float mom, hipStream_t s)
 {
-    hipLaunchKernelGGL(bias_update_partials_kernel, dim3((n + 255) / 256), dim3(256), 0, s, part, tiles, n, B, bias, vb, lr, mom);
+    hipLaunchKernelGGL(bias_update_partials_kernel, dim3((n + 63) / 64), dim3(64), 0, s, part, tiles, n, B, bias, vb, lr, mom);
     return hipGetLastError();
 }
 
