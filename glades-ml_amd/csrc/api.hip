@@ -61,6 +61,9 @@ struct ghip_net {
     int exMetricsCap = 0;
     int64_t exPredsCap = 0;
     int* exEpochs = nullptr;
+    int* cm = nullptr;              // confusion counters (both modes), n_out x n_out
+    float* exClass = nullptr;       // exact mode: 5 floats per epoch of the last call
+    int exClassCap = 0, exClassRan = 0;
     // canonical fp32 state (also the master copy for BF16 / the source for FP8)
     float* W[GHIP_MAX_LAYERS] = {};
     float* b[GHIP_MAX_LAYERS] = {};
@@ -383,6 +386,7 @@ int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
     a.P = P; a.Y = Y; a.D = D; a.Dbf = Dbf; a.DbfT = nullptr;
     a.B = B; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
     a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost; a.acc = n->dAcc;
+    a.cm = n->cm;
     LAUNCH(n, "output_delta", ghip_output_delta(a, n->stream));
     return 0;
 }
@@ -573,7 +577,7 @@ int ghip_net_destroy(ghip_net* n)
     free_batch_buffers(n);
     dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf);
     dfree(n->exW); dfree(n->exSum); dfree(n->exLast); dfree(n->exBias); dfree(n->exPreds);
-    dfree(n->exMetrics); dfree(n->exEpochs);
+    dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass);
     for (int l = 0; l < GHIP_MAX_LAYERS; ++l) {
         dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]); dfree(n->gW[l]);
         dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
@@ -711,11 +715,24 @@ int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_a
     e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
     e.preds = host_preds ? n->exPreds : nullptr;
     e.metrics = (float*)n->exMetrics;
+    e.cm = n->cm;
+    e.class_metrics = nullptr;
+    if (n->cm && nout <= 64) {
+        if (n_epochs > n->exClassCap) {
+            HIP_TRY(hipStreamSynchronize(n->stream));
+            dfree(n->exClass);
+            TRY(dalloc(&n->exClass, (size_t)n_epochs * 5));
+            n->exClassCap = n_epochs;
+        }
+        e.class_metrics = n->exClass;
+    }
+    n->exClassRan = 0;
     LAUNCH(n, "exact_epochs", ghip_launch_exact(e, n->ex_threads, n->ex_lds, n->stream));
     int ran = 0;
     HIP_TRY(hipMemcpyAsync(&ran, n->exEpochs, sizeof(int), hipMemcpyDeviceToHost, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
     if (epochs_run) *epochs_run = ran;
+    n->exClassRan = e.class_metrics ? ran : 0;
     if (host_metrics && ran > 0) HIP_TRY(hipMemcpy(host_metrics, n->exMetrics, sizeof(ghip_metrics) * ran, hipMemcpyDeviceToHost));
     if (host_preds) HIP_TRY(hipMemcpy(host_preds, n->exPreds, sizeof(float) * n->n_rows * nout, hipMemcpyDeviceToHost));
     return 0;
@@ -830,6 +847,50 @@ int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* h
     TRY(output_delta_f32(n, P, n->dY + row0 * s.sizes[L], nullptr, nullptr, batch));
     n->last_batch = batch;
     return fetch_metrics(n, host_metrics);
+}
+
+int ghip_net_confusion_enable(ghip_net* n, int enable)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    dfree(n->cm);
+    if (!enable) return 0;
+    const int nout = n->spec.sizes[n->L];
+    if (nout > 8192) return fail(GHIP_EINVAL, "confusion matrix of %d classes is not supported", nout);
+    TRY(dalloc(&n->cm, (size_t)nout * nout));
+    HIP_TRY(hipMemsetAsync(n->cm, 0, sizeof(int) * (size_t)nout * nout, n->stream));
+    return 0;
+}
+
+int ghip_net_confusion_reset(ghip_net* n)
+{
+    if (!n) return fail(GHIP_EINVAL, "net is NULL");
+    if (!n->cm) return fail(GHIP_ESTATE, "confusion matrix is not enabled");
+    const int nout = n->spec.sizes[n->L];
+    LAUNCH(n, "fill_confusion", ghip_fill_u32((unsigned int*)n->cm, (long long)nout * nout, 0u, n->stream));
+    return 0;
+}
+
+int ghip_net_confusion_get(ghip_net* n, int32_t* host_matrix, int64_t len)
+{
+    if (!n || !host_matrix) return fail(GHIP_EINVAL, "bad arguments");
+    if (!n->cm) return fail(GHIP_ESTATE, "confusion matrix is not enabled");
+    const int64_t nout = n->spec.sizes[n->L];
+    if (len != nout * nout) return fail(GHIP_EINVAL, "matrix has %lld cells, caller gave room for %lld", (long long)(nout * nout), (long long)len);
+    HIP_TRY(hipMemcpyAsync(host_matrix, n->cm, sizeof(int32_t) * len, hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    return 0;
+}
+
+int ghip_net_class_metrics(ghip_net* n, int epoch, ghip_class_metrics* out)
+{
+    if (!n || !out) return fail(GHIP_EINVAL, "bad arguments");
+    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "per-epoch class metrics are an exact-mode figure");
+    if (epoch < 0 || epoch >= n->exClassRan)
+        return fail(GHIP_EINVAL, "epoch %d of %d with class metrics (enable the confusion matrix before the run; n_out <= 64)", epoch, n->exClassRan);
+    HIP_TRY(hipMemcpyAsync(out, n->exClass + 5 * epoch, sizeof(float) * 5, hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    return 0;
 }
 
 int ghip_net_quantize_fp8(ghip_net* n, float* const* host_scales, uint8_t* const* host_codes)

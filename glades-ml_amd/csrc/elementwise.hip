@@ -118,6 +118,8 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
         loss += (double)wave_sum(l);
         accs += (double)wave_sum(ac);
         if (ip == iy) corr += 1.0;
+        // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
+        if (a.cm && lane == 0 && ip != 0x7fffffff && iy != 0x7fffffff) atomicAdd(&a.cm[(long long)iy * a.n + ip], 1);
     }
     __shared__ double red[4][3];
     if (lane == 0) { red[w][0] = loss; red[w][1] = accs; red[w][2] = corr; }
@@ -216,6 +218,8 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
         loss = (double)wave_sum(l);
         accs = (double)wave_sum(ac);
         if (ip == iy) corr = 1.0;
+        // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
+        if (a.cm && lane == 0 && ip != 0x7fffffff && iy != 0x7fffffff) atomicAdd(&a.cm[(long long)iy * a.n + ip], 1);
     }
     __shared__ double red[4][3];
     if (lane == 0) { red[w][0] = loss; red[w][1] = accs; red[w][2] = corr; }

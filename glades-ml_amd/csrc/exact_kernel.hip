@@ -104,6 +104,11 @@ exact_kernel(ExactLaunch p)
         float tot_err = 0.0f, tot_acc = 0.0f;
         long long correct = 0;
         const bool last_epoch = (ep == p.n_epochs - 1) || (p.stop_accuracy > 0.0f);
+        if (p.cm) {  // CMatrix::reset at the head of every epoch (network.cpp:183-185)
+            for (int k = tid; k < nout * nout; k += T) p.cm[k] = 0;
+            __threadfence();
+            __syncthreads();
+        }
         for (long long r = 0; r < p.n_rows; ++r) {
             // ---- stage the row (prefetched) and start fetching the next one
             if (small_row) {
@@ -164,6 +169,8 @@ exact_kernel(ExactLaunch p)
                     if (ex > my) { my = ex; iy = o; }
                 }
                 if (ip == iy) ++correct;
+                // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
+                if (p.cm && ip >= 0 && iy >= 0) atomicAdd(&p.cm[iy * nout + ip], 1);
             }
 
             if (p.train) {
@@ -271,6 +278,10 @@ exact_kernel(ExactLaunch p)
             m->loss = tot_err;
             m->accuracy = acc;
             m->correct = correct;
+            if (p.cm && p.class_metrics) {  // network.cpp:218-224, read back through the atomics' path
+                __threadfence();
+                ghip_cmatrix_overall(p.cm, nout, p.class_metrics + 5 * ep);
+            }
             if (p.stop_accuracy > 0.0f && acc >= p.stop_accuracy) sflag[0] = 1;
         }
         __syncthreads();

@@ -124,6 +124,39 @@ __device__ __forceinline__ float ghip_accuracy_term(float pred, float expect)
     return acc < 0.0f ? 0.0f : acc;
 }
 
+// Overall class metrics of the reference's confusion matrix (ML/GMath/cmatrix.cpp:100-132 for the
+// per-class counts, :139-265 for the ratios): M is n x n, row = expected class, column = predicted.
+// falsePositive[c] / falseNegative[r] collect the off-diagonal cells of column c / row r;
+// truePositive[i] is the diagonal cell; trueNegative[i] is the sum of the OTHER classes' diagonal
+// cells only.  Ratios are float, the overall figure is the mean over classes in class order (0/0
+// gives NaN and stays).  out[0..4] = accuracy, precision, recall, specificity, F1 as fractions.
+// Meant for one lane and a small n: O(n^2) reads.
+__device__ inline void ghip_cmatrix_overall(const int* M, int n, float* out)
+{
+    // device-scope atomic loads: the counters are bumped with atomics, which live in L2
+    auto at = [&](int idx) { return __hip_atomic_load(M + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+    int diag_sum = 0;
+    for (int i = 0; i < n; ++i) diag_sum += at(i * n + i);
+    float acc = 0.0f, pre = 0.0f, rec = 0.0f, spe = 0.0f, f1 = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        int fp = 0, fn = 0;
+        for (int k = 0; k < n; ++k)
+            if (k != i) { fp += at(k * n + i); fn += at(i * n + k); }
+        const int tp = at(i * n + i), tn = diag_sum - tp;
+        const float truth = (float)(tp + tn), untruth = (float)(fp + fn);
+        acc = __fadd_rn(acc, __fdiv_rn(truth, __fadd_rn(truth, untruth)));
+        const float cp = __fdiv_rn((float)tp, (float)(tp + fp));
+        const float cr = __fdiv_rn((float)tp, (float)(tp + fn));
+        pre = __fadd_rn(pre, cp);
+        rec = __fadd_rn(rec, cr);
+        spe = __fadd_rn(spe, __fdiv_rn((float)tn, (float)(tn + fp)));
+        f1 = __fadd_rn(f1, __fdiv_rn(__fmul_rn(__fmul_rn(2.0f, cr), cp), __fadd_rn(cr, cp)));
+    }
+    const float nn = (float)n;
+    out[0] = __fdiv_rn(acc, nn); out[1] = __fdiv_rn(pre, nn); out[2] = __fdiv_rn(rec, nn);
+    out[3] = __fdiv_rn(spe, nn); out[4] = __fdiv_rn(f1, nn);
+}
+
 // ---------------------------------------------------------------- bf16 helpers (bit level)
 
 __device__ __forceinline__ uint16_t ghip_f32_to_bf16(float x)
@@ -193,6 +226,8 @@ struct ExactLaunch {
     float* metrics;// per epoch: loss, accuracy, correct (as float bits of an int), spare
     int*   epochs_run;
     int    state_in_lds;
+    int*   cm;            // n_out x n_out confusion counters of the running epoch, or NULL
+    float* class_metrics; // per epoch: overall accuracy, precision, recall, specificity, F1 (NULL with cm)
 };
 
 hipError_t ghip_launch_exact(const ExactLaunch& p, int threads, size_t lds_bytes, hipStream_t s);
@@ -229,6 +264,7 @@ struct DeltaArgs {
     int B, n, ldp, ldy;
     int act; float act_param; int cost;
     double* acc;
+    int* cm;       // n x n confusion counters (row expected, column predicted) or NULL
     int store_p;   // write the activated outputs (softmax probabilities) back into P
 };
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s);

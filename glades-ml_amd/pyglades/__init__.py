@@ -22,6 +22,7 @@ EXPORTS = [
     "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact",
     "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
+    "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
     "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
     "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
 ]
@@ -47,6 +48,11 @@ class Spec(C.Structure):
 
 class Metrics(C.Structure):
     _fields_ = [("loss", C.c_float), ("accuracy", C.c_float), ("correct", C.c_int64)]
+
+
+class ClassMetrics(C.Structure):
+    _fields_ = [("accuracy", C.c_float), ("precision", C.c_float), ("recall", C.c_float),
+                ("specificity", C.c_float), ("f1", C.c_float)]
 
 
 class GladesHipError(RuntimeError):
@@ -78,6 +84,10 @@ def load():
             "ghip_net_forward": (i, [vp, vp, i, vp]),
             "ghip_net_forward_resident": (i, [vp, i64, i, vp]),
             "ghip_net_eval_resident": (i, [vp, i64, i, C.POINTER(Metrics)]),
+            "ghip_net_confusion_enable": (i, [vp, i]),
+            "ghip_net_confusion_reset": (i, [vp]),
+            "ghip_net_confusion_get": (i, [vp, vp, i64]),
+            "ghip_net_class_metrics": (i, [vp, i, C.POINTER(ClassMetrics)]),
             "ghip_net_quantize_fp8": (i, [vp, vp, vp]),
             "ghip_net_sync": (i, [vp]),
             "ghip_net_profile": (i, [vp, i]),
@@ -189,6 +199,24 @@ class Net:
                                                   C.cast(ms, C.c_void_p), C.byref(ran), _ptr(preds)))
         out = [(ms[k].loss, ms[k].accuracy, ms[k].correct) for k in range(ran.value)]
         return out, preds
+
+    # ---- confusion matrix
+    def confusion_enable(self, enable=True):
+        _check(self.lib.ghip_net_confusion_enable(self.h, 1 if enable else 0))
+
+    def confusion_reset(self):
+        _check(self.lib.ghip_net_confusion_reset(self.h))
+
+    def confusion(self):
+        n = self.sizes[-1]
+        M = np.zeros((n, n), np.int32)
+        _check(self.lib.ghip_net_confusion_get(self.h, _ptr(M), n * n))
+        return M
+
+    def class_metrics(self, epoch):
+        m = ClassMetrics()
+        _check(self.lib.ghip_net_class_metrics(self.h, epoch, C.byref(m)))
+        return np.array([m.accuracy, m.precision, m.recall, m.specificity, m.f1], np.float32)
 
     # ---- canonical mode
     def train_step(self, row0, batch, want_metrics=True):

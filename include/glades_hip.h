@@ -141,6 +141,27 @@ int ghip_net_forward_resident(ghip_net* net, int64_t row0, int batch, float* dev
  * resident table: forward and metrics, no parameter changes. */
 int ghip_net_eval_resident(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);
 
+/* Confusion matrix on the device: replaces CMatrix::addResult per sample (ML/GMath/cmatrix.cpp:57-98,
+ * called from network.cpp:420-423) with counters the kernels that already compute both argmaxes
+ * bump, so no prediction leaves the device for it.  n_out x n_out int32, row = expected class,
+ * column = predicted class, both under the argmax rule of gmath.cpp:412-455 (a row with no
+ * positive entry has no class and counts nowhere).
+ * enable != 0 allocates and zeroes the counters; 0 frees them.
+ * exact mode: the counters restart at every epoch (CMatrix::reset, network.cpp:183-185), so after
+ *   ghip_net_run_epochs_exact they hold the last epoch run; ghip_net_class_metrics returns the
+ *   overall accuracy / precision / recall / specificity / F1 of epoch `epoch` of that call
+ *   (CMatrix::updateResultParams + getOverall*, cmatrix.cpp:100-265; network.cpp:218-224), as
+ *   fractions, computed on the device at the epoch's end (n_out <= 64).
+ * canonical mode: ghip_net_train_step / ghip_net_eval_resident add to the counters until
+ *   ghip_net_confusion_reset. */
+typedef struct {
+    float accuracy, precision, recall, specificity, f1;
+} ghip_class_metrics;
+int ghip_net_confusion_enable(ghip_net* net, int enable);
+int ghip_net_confusion_reset(ghip_net* net);
+int ghip_net_confusion_get(ghip_net* net, int32_t* host_matrix, int64_t len);
+int ghip_net_class_metrics(ghip_net* net, int epoch, ghip_class_metrics* host_out);
+
 /* GHIP_FP8_INFER: quantises the current fp32 weights to e4m3 with one fp32 scale per output
  * channel (scale = amax(row)/448).  host_scales[l] (may be NULL) receives sizes[l+1] scales and
  * host_codes[l] (may be NULL) the sizes[l+1]*sizes[l] code bytes.  No reference counterpart (the

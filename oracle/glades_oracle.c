@@ -113,6 +113,62 @@ int go_argmax_ref(const float* v, int n)
     return idx;
 }
 
+/* ------------------------------------------------------------------ confusion matrix */
+
+/* ML/GMath/cmatrix.cpp:57-98: both vectors go through the argmax rule above (a 0/1 vector with
+ * at most one 1); for the expected class i (if any) row i gains the predicted 0/1 vector, i.e.
+ * M[i][j] += 1 for the predicted class j (if any).  Row = expected, column = predicted. */
+void go_cmatrix_add(int n, int32_t* M, const float* expected, const float* predicted)
+{
+    const int i = go_argmax_ref(expected, n);
+    const int j = go_argmax_ref(predicted, n);
+    if (i >= 0 && j >= 0) M[(int64_t)i * n + j] += 1;
+}
+
+/* ML/GMath/cmatrix.cpp:100-132, starting from the zeroed lists reset() leaves (:285-298).
+ * Off-diagonal cells feed falsePositive[col] and falseNegative[row]; a diagonal cell sets
+ * truePositive[row] and is ADDED to trueNegative of every other class, so trueNegative[i] is the
+ * sum of the other classes' diagonal cells only (off-diagonal cells never count as negatives). */
+void go_cmatrix_params(int n, const int32_t* M, int32_t* tp, int32_t* tn, int32_t* fp, int32_t* fn)
+{
+    for (int i = 0; i < n; ++i) tp[i] = tn[i] = fp[i] = fn[i] = 0;
+    for (int row = 0; row < n; ++row)
+        for (int col = 0; col < n; ++col) {
+            const int32_t v = M[(int64_t)row * n + col];
+            if (row != col) {
+                fp[col] += v;
+                fn[row] += v;
+            } else {
+                for (int itr = 0; itr < n; ++itr) {
+                    if (itr == row) tp[itr] = v;
+                    else tn[itr] += v;
+                }
+            }
+        }
+}
+
+/* ML/GMath/cmatrix.cpp:139-265: per-class ratios in float, overall = mean over the classes
+ * accumulated in class order (0/0 gives NaN and poisons the mean, as in the reference).
+ * out[0..5] = accuracy, precision, recall, specificity, F1, false alarm (fractions, not percent) */
+void go_cmatrix_overall(int n, const int32_t* tp, const int32_t* tn, const int32_t* fp, const int32_t* fn, float* out)
+{
+    float acc = 0.0f, pre = 0.0f, rec = 0.0f, spe = 0.0f, f1 = 0.0f, fa = 0.0f;
+    for (int i = 0; i < n; ++i) {
+        const float truth = (float)(tp[i] + tn[i]);
+        const float untruth = (float)(fp[i] + fn[i]);
+        acc += truth / (truth + untruth);
+        const float cp = ((float)tp[i]) / ((float)(tp[i] + fp[i]));
+        const float cr = ((float)tp[i]) / ((float)(tp[i] + fn[i]));
+        pre += cp;
+        rec += cr;
+        spe += ((float)tn[i]) / ((float)(tn[i] + fp[i]));
+        fa += ((float)fp[i]) / ((float)(tn[i] + fp[i]));
+        f1 += (2.0f * cr * cp) / (cr + cp);
+    }
+    const float nn = (float)n;
+    out[0] = acc / nn; out[1] = pre / nn; out[2] = rec / nn; out[3] = spe / nn; out[4] = f1 / nn; out[5] = fa / nn;
+}
+
 /* ------------------------------------------------------------------ init sampler */
 
 /* ML/GMath/gmath.cpp:355-405 (Acklam).  log/sqrt on float arguments are the float

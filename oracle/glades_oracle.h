@@ -40,6 +40,10 @@
  *       training, softmax or per-channel bias): pinned against torch autograd +
  *       torch.optim.SGD and finite differences; forward pinned against go_exact
  *       forward (bit-exact for equal parameters).
+ *   go_cmatrix_*  ML/GMath/cmatrix.cpp needs the un-vendored shmea containers and cannot be
+ *       compiled here: restated from the source text -- parity unpinned by execution; pinned
+ *       by hand-computed matrices, the perfect-classifier closed form and brute force on
+ *       tiny inputs (tests/test_oracle_cmatrix.py).
  *   go_bf16_* / go_e4m3_*  format conversions: pinned against torch's bf16 /
  *       float8_e4m3fn casts, exhaustive over all 256 e4m3 codes.
  */
@@ -86,6 +90,12 @@ float go_cost(float expect, float pred, float data_size, int cost);
 float go_cost_der(float expect, float pred, int cost);
 float go_percent_error(float pred, float expect);
 int   go_argmax_ref(const float* v, int n);  /* -1 when no element is > 0 */
+
+/* confusion matrix, ML/GMath/cmatrix.cpp: M is n x n int32 row-major (row expected, column predicted) */
+void go_cmatrix_add(int n, int32_t* M, const float* expected, const float* predicted);
+void go_cmatrix_params(int n, const int32_t* M, int32_t* tp, int32_t* tn, int32_t* fp, int32_t* fn);
+/* out[6]: overall accuracy, precision, recall, specificity, F1, false alarm (fractions) */
+void go_cmatrix_overall(int n, const int32_t* tp, const int32_t* tn, const int32_t* fp, const int32_t* fn, float* out);
 
 /* ---- the reference's weight sampler (layer.cpp:196-217, node.cpp:241-276); uses libc rand() ---- */
 void  go_ref_xavier_layer(int fan_in, int n_out, int act_type, float* W /* n_out*fan_in */);

@@ -56,6 +56,7 @@ def lib():
         L = C.CDLL(LIB_PATH)
         f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
         u8p = np.ctypeslib.ndpointer(np.uint8, flags="C_CONTIGUOUS")
+        i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
         vp = C.c_void_p
         sig = {
             "go_squash": (C.c_float, [C.c_float, C.c_int, C.c_float]),
@@ -64,6 +65,9 @@ def lib():
             "go_cost_der": (C.c_float, [C.c_float, C.c_float, C.c_int]),
             "go_percent_error": (C.c_float, [C.c_float, C.c_float]),
             "go_argmax_ref": (C.c_int, [f32p, C.c_int]),
+            "go_cmatrix_add": (None, [C.c_int, i32p, f32p, f32p]),
+            "go_cmatrix_params": (None, [C.c_int, i32p, i32p, i32p, i32p, i32p]),
+            "go_cmatrix_overall": (None, [C.c_int, i32p, i32p, i32p, i32p, f32p]),
             "go_ref_xavier_layer": (None, [C.c_int, C.c_int, C.c_int, f32p]),
             "go_exact_create": (vp, [C.POINTER(Spec)]),
             "go_exact_destroy": (None, [vp]),
@@ -311,3 +315,26 @@ def ref_train(spec, weights, biases, X, Y, epochs, tmpdir):
         pos += 2 * cnt
     assert pos == raw.size
     return out
+
+
+def cmatrix(expected, predicted):
+    """Confusion matrix of the reference (row expected, column predicted) over the rows of two [N][n] arrays."""
+    expected = np.ascontiguousarray(expected, np.float32)
+    predicted = np.ascontiguousarray(predicted, np.float32)
+    n = expected.shape[1]
+    M = np.zeros((n, n), np.int32)
+    for e, p in zip(expected, predicted):
+        lib().go_cmatrix_add(n, M, np.ascontiguousarray(e), np.ascontiguousarray(p))
+    return M
+
+
+def cmatrix_metrics(M):
+    """(tp, tn, fp, fn, overall[6]) of cmatrix.cpp for an n x n int32 matrix."""
+    M = np.ascontiguousarray(M, np.int32)
+    n = M.shape[0]
+    tp, tn, fp, fn = (np.zeros(n, np.int32) for _ in range(4))
+    lib().go_cmatrix_params(n, M, tp, tn, fp, fn)
+    out = np.zeros(6, np.float32)
+    with np.errstate(all="ignore"):
+        lib().go_cmatrix_overall(n, tp, tn, fp, fn, out)
+    return tp, tn, fp, fn, out
