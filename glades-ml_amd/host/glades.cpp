@@ -326,14 +326,16 @@ static int64_t g_next_id = 1;
 
 NNetwork::NNetwork()
     : di(NULL), skeleton(NULL), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
-      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallCorrect(0),
+      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
+      overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
       minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
 {
 }
 
 NNetwork::NNetwork(NNInfo* newNNInfo)
     : di(NULL), skeleton(newNNInfo), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
-      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallCorrect(0),
+      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
+      overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
       minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
 {
 }
@@ -449,7 +451,149 @@ bool NNetwork::build()
         if (ghip_net_set_params(dev, l, W.data(), bp, bl) != 0) { lastError = ghip_last_error(); return false; }
     }
     if (ghip_net_set_dataset(dev, X.data(), Y.data(), (int64_t)nRows) != 0) { lastError = ghip_last_error(); return false; }
+    // network.cpp:143-145: classification and KL runs keep a confusion matrix (counted on the device)
+    confusionMatrix.clean();
+    if ((s.cost == GMath::CLASSIFICATION || s.cost == GMath::KL) && nOut <= 4096) {
+        if (ghip_net_confusion_enable(dev, 1) != 0) { lastError = ghip_last_error(); return false; }
+        confusionMatrix.build(nOut);
+    }
     return true;
+}
+
+// ------------------------------------------------------------------ CMatrix (ML/GMath/cmatrix.cpp)
+
+void CMatrix::build(unsigned int numberOfClasses)
+{
+    clean();
+    n = numberOfClasses;
+    matrix.assign((size_t)n * n, 0);
+    truePositive.assign(n, 0); trueNegative.assign(n, 0); falsePositive.assign(n, 0); falseNegative.assign(n, 0);
+}
+
+static int naiveArgmax(const std::vector<float>& v)  // gmath.cpp:412-433
+{
+    float mx = 0.0f;
+    int index = -1;
+    for (size_t i = 0; i < v.size(); ++i)
+        if (v[i] > mx) { mx = v[i]; index = (int)i; }
+    return index;
+}
+
+void CMatrix::addResult(const std::vector<float>& result)  // cmatrix.cpp:57-98
+{
+    if ((result.size() % 2) != 0) { printf("[CMATRIX] Bad result list size [0]: %d\n", (int)result.size()); return; }
+    if ((result.size() / 2) != n) { printf("[CMATRIX] Bad result list size [1]: %d\n", (int)result.size()); return; }
+    std::vector<float> expected, predicted;
+    for (size_t i = 0; i < result.size(); ++i) ((i % 2) == 0 ? expected : predicted).push_back(result[i]);
+    const int e = naiveArgmax(expected), p = naiveArgmax(predicted);
+    if (e >= 0 && p >= 0) matrix[(size_t)e * n + p] += 1;
+}
+
+void CMatrix::setMatrix(const std::vector<int>& cells)
+{
+    if (cells.size() == matrix.size()) matrix = cells;
+}
+
+void CMatrix::updateResultParams()  // cmatrix.cpp:100-132 (the lists are NOT cleared here, as there)
+{
+    const int size = (int)n;
+    for (int row = 0; row < size; ++row)
+        for (int col = 0; col < size; ++col) {
+            const int value = matrix[(size_t)row * n + col];
+            if (row != col) {
+                falsePositive[col] += value;
+                falseNegative[row] += value;
+            } else {
+                for (int itr = 0; itr < size; ++itr) {
+                    if (itr == row) truePositive[itr] = value;
+                    else trueNegative[itr] += value;
+                }
+            }
+        }
+}
+
+std::vector<std::vector<int> > CMatrix::getMatrix() const
+{
+    std::vector<std::vector<int> > out(n, std::vector<int>(n, 0));
+    for (unsigned int r = 0; r < n; ++r)
+        for (unsigned int c = 0; c < n; ++c) out[r][c] = matrix[(size_t)r * n + c];
+    return out;
+}
+
+// the reference's guard is `index > rows` (cmatrix.cpp:141); index == rows is rejected here as well
+float CMatrix::getClassAccuracy(unsigned int i) const
+{
+    if (i >= n) return 0.0f;
+    const float truth = (float)(truePositive[i] + trueNegative[i]);
+    const float untruth = (float)(falsePositive[i] + falseNegative[i]);
+    return truth / (truth + untruth);
+}
+float CMatrix::getClassPrecision(unsigned int i) const
+{
+    if (i >= n) return 0.0f;
+    return ((float)truePositive[i]) / ((float)(truePositive[i] + falsePositive[i]));
+}
+float CMatrix::getClassRecall(unsigned int i) const
+{
+    if (i >= n) return 0.0f;
+    return ((float)truePositive[i]) / ((float)(truePositive[i] + falseNegative[i]));
+}
+float CMatrix::getClassSpecificity(unsigned int i) const
+{
+    if (i >= n) return 0.0f;
+    return ((float)trueNegative[i]) / ((float)(trueNegative[i] + falsePositive[i]));
+}
+float CMatrix::getClassFalseAlarm(unsigned int i) const
+{
+    if (i >= n) return 0.0f;
+    return ((float)falsePositive[i]) / ((float)(trueNegative[i] + falsePositive[i]));
+}
+float CMatrix::getClassF1Score(unsigned int i) const
+{
+    if (i >= n) return 0.0f;
+    const float cRecall = getClassRecall(i), cPrecision = getClassPrecision(i);
+    return (2.0f * cRecall * cPrecision) / (cRecall + cPrecision);
+}
+#define GLADES_OVERALL(NAME, CLASSFN)                          \
+    float CMatrix::NAME() const                                \
+    {                                                          \
+        float total = 0.0f;                                    \
+        for (unsigned int i = 0; i < n; ++i) total += CLASSFN(i); \
+        total /= ((float)n);                                   \
+        return total;                                          \
+    }
+GLADES_OVERALL(getOverallAccuracy, getClassAccuracy)
+GLADES_OVERALL(getOverallPrecision, getClassPrecision)
+GLADES_OVERALL(getOverallRecall, getClassRecall)
+GLADES_OVERALL(getOverallSpecificity, getClassSpecificity)
+GLADES_OVERALL(getOverallFalseAlarm, getClassFalseAlarm)
+GLADES_OVERALL(getOverallF1Score, getClassF1Score)
+#undef GLADES_OVERALL
+
+void CMatrix::print() const
+{
+    printf("[CMATRIX] Confusion Matrix...\n");
+    for (unsigned int r = 0; r < n; ++r) {
+        for (unsigned int c = 0; c < n; ++c) printf("%d%s", matrix[(size_t)r * n + c], c + 1 < n ? "," : "\n");
+    }
+    const char* names[4] = {"True Positives", "True Negatives", "False Positives", "False Negatives"};
+    const std::vector<int>* lists[4] = {&truePositive, &trueNegative, &falsePositive, &falseNegative};
+    for (int k = 0; k < 4; ++k) {
+        printf("[CMATRIX] %s...\n", names[k]);
+        for (unsigned int i = 0; i < n; ++i) printf("%d%s", (*lists[k])[i], i + 1 < n ? "," : "\n");
+    }
+}
+
+void CMatrix::reset()  // cmatrix.cpp:285-298: keeps the shape
+{
+    matrix.assign((size_t)n * n, 0);
+    truePositive.assign(n, 0); trueNegative.assign(n, 0); falsePositive.assign(n, 0); falseNegative.assign(n, 0);
+}
+
+void CMatrix::clean()
+{
+    n = 0;
+    matrix.clear(); truePositive.clear(); trueNegative.clear(); falsePositive.clear(); falseNegative.clear();
 }
 
 // NNetwork::run (ML/Networks/network.cpp:114-397)
@@ -499,6 +643,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             overallTotalAccuracy = ms[ran - 1].accuracy;
             overallCorrect = ms[ran - 1].correct;
         } else {
+            if (confusionMatrix.size() > 0) ghip_net_confusion_reset(dev);  // network.cpp:183-185
             // canonical mode: batches [k*mb, (k+1)*mb), the last one averaged over its true size
             const int mb = minibatchSize > 0 ? minibatchSize : (int)nRows;
             double loss = 0.0, acc = 0.0;
@@ -517,8 +662,27 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             overallTotalAccuracy = (float)(acc / nRows);
             overallCorrect = correct;
         }
+        const bool classes = confusionMatrix.size() > 0;
+        if (classes) {
+            // network.cpp:218-224: the device counted the last epoch's cells; the ratios are CMatrix's
+            std::vector<int> cells((size_t)nOut * nOut);
+            if (ghip_net_confusion_get(dev, cells.data(), (int64_t)cells.size()) == 0) {
+                confusionMatrix.reset();
+                confusionMatrix.setMatrix(cells);
+                confusionMatrix.updateResultParams();
+                overallClassAccuracy = confusionMatrix.getOverallAccuracy() * 100.0f;
+                overallClassPrecision = confusionMatrix.getOverallPrecision() * 100.0f;
+                overallClassRecall = confusionMatrix.getOverallRecall() * 100.0f;
+                overallClassSpecificity = confusionMatrix.getOverallSpecificity() * 100.0f;
+                overallClassF1 = confusionMatrix.getOverallF1Score() * 100.0f;
+            }
+        }
         if (runType == RUN_TRAIN) {
-            printf("\33[2K[NN] %d\t%f%%\r", epochs, overallTotalAccuracy);
+            if (classes)
+                printf("\33[2K[NN] %d\t%s%f%%\t%f%%\t%f%%\t%f%%\t%f%%\r", epochs, epochs < 100 ? "\t" : "", overallClassAccuracy,
+                       overallClassPrecision, overallClassRecall, overallClassSpecificity, overallClassF1);
+            else
+                printf("\33[2K[NN] %d\t%f%%\r", epochs, overallTotalAccuracy);
             fflush(stdout);
         }
         if (terminator.triggered(time(NULL), epochs, overallTotalAccuracy)) break;

@@ -11,6 +11,7 @@
 //   NNInfo                 ML/Structure/nninfo.h:41-127 (index-shifted getters: nninfo.cpp:240-373)
 //   Terminator             ML/State/Terminator.h:27-51
 //   DataInput              ML/DataObjects/DataInput.h:26-50
+//   CMatrix                ML/GMath/cmatrix.h:27-67
 //   NNetwork               ML/Networks/network.h:59-141
 //   MetaNetwork            ML/Networks/metanetwork.h:44-64
 //   glades::init/train/test  ML/main.h:44-54
@@ -213,6 +214,43 @@ public:
     void denseTrain(std::vector<float>& x, std::vector<float>& y, unsigned int& nOut) const;
 };
 
+// Confusion matrix of a classification run (ML/GMath/cmatrix.cpp).  Row = expected class, column =
+// predicted class, both chosen by the strictly-greater-than scan from 0 of GMath::naiveVectorDecomp
+// (gmath.cpp:412-455).  The GTable / GLists of the reference are plain int vectors here.  During a
+// run the cells are counted on the device and copied in with setMatrix(); addResult() is the
+// host-side form for callers that feed (expected, predicted) pairs themselves.
+class CMatrix
+{
+    unsigned int n;
+    std::vector<int> matrix;  // n x n, row-major
+    std::vector<int> truePositive, trueNegative, falsePositive, falseNegative;
+
+public:
+    CMatrix() : n(0) {}
+    void build(unsigned int numberOfClasses);
+    void addResult(const std::vector<float>& result);  // e0, p0, e1, p1, ... (network.cpp:529-530)
+    void setMatrix(const std::vector<int>& cells);     // n x n cells counted elsewhere
+    void updateResultParams();
+    std::vector<std::vector<int> > getMatrix() const;
+    int getCell(unsigned int row, unsigned int col) const { return matrix[(size_t)row * n + col]; }
+    unsigned int size() const { return n; }
+    float getClassAccuracy(unsigned int) const;
+    float getOverallAccuracy() const;
+    float getClassPrecision(unsigned int) const;
+    float getOverallPrecision() const;
+    float getClassRecall(unsigned int) const;
+    float getOverallRecall() const;
+    float getClassSpecificity(unsigned int) const;
+    float getOverallSpecificity() const;
+    float getClassFalseAlarm(unsigned int) const;
+    float getOverallFalseAlarm() const;
+    float getClassF1Score(unsigned int) const;
+    float getOverallF1Score() const;
+    void print() const;
+    void reset();
+    void clean();
+};
+
 class MetaNetwork;
 
 class NNetwork
@@ -224,6 +262,8 @@ class NNetwork
     volatile bool running;
     int netType, epochs, mode, dtype, biasMode;
     float overallTotalError, overallTotalAccuracy;
+    float overallClassAccuracy, overallClassPrecision, overallClassRecall, overallClassSpecificity, overallClassF1;
+    CMatrix confusionMatrix;
     int64_t overallCorrect;
     int minibatchSize;
     int64_t id;
@@ -267,6 +307,14 @@ public:
     // ---- absent from the reference (its loss has no getter and its weights are not reachable)
     float getLoss() const { return overallTotalError; }
     int64_t getCorrect() const { return overallCorrect; }
+    // the five figures of the reference's progress line (network.cpp:218-224), in percent, and the matrix
+    // behind them (private members without getters in the reference)
+    float getClassAccuracy() const { return overallClassAccuracy; }
+    float getClassPrecision() const { return overallClassPrecision; }
+    float getClassRecall() const { return overallClassRecall; }
+    float getClassSpecificity() const { return overallClassSpecificity; }
+    float getClassF1() const { return overallClassF1; }
+    const CMatrix& getConfusionMatrix() const { return confusionMatrix; }
     void setMode(int newMode, int newDtype = DTYPE_F32) { mode = newMode; dtype = newDtype; }
     void setSequentialBias(bool faithful) { biasMode = faithful ? 0 : 1; }
     // layer = weight layer 0..numHiddenLayers(); W is [n_out][n_in] row-major

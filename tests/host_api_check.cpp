@@ -5,6 +5,7 @@
 //
 //   host_api_check xavier <seed> <fan_in> <n_out> <act> <out.bin>        (no GPU needed)
 //   host_api_check nninfo <table.csv> <resaved.csv>                      (no GPU needed)
+//   host_api_check cmatrix <n> <pairs.bin> <out.bin>                     (no GPU needed)
 //   host_api_check train  <case.bin> <out.bin> <stop_epoch> <stop_accuracy> <mode>
 #include <stdio.h>
 #include <stdlib.h>
@@ -39,6 +40,28 @@ static int do_nninfo(const char* path, const char* resave)
                s->getWeightDecay1(i), s->getWeightDecay2(i), s->getPDropout(i), s->getActivationType(i), s->getActivationParam(i));
     for (int i = 0; i < s->numHiddenLayers(); ++i) printf("hsize %d %d\n", i, s->getHiddenLayerSize(i));
     return net.save(resave) ? 0 : 2;
+}
+
+// pairs.bin: rows of n (expected, predicted) float pairs, interleaved as NNetwork's results list holds them
+static int do_cmatrix(int n, const char* in, const char* out)
+{
+    FILE* f = fopen(in, "rb");
+    if (!f) return 1;
+    CMatrix cm;
+    cm.build(n);
+    std::vector<float> row(2 * n);
+    while (fread(row.data(), 4, row.size(), f) == row.size()) cm.addResult(row);
+    fclose(f);
+    cm.updateResultParams();
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    for (int r = 0; r < n; ++r)
+        for (int c = 0; c < n; ++c) { float v = (float)cm.getCell(r, c); fwrite(&v, 4, 1, fo); }
+    float ov[6] = {cm.getOverallAccuracy(), cm.getOverallPrecision(), cm.getOverallRecall(), cm.getOverallSpecificity(),
+                   cm.getOverallF1Score(), cm.getOverallFalseAlarm()};
+    fwrite(ov, 4, 6, fo);
+    fclose(fo);
+    return 0;
 }
 
 static int do_train(const char* in, const char* out, long stop_epoch, float stop_acc, int mode)
@@ -95,6 +118,15 @@ static int do_train(const char* in, const char* out, long stop_epoch, float stop
     const int trained = net.getEpochs();
     const float acc = net.getAccuracy(), loss = net.getLoss();
     std::vector<float> results = net.getResults();
+    // the class figures of the last training epoch (network.cpp:218-224) and the matrix behind them
+    const CMatrix& cm = net.getConfusionMatrix();
+    std::vector<float> tail(1, (float)cm.size());
+    if (cm.size() > 0) {
+        const float five[5] = {net.getClassAccuracy(), net.getClassPrecision(), net.getClassRecall(), net.getClassSpecificity(), net.getClassF1()};
+        tail.insert(tail.end(), five, five + 5);
+        for (unsigned int r = 0; r < cm.size(); ++r)
+            for (unsigned int c = 0; c < cm.size(); ++c) tail.push_back((float)cm.getCell(r, c));
+    }
     glades::test(&net, &di);   // RUN_TEST pass: one more epoch counted, parameters untouched
     FILE* fo = fopen(out, "wb");
     if (!fo) return 1;
@@ -109,6 +141,7 @@ static int do_train(const char* in, const char* out, long stop_epoch, float stop
         std::vector<float> b = net.getBias(l);
         fwrite(b.data(), 4, b.size(), fo);
     }
+    fwrite(tail.data(), 4, tail.size(), fo);
     fclose(fo);
     delete meta;
     return 0;
@@ -118,6 +151,7 @@ int main(int argc, char** argv)
 {
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
+    if (argc >= 5 && !strcmp(argv[1], "cmatrix")) return do_cmatrix(atoi(argv[2]), argv[3], argv[4]);
     if (argc >= 7 && !strcmp(argv[1], "train")) return do_train(argv[2], argv[3], atol(argv[4]), (float)atof(argv[5]), atoi(argv[6]));
     fprintf(stderr, "usage: see the header of host_api_check.cpp\n");
     return 64;

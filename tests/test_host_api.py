@@ -49,6 +49,28 @@ def test_nninfo_table_round_trip_and_index_shift():
         assert open(dst).read() == table
 
 
+@needs_bin
+def test_cmatrix_class_matches_restatement():
+    """CMatrix::addResult / updateResultParams / getOverall* fed with (expected, predicted) pairs."""
+    rng = np.random.default_rng(9)
+    n, N = 4, 300
+    E = np.eye(n, dtype=np.float32)[rng.integers(0, n, N)] * 0.98 + 0.01
+    P = rng.random((N, n)).astype(np.float32)
+    E[5] = 0.0   # no expected class
+    P[9] = -1.0  # no predicted class
+    pairs = np.empty((N, 2 * n), np.float32)
+    pairs[:, 0::2], pairs[:, 1::2] = E, P
+    with tempfile.TemporaryDirectory() as td:
+        fin, fout = os.path.join(td, "p.bin"), os.path.join(td, "o.bin")
+        pairs.tofile(fin)
+        subprocess.check_call([BIN, "cmatrix", str(n), fin, fout])
+        raw = np.fromfile(fout, np.float32)
+    M = raw[:n * n].reshape(n, n).astype(np.int32)
+    want_M = po.cmatrix(E, P)
+    assert np.array_equal(M, want_M) and M.sum() == N - 2
+    assert bits_equal(raw[n * n:], po.cmatrix_metrics(want_M)[4])
+
+
 def write_case(path, c, wd2_layer0_from_wd1=True):
     s = c["spec"]
     nl = c["nl"]
@@ -82,8 +104,13 @@ def read_out(path, c, exact=True):
         k = 1 if exact else c["sizes"][l + 1]
         bs.append(raw[pos:pos + k])
         pos += k
+    ncls = int(raw[pos]); pos += 1
+    cls = None
+    if ncls > 0:
+        cls = (raw[pos:pos + 5], raw[pos + 5:pos + 5 + ncls * ncls].reshape(ncls, ncls).astype(np.int32))
+        pos += 5 + ncls * ncls
     assert pos == raw.size
-    return head, res, Ws, bs
+    return head, res, Ws, bs, cls
 
 
 @needs_bin
@@ -99,7 +126,7 @@ def test_train_through_class_api_matches_fixture(name):
         cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
         write_case(cin, c)
         subprocess.check_call([BIN, "train", cin, cout, str(c["epochs"]), "0", "0"], stdout=subprocess.DEVNULL)
-        head, res, Ws, bs = read_out(cout, c)
+        head, res, Ws, bs, cls = read_out(cout, c)
     d = c["d"]
     assert int(head[0]) == c["epochs"] and int(head[3]) == c["epochs"] + 1   # test() counts one more epoch
     np.testing.assert_allclose(head[1], d["epochs"][-1, 1], rtol=1e-4)
@@ -110,6 +137,17 @@ def test_train_through_class_api_matches_fixture(name):
         np.testing.assert_allclose(Ws[l], d[f"W_{l}"], rtol=1e-4, atol=1e-4 * np.abs(d[f"W_{l}"]).max())
         if l >= 1:
             np.testing.assert_allclose(bs[l][0], d["bias"][l], rtol=1e-4, atol=1e-7)
+    if c["cost"] != po.REGRESSION:
+        # confusion matrix and class figures of the last training epoch: counted on the device,
+        # ratios by the CMatrix class; against the restatement on the fixture's last-epoch predictions
+        want_M = po.cmatrix(c["Y"], d["preds"])
+        assert cls is not None and np.array_equal(cls[1], want_M)
+        want = po.cmatrix_metrics(want_M)[4][:5] * np.float32(100.0)
+        assert np.array_equal(np.isnan(cls[0]), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert np.array_equal(cls[0][ok], want[ok])
+    else:
+        assert cls is None
     # the RUN_TEST pass afterwards evaluates the trained weights
     o = po.ExactNet(c["spec"])
     for l in range(c["nl"]):
@@ -129,7 +167,7 @@ def test_terminator_accuracy_stops_training():
         cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
         write_case(cin, c)
         subprocess.check_call([BIN, "train", cin, cout, "100000", repr(target), "0"], stdout=subprocess.DEVNULL)
-        head, _, _, _ = read_out(cout, c)
+        head, _, _, _, _ = read_out(cout, c)
     assert int(head[0]) == first
     assert head[1] >= target
 
@@ -156,7 +194,7 @@ def test_canonical_mode_through_class_api():
         cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
         write_case(cin, c)
         subprocess.check_call([BIN, "train", cin, cout, str(epochs), "0", "1"], stdout=subprocess.DEVNULL)
-        head, _, Ws, bs = read_out(cout, c, exact=False)
+        head, _, Ws, bs, _ = read_out(cout, c, exact=False)
     assert int(head[0]) == epochs
     for l in range(2):
         Wo, bo = o.get_params(l)
