@@ -460,6 +460,210 @@ bool NNetwork::build()
     return true;
 }
 
+// ------------------------------------------------------------------ OHE (ML/GMath/OHE.cpp)
+
+void OHE::addString(const std::string& newString)  // OHE.cpp:54-64
+{
+    const int at = indexAt(newString);
+    if (at < 0) { OHEStrings.push_back(newString); classCount.push_back(1); }
+    else ++classCount[at];
+}
+bool OHE::contains(const std::string& s) const { return indexAt(s) >= 0; }
+int OHE::indexAt(const std::string& needle) const
+{
+    for (size_t i = 0; i < OHEStrings.size(); ++i)
+        if (OHEStrings[i] == needle) return (int)i;
+    return -1;
+}
+std::string OHE::classAt(unsigned int cid) const { return cid < OHEStrings.size() ? OHEStrings[cid] : std::string(); }
+std::vector<float> OHE::operator[](const std::string& needle) const  // OHE.cpp:179-198
+{
+    std::vector<float> retVal(size(), 0.01f);
+    const int at = indexAt(needle);
+    if (at >= 0) retVal[at] = 0.99f;
+    return retVal;
+}
+std::string OHE::operator[](const std::vector<float>& needle) const  // OHE.cpp:216-238: >= scan from 0
+{
+    float max = 0.0f;
+    int index = -1;
+    for (size_t i = 0; i < needle.size(); ++i)
+        if (needle[i] >= max) { max = needle[i]; index = (int)i; }
+    return (index >= 0 && (size_t)index < OHEStrings.size()) ? OHEStrings[index] : std::string();
+}
+
+// ------------------------------------------------------------------ NumberInput (ML/DataObjects/NumberInput.cpp)
+
+namespace {
+std::string trimmed(const std::string& s)
+{
+    size_t a = 0, b = s.size();
+    while (a < b && (s[a] == ' ' || s[a] == '\t' || s[a] == '\r' || s[a] == '\n')) ++a;
+    while (b > a && (s[b - 1] == ' ' || s[b - 1] == '\t' || s[b - 1] == '\r' || s[b - 1] == '\n')) --b;
+    return s.substr(a, b - a);
+}
+std::vector<std::string> splitLine(const std::string& line)
+{
+    std::vector<std::string> out;
+    size_t start = 0;
+    for (;;) {
+        size_t c = line.find(',', start);
+        out.push_back(trimmed(line.substr(start, c == std::string::npos ? std::string::npos : c - start)));
+        if (c == std::string::npos) break;
+        start = c + 1;
+    }
+    return out;
+}
+bool parseNumber(const std::string& cell, float* v)
+{
+    if (cell.empty()) return false;
+    char* end = NULL;
+    const float f = strtof(cell.c_str(), &end);
+    if (end == cell.c_str() || *end != '\0') return false;
+    *v = f;
+    return true;
+}
+}  // namespace
+
+void NumberInput::import(std::string fname)
+{
+    if (loaded) return;
+    name = fname;
+    standardizeInputTable(fname);
+    loaded = true;
+}
+
+bool NumberInput::standardizeInputTable(const std::string& fname, int standardizeFlag)
+{
+    FILE* f = fopen(fname.c_str(), "rb");
+    if (!f) return false;
+    std::string text;
+    char buf[4096];
+    size_t got;
+    while ((got = fread(buf, 1, sizeof(buf), f)) > 0) text.append(buf, got);
+    fclose(f);
+    return standardizeText(text, standardizeFlag);
+}
+
+bool NumberInput::standardizeText(const std::string& text, int standardizeFlag)
+{
+    trainTable.clear(); trainExpectedTable.clear(); trainHeaders.clear(); expectedHeaders.clear();
+    OHEMaps.clear(); featureIsCategorical.clear(); rows = 0;
+    // ---- the table as parsed (stands in for GTable(fname, ',', TYPE_FILE))
+    std::vector<std::string> header;
+    std::vector<std::vector<std::string> > raw;
+    size_t pos = 0;
+    bool first = true;
+    while (pos <= text.size()) {
+        size_t nl = text.find('\n', pos);
+        std::string line = text.substr(pos, nl == std::string::npos ? std::string::npos : nl - pos);
+        pos = (nl == std::string::npos) ? text.size() + 1 : nl + 1;
+        if (trimmed(line).empty()) continue;
+        if (first) { header = splitLine(line); first = false; continue; }
+        std::vector<std::string> cells = splitLine(line);
+        cells.resize(header.size());
+        raw.push_back(cells);
+    }
+    const unsigned int nRows = (unsigned int)raw.size(), nCols = (unsigned int)header.size();
+    if (nRows == 0 || nCols == 0) return false;
+    std::vector<bool> isOutput(nCols, false);
+    if (outputColumns.empty()) isOutput[nCols - 1] = true;
+    for (size_t k = 0; k < outputColumns.size(); ++k)
+        if (outputColumns[k] >= 0 && (unsigned int)outputColumns[k] < nCols) isOutput[outputColumns[k]] = true;
+    std::vector<std::vector<float> > val(nRows, std::vector<float>(nCols, 0.0f));
+    std::vector<std::vector<char> > isString(nRows, std::vector<char>(nCols, 0));
+    for (unsigned int r = 0; r < nRows; ++r)
+        for (unsigned int c = 0; c < nCols; ++c) isString[r][c] = parseNumber(raw[r][c], &val[r][c]) ? 0 : 1;
+
+    std::vector<std::vector<float> > trainCols, expectedCols;  // column major while building
+    // ---- NumberInput.cpp:55-73: categorical = first cell is a string; map its feature space
+    bool isClassification = false;
+    for (unsigned int c = 0; c < nCols; ++c) {
+        OHE cOHE;
+        featureIsCategorical.push_back(false);
+        if (isString[0][c]) {
+            for (unsigned int r = 0; r < nRows; ++r)
+                if (isString[r][c]) cOHE.addString(raw[r][c]);   // OHE::mapFeatureSpace, OHE.cpp:240-258
+            featureIsCategorical[c] = true;
+            isClassification = true;
+        }
+        OHEMaps.push_back(cOHE);
+    }
+    // ---- NumberInput.cpp:75-283
+    for (unsigned int c = 0; c < nCols; ++c) {
+        float fMin = 0.0f, fMax = 0.0f, fMean = 0.0f;
+        for (unsigned int r = 0; r < nRows; ++r) {
+            if (featureIsCategorical[c]) continue;
+            if (isString[r][c]) continue;
+            const float cell = val[r][c];
+            if ((r == 0) && (c == 0)) { fMin = cell; fMax = cell; }
+            if (cell < fMin) fMin = cell;
+            if (cell > fMax) fMax = cell;
+            fMean += cell;
+            if (r == (nRows - 1)) fMean /= nRows;
+        }
+        if (featureIsCategorical[c]) {
+            const OHE& vec = OHEMaps[c];
+            for (unsigned int cInt = 0; cInt < vec.size(); ++cInt) {
+                std::vector<float> newCol(nRows);
+                for (unsigned int r = 0; r < nRows; ++r) newCol[r] = vec[raw[r][c]][cInt];
+                char num[16];
+                snprintf(num, sizeof(num), "%u", cInt);
+                if (isOutput[c]) { expectedCols.push_back(newCol); expectedHeaders.push_back(header[c] + num); }
+                else { trainCols.push_back(newCol); trainHeaders.push_back(header[c] + num); }
+            }
+            continue;
+        }
+        std::vector<float> newCol(nRows);
+        if (standardizeFlag == GMath::MINMAX) {
+            const float xRange = fMax - fMin;
+            if (xRange == 0.0f) {  // a constant: added as it is, to the feature table (:171-176)
+                for (unsigned int r = 0; r < nRows; ++r) newCol[r] = val[r][c];
+                trainCols.push_back(newCol); trainHeaders.push_back(header[c]);
+                continue;
+            }
+            for (unsigned int r = 0; r < nRows; ++r) {
+                if (isString[r][c]) {  // strings MUST be categorical (:186-192)
+                    printf("ERROR: String found in non-categorical column.\n");
+                    trainTable.clear();
+                    return false;
+                }
+                float cell = val[r][c];
+                if (isClassification) cell = ((((cell - fMin) / (xRange)) * 0.98f) + 0.01f);
+                else cell = ((cell - fMin) / (xRange));
+                newCol[r] = cell;
+            }
+        } else if (standardizeFlag == GMath::ZSCORE) {
+            float fStDev = 0.0f;
+            for (unsigned int r = 0; r < nRows; ++r) {
+                if (isString[r][c]) { trainTable.clear(); return false; }
+                const float cell = val[r][c];
+                fStDev += ((cell - fMean) * (cell - fMean));
+            }
+            fStDev = sqrtf(fStDev / (nRows - 1));
+            for (unsigned int r = 0; r < nRows; ++r) newCol[r] = ((val[r][c] - fMean) / fStDev);
+        } else {
+            continue;
+        }
+        if (isOutput[c]) { expectedCols.push_back(newCol); expectedHeaders.push_back(header[c]); }
+        else { trainCols.push_back(newCol); trainHeaders.push_back(header[c]); }
+    }
+    rows = nRows;
+    trainTable.assign(nRows, std::vector<float>(trainCols.size()));
+    trainExpectedTable.assign(nRows, std::vector<float>(expectedCols.size()));
+    for (unsigned int r = 0; r < nRows; ++r) {
+        for (size_t c = 0; c < trainCols.size(); ++c) trainTable[r][c] = trainCols[c][r];
+        for (size_t c = 0; c < expectedCols.size(); ++c) trainExpectedTable[r][c] = expectedCols[c][r];
+    }
+    return true;
+}
+
+std::vector<float> NumberInput::getTrainRow(unsigned int i) const { return i < trainTable.size() ? trainTable[i] : std::vector<float>(); }
+std::vector<float> NumberInput::getTrainExpectedRow(unsigned int i) const
+{
+    return i < trainExpectedTable.size() ? trainExpectedTable[i] : std::vector<float>();
+}
+
 // ------------------------------------------------------------------ CMatrix (ML/GMath/cmatrix.cpp)
 
 void CMatrix::build(unsigned int numberOfClasses)

@@ -12,6 +12,8 @@
 //   Terminator             ML/State/Terminator.h:27-51
 //   DataInput              ML/DataObjects/DataInput.h:26-50
 //   CMatrix                ML/GMath/cmatrix.h:27-67
+//   OHE                    ML/GMath/OHE.h:27-78
+//   NumberInput            ML/DataObjects/NumberInput.h:27-84
 //   NNetwork               ML/Networks/network.h:59-141
 //   MetaNetwork            ML/Networks/metanetwork.h:44-64
 //   glades::init/train/test  ML/main.h:44-54
@@ -212,6 +214,65 @@ public:
     unsigned int getFeatureCount() const { return feats; }
     int getType() const { return CSV; }
     void denseTrain(std::vector<float>& x, std::vector<float>& y, unsigned int& nOut) const;
+};
+
+// One-hot encoder of a string column (ML/GMath/OHE.cpp): classes in order of first appearance,
+// a class encodes as 0.99 at its index and 0.01 elsewhere (OHE.cpp:159-198).
+class OHE
+{
+    std::vector<std::string> OHEStrings;
+    std::vector<int> classCount;
+
+public:
+    void addString(const std::string&);
+    unsigned int size() const { return (unsigned int)OHEStrings.size(); }
+    std::vector<std::string> getStrings() const { return OHEStrings; }
+    bool contains(const std::string&) const;
+    int indexAt(const std::string&) const;                     // -1 if absent
+    std::string classAt(unsigned int) const;
+    std::vector<float> operator[](const std::string&) const;   // 0.99 / 0.01 vector
+    std::string operator[](const std::vector<float>&) const;   // class of the largest entry (>= scan, OHE.cpp:216-238)
+};
+
+// CSV table -> standardised training table (ML/DataObjects/NumberInput.cpp:43-285).
+// The reference reads the file with the shmea GTable parser, which is not part of its tree; this
+// class states that boundary itself: first line = header, comma separated, cells trimmed, a cell
+// is a string iff it does not parse completely as a number, the LAST column is the output column
+// (the convention its fixtures xornet / iris rely on; setOutputColumns overrides it).
+// What happens to the parsed table is the reference's: a column whose first cell is a string is
+// categorical and one-hot encoded (0.99 / 0.01); any categorical column makes the run a
+// classification; numeric columns are min-max scaled to [0.01, 0.99] (classification) or [0, 1]
+// (regression), or z-scored; the running minimum / maximum start at the first cell only for
+// column 0 and at 0 for every other column (NumberInput.cpp:103-107); a constant column goes to
+// the feature table unscaled, output column or not (:171-176).
+class NumberInput : public DataInput
+{
+    std::string name;
+    bool loaded;
+    std::vector<std::vector<float> > trainTable, trainExpectedTable;  // [row][col]
+    std::vector<std::string> trainHeaders, expectedHeaders;
+    std::vector<OHE> OHEMaps;
+    std::vector<int> outputColumns;  // empty: the last column
+    unsigned int rows;
+
+public:
+    NumberInput() : loaded(false), rows(0) {}
+    void setOutputColumns(const std::vector<int>& cols) { outputColumns = cols; }
+    void import(std::string fname);  // NumberInput.cpp:27-41: loads once
+    bool standardizeInputTable(const std::string& fname, int standardizeFlag = GMath::MINMAX);
+    bool standardizeText(const std::string& csvText, int standardizeFlag = GMath::MINMAX);
+    std::vector<float> getTrainRow(unsigned int) const;
+    std::vector<float> getTrainExpectedRow(unsigned int) const;
+    std::vector<float> getTestRow(unsigned int) const { return std::vector<float>(); }
+    std::vector<float> getTestExpectedRow(unsigned int) const { return std::vector<float>(); }
+    unsigned int getTrainSize() const { return rows; }
+    unsigned int getTestSize() const { return 0; }
+    unsigned int getFeatureCount() const { return trainTable.empty() ? 0 : (unsigned int)trainTable[0].size(); }
+    unsigned int getOutputCount() const { return trainExpectedTable.empty() ? 0 : (unsigned int)trainExpectedTable[0].size(); }
+    int getType() const { return CSV; }
+    const std::vector<OHE>& getOHEMaps() const { return OHEMaps; }
+    std::vector<std::string> getTrainHeaders() const { return trainHeaders; }
+    std::vector<std::string> getExpectedHeaders() const { return expectedHeaders; }
 };
 
 // Confusion matrix of a classification run (ML/GMath/cmatrix.cpp).  Row = expected class, column =

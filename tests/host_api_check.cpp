@@ -6,6 +6,9 @@
 //   host_api_check xavier <seed> <fan_in> <n_out> <act> <out.bin>        (no GPU needed)
 //   host_api_check nninfo <table.csv> <resaved.csv>                      (no GPU needed)
 //   host_api_check cmatrix <n> <pairs.bin> <out.bin>                     (no GPU needed)
+//   host_api_check ohe                                                   (no GPU needed)
+//   host_api_check numberinput <file.csv> <minmax|zscore> <out.bin>      (no GPU needed)
+//   host_api_check traincsv <file.csv> <nninfo table> <stop_epoch> <stop_accuracy> <seed> <out.bin> [case.bin with the initial weights]
 //   host_api_check train  <case.bin> <out.bin> <stop_epoch> <stop_accuracy> <mode>
 #include <stdio.h>
 #include <stdlib.h>
@@ -64,55 +67,92 @@ static int do_cmatrix(int n, const char* in, const char* out)
     return 0;
 }
 
-static int do_train(const char* in, const char* out, long stop_epoch, float stop_acc, int mode)
+// the assertions of the reference's own OHE unit test ("unit-tests/Backend/Machine Learning/ohe-test.cpp":17-45)
+static int do_ohe()
+{
+    OHE ohe;
+    if (ohe.size() != 0) return 1;
+    ohe.addString("cat");
+    ohe.addString("dog");
+    ohe.addString("cat");
+    if (ohe.size() != 2 || !ohe.contains("cat") || !ohe.contains("dog")) return 2;
+    std::vector<float> cat = ohe["cat"], dog = ohe["dog"];
+    if (cat.size() != 2 || dog.size() != 2) return 3;
+    if (!(cat[0] == 0.99f && cat[1] == 0.01f)) return 4;
+    if (!(dog[0] == 0.01f && dog[1] == 0.99f)) return 5;
+    if (ohe.indexAt("cat") != 0 || ohe.indexAt("dog") != 1 || ohe.indexAt("bird") != -1) return 6;
+    std::vector<float> probe(2); probe[0] = 0.2f; probe[1] = 0.7f;
+    if (ohe[probe] != "dog" || ohe.classAt(0) != "cat" || ohe.classAt(5) != "") return 7;
+    printf("ohe ok\n");
+    return 0;
+}
+
+static int do_numberinput(const char* csv, const char* flag, const char* out)
+{
+    NumberInput di;
+    if (!di.standardizeInputTable(csv, !strcmp(flag, "zscore") ? GMath::ZSCORE : GMath::MINMAX)) return 1;
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    float head[3] = {(float)di.getTrainSize(), (float)di.getFeatureCount(), (float)di.getOutputCount()};
+    fwrite(head, 4, 3, fo);
+    for (unsigned int r = 0; r < di.getTrainSize(); ++r) { std::vector<float> v = di.getTrainRow(r); fwrite(v.data(), 4, v.size(), fo); }
+    for (unsigned int r = 0; r < di.getTrainSize(); ++r) { std::vector<float> v = di.getTrainExpectedRow(r); fwrite(v.data(), 4, v.size(), fo); }
+    fclose(fo);
+    for (size_t c = 0; c < di.getOHEMaps().size(); ++c) {
+        printf("col %d categorical %d classes", (int)c, (int)di.featureIsCategorical[c]);
+        std::vector<std::string> cls = di.getOHEMaps()[c].getStrings();
+        for (size_t k = 0; k < cls.size(); ++k) printf(" %s", cls[k].c_str());
+        printf("\n");
+    }
+    return 0;
+}
+
+// the flow of the reference's network test ("unit-tests/Backend/Machine Learning/nn-test.cpp":27-75):
+// NumberInput::import(csv), NNetwork::load(table), Terminator, glades::train.  Initial weights come
+// from srand(seed) + the sampler, or, when a case file is given, from that file (its table is ignored).
+struct Case {
+    int nl, batch, cost, N;
+    std::vector<int32_t> sizes, act;
+    std::vector<float> lr, mom, wd1, wd2, par, bias, X, Y;
+    std::vector<std::vector<float> > W;
+};
+
+static int read_case(const char* in, Case& c)
 {
     FILE* f = fopen(in, "rb");
     if (!f) return 1;
     int32_t magic, nl;
     if (fread(&magic, 4, 1, f) != 1 || fread(&nl, 4, 1, f) != 1 || magic != 0x474c4144) return 2;
-    std::vector<int32_t> sizes(nl + 1);
-    if (fread(sizes.data(), 4, nl + 1, f) != (size_t)nl + 1) return 2;
+    c.nl = nl;
+    c.sizes.resize(nl + 1);
+    if (fread(c.sizes.data(), 4, nl + 1, f) != (size_t)nl + 1) return 2;
     int32_t h4[4];
     if (fread(h4, 4, 4, f) != 4) return 2;
-    const int batch = h4[0], cost = h4[1], N = h4[2];
-    std::vector<float> lr(nl), mom(nl), wd1(nl), wd2(nl), par(nl);
-    std::vector<int32_t> act(nl);
+    c.batch = h4[0]; c.cost = h4[1]; c.N = h4[2];
+    c.lr.resize(nl); c.mom.resize(nl); c.wd1.resize(nl); c.wd2.resize(nl); c.par.resize(nl); c.act.resize(nl);
     for (int l = 0; l < nl; ++l) {
         float p[4];
-        if (fread(p, 4, 4, f) != 4 || fread(&act[l], 4, 1, f) != 1 || fread(&par[l], 4, 1, f) != 1) return 2;
-        lr[l] = p[0]; mom[l] = p[1]; wd1[l] = p[2]; wd2[l] = p[3];
+        if (fread(p, 4, 4, f) != 4 || fread(&c.act[l], 4, 1, f) != 1 || fread(&c.par[l], 4, 1, f) != 1) return 2;
+        c.lr[l] = p[0]; c.mom[l] = p[1]; c.wd1[l] = p[2]; c.wd2[l] = p[3];
     }
-    std::vector<std::vector<float> > W(nl);
+    c.W.resize(nl);
     for (int l = 0; l < nl; ++l) {
-        W[l].resize((size_t)sizes[l] * sizes[l + 1]);
-        if (fread(W[l].data(), 4, W[l].size(), f) != W[l].size()) return 2;
+        c.W[l].resize((size_t)c.sizes[l] * c.sizes[l + 1]);
+        if (fread(c.W[l].data(), 4, c.W[l].size(), f) != c.W[l].size()) return 2;
     }
-    std::vector<float> bias(nl);
-    if (fread(bias.data(), 4, nl, f) != (size_t)nl) return 2;
-    std::vector<float> X((size_t)N * sizes[0]), Y((size_t)N * sizes[nl]);
-    if (fread(X.data(), 4, X.size(), f) != X.size() || fread(Y.data(), 4, Y.size(), f) != Y.size()) return 2;
+    c.bias.resize(nl);
+    if (fread(c.bias.data(), 4, nl, f) != (size_t)nl) return 2;
+    c.X.resize((size_t)c.N * c.sizes[0]); c.Y.resize((size_t)c.N * c.sizes[nl]);
+    if (fread(c.X.data(), 4, c.X.size(), f) != c.X.size() || fread(c.Y.data(), 4, c.Y.size(), f) != c.Y.size()) return 2;
     fclose(f);
+    return 0;
+}
 
-    // skeleton rows: the input row carries weight layer 0's hyper-parameters, hidden row k those of
-    // weight layer k (ML/Structure/nninfo.cpp:240-373)
-    InputLayerInfo* il = new InputLayerInfo(batch, lr[0], mom[0], wd1[0], wd2[0], 0.0f, act[0], par[0]);
-    std::vector<HiddenLayerInfo*> hidden;
-    for (int k = 1; k < nl; ++k) hidden.push_back(new HiddenLayerInfo(sizes[k], lr[k], mom[k], wd1[k], wd2[k], 0.0f, act[k], par[k]));
-    OutputLayerInfo* ol = new OutputLayerInfo(sizes[nl], cost);
-    NNInfo info("check", il, hidden, ol);
-
-    glades::init();
-    DenseInput di(X.data(), Y.data(), N, sizes[0], sizes[nl]);
-    NNetwork net(&info);
-    net.setMode(mode);
-    for (int l = 0; l < nl; ++l) {
-        net.setWeights(l, W[l]);
-        if (mode == NNetwork::MODE_EXACT) net.setBias(l, std::vector<float>(1, bias[l]));
-    }
-    net.terminator.setEpoch(stop_epoch);
-    net.terminator.setAccuracy(stop_acc);
+// trains `net` on `di`, then runs the RUN_TEST pass, and writes what the tests read
+static int train_and_dump(NNetwork& net, DataInput* di, int nl, const char* out)
+{
     if (!(net.getAccuracy() < 95.0f)) return 3;  // the reference test's own pre-training assertion
-    MetaNetwork* meta = glades::train(&net, &di);
+    MetaNetwork* meta = glades::train(&net, di);
     if (!meta || meta->size() != 1) return 4;
     if (!net.getLastError().empty()) { fprintf(stderr, "error: %s\n", net.getLastError().c_str()); return 5; }
     const int trained = net.getEpochs();
@@ -127,7 +167,7 @@ static int do_train(const char* in, const char* out, long stop_epoch, float stop
         for (unsigned int r = 0; r < cm.size(); ++r)
             for (unsigned int c = 0; c < cm.size(); ++c) tail.push_back((float)cm.getCell(r, c));
     }
-    glades::test(&net, &di);   // RUN_TEST pass: one more epoch counted, parameters untouched
+    glades::test(&net, di);   // RUN_TEST pass: one more epoch counted, parameters untouched
     FILE* fo = fopen(out, "wb");
     if (!fo) return 1;
     float head[6] = {(float)trained, acc, loss, (float)net.getEpochs(), net.getAccuracy(), (float)results.size()};
@@ -147,10 +187,64 @@ static int do_train(const char* in, const char* out, long stop_epoch, float stop
     return 0;
 }
 
+static int do_train(const char* in, const char* out, long stop_epoch, float stop_acc, int mode)
+{
+    Case c;
+    int rc = read_case(in, c);
+    if (rc) return rc;
+    const int nl = c.nl;
+    // skeleton rows: the input row carries weight layer 0's hyper-parameters, hidden row k those of
+    // weight layer k (ML/Structure/nninfo.cpp:240-373)
+    InputLayerInfo* il = new InputLayerInfo(c.batch, c.lr[0], c.mom[0], c.wd1[0], c.wd2[0], 0.0f, c.act[0], c.par[0]);
+    std::vector<HiddenLayerInfo*> hidden;
+    for (int k = 1; k < nl; ++k) hidden.push_back(new HiddenLayerInfo(c.sizes[k], c.lr[k], c.mom[k], c.wd1[k], c.wd2[k], 0.0f, c.act[k], c.par[k]));
+    OutputLayerInfo* ol = new OutputLayerInfo(c.sizes[nl], c.cost);
+    NNInfo info("check", il, hidden, ol);
+
+    glades::init();
+    DenseInput di(c.X.data(), c.Y.data(), c.N, c.sizes[0], c.sizes[nl]);
+    NNetwork net(&info);
+    net.setMode(mode);
+    for (int l = 0; l < nl; ++l) {
+        net.setWeights(l, c.W[l]);
+        if (mode == NNetwork::MODE_EXACT) net.setBias(l, std::vector<float>(1, c.bias[l]));
+    }
+    net.terminator.setEpoch(stop_epoch);
+    net.terminator.setAccuracy(stop_acc);
+    return train_and_dump(net, &di, nl, out);
+}
+
+static int do_traincsv(const char* csv, const char* table, long stop_epoch, float stop_acc, int seed, const char* out, const char* weights)
+{
+    glades::init();
+    srand(seed);
+    NumberInput di;
+    di.import(csv);
+    NNetwork net;
+    if ((net.getEpochs() == 0) && (!net.load(table))) { printf("[NN] Unable to load \"%s\"", table); return 1; }
+    const int nl = net.getNNInfo()->numHiddenLayers() + 1;
+    if (weights) {
+        Case c;
+        int rc = read_case(weights, c);
+        if (rc) return rc;
+        if (c.nl != nl) return 6;
+        for (int l = 0; l < nl; ++l) {
+            net.setWeights(l, c.W[l]);
+            net.setBias(l, std::vector<float>(1, c.bias[l]));
+        }
+    }
+    net.terminator.setEpoch(stop_epoch);
+    net.terminator.setAccuracy(stop_acc);
+    return train_and_dump(net, &di, nl, out);
+}
+
 int main(int argc, char** argv)
 {
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
+    if (argc >= 2 && !strcmp(argv[1], "ohe")) return do_ohe();
+    if (argc >= 5 && !strcmp(argv[1], "numberinput")) return do_numberinput(argv[2], argv[3], argv[4]);
+    if (argc >= 8 && !strcmp(argv[1], "traincsv")) return do_traincsv(argv[2], argv[3], atol(argv[4]), (float)atof(argv[5]), atoi(argv[6]), argv[7], argc >= 9 ? argv[8] : NULL);
     if (argc >= 5 && !strcmp(argv[1], "cmatrix")) return do_cmatrix(atoi(argv[2]), argv[3], argv[4]);
     if (argc >= 7 && !strcmp(argv[1], "train")) return do_train(argv[2], argv[3], atol(argv[4]), (float)atof(argv[5]), atoi(argv[6]));
     fprintf(stderr, "usage: see the header of host_api_check.cpp\n");

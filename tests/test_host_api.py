@@ -71,6 +71,115 @@ def test_cmatrix_class_matches_restatement():
     assert bits_equal(raw[n * n:], po.cmatrix_metrics(want_M)[4])
 
 
+DATASETS = os.path.join(GOLDEN, "datasets")      # data files of the reference's own unit tests
+NETS = os.path.join(GOLDEN, "neuralnetworks")    # its NNInfo table fixtures
+
+
+def number_input(csv_path, flag="minmax"):
+    with tempfile.TemporaryDirectory() as td:
+        out = os.path.join(td, "ni.bin")
+        log = subprocess.check_output([BIN, "numberinput", csv_path, flag, out], text=True)
+        raw = np.fromfile(out, np.float32)
+    n, f, o = (int(v) for v in raw[:3])
+    X = raw[3:3 + n * f].reshape(n, f)
+    Y = raw[3 + n * f:].reshape(n, o)
+    assert raw.size == 3 + n * (f + o)
+    return X, Y, log.splitlines()
+
+
+@needs_bin
+def test_ohe_passes_the_reference_unit_test():
+    """The assertions of the reference's ohe-test.cpp:17-45 (0.99 / 0.01 encoding, duplicates, indexAt)."""
+    assert subprocess.check_output([BIN, "ohe"], text=True).strip() == "ohe ok"
+
+
+@needs_bin
+def test_number_input_on_the_reference_datasets():
+    # iris.data: the table the iris fixture was trained on by the reference's objects
+    X, Y, log = number_input(os.path.join(DATASETS, "iris.data"))
+    c = load_case("iris")
+    assert bits_equal(X, c["X"]) and bits_equal(Y, c["Y"])
+    assert log[-1] == "col 4 categorical 1 classes Iris-setosa Iris-versicolor Iris-virginica"
+    assert X[:, 0].min() == np.float32(0.01) and np.all(X.max(0) == np.float32(0.99))
+    assert np.all(X[:, 1:].min(0) > 0.04)   # minima of later columns are taken against 0, not the column
+    # xorgate.csv: no string column -> regression scaling to [0, 1], last column expected
+    X, Y, _ = number_input(os.path.join(DATASETS, "xorgate.csv"))
+    assert X.tolist() == [[0, 0], [0, 1], [1, 0], [1, 1]] and Y.tolist() == [[0], [1], [1], [0]]
+    # xorgateText.csv: every column categorical, classes in order of first appearance (dog, cat)
+    X, Y, log = number_input(os.path.join(DATASETS, "xorgateText.csv"))
+    hi, lo = np.float32(0.99), np.float32(0.01)
+    assert X.tolist() == [[hi, lo, hi, lo], [hi, lo, lo, hi], [lo, hi, hi, lo], [lo, hi, lo, hi]]
+    assert Y.tolist() == [[hi, lo], [lo, hi], [lo, hi], [hi, lo]]
+    assert log == ["col %d categorical 1 classes dog cat" % k for k in range(3)]
+
+
+@needs_bin
+def test_number_input_scaling_rules_by_hand():
+    with tempfile.TemporaryDirectory() as td:
+        p = os.path.join(td, "t.csv")
+        open(p, "w").write("a, b ,c\n2,5,10\n4,5,30\n\n6,5,20\n")
+        X, Y, _ = number_input(p)
+        # column 0 starts its min/max at the first cell; later columns start both at 0, so the
+        # constant 5 is scaled against [0, 5] and only an all-zero column counts as constant
+        np.testing.assert_array_equal(X, np.array([[0, 1], [0.5, 1], [1, 1]], np.float32))
+        np.testing.assert_array_equal(Y, np.array([[np.float32(10) / np.float32(30)], [1], [np.float32(20) / np.float32(30)]], np.float32))
+        open(p, "w").write("a,b,c\n1,0,-2\n2,0,4\n")
+        X, Y, _ = number_input(p)
+        np.testing.assert_array_equal(X, np.array([[0, 0], [1, 0]], np.float32))   # the all-zero column passes through
+        np.testing.assert_array_equal(Y, np.array([[0], [1]], np.float32))         # (-2 - -2) / 6, (4 - -2) / 6
+        # a string column anywhere makes it a classification table: [0.01, 0.99]
+        open(p, "w").write("a,k\n1,u\n3,v\n2,u\n")
+        X, Y, _ = number_input(p)
+        np.testing.assert_array_equal(X[:, 0], np.array([0.01, 0.99, np.float32(0.5) * np.float32(0.98) + np.float32(0.01)], np.float32))
+        np.testing.assert_array_equal(Y, np.array([[0.99, 0.01], [0.01, 0.99], [0.99, 0.01]], np.float32))
+        # z-score: mean over the rows, deviation with n - 1 (NumberInput.cpp:229-266)
+        open(p, "w").write("a,b\n1,2\n2,4\n6,9\n")
+        X, Y, _ = number_input(p, "zscore")
+        a = np.array([1, 2, 6], np.float64)
+        np.testing.assert_allclose(X[:, 0], (a - a.mean()) / a.std(ddof=1), rtol=1e-6)
+        b = np.array([2, 4, 9], np.float64)
+        np.testing.assert_allclose(Y[:, 0], (b - b.mean()) / b.std(ddof=1), rtol=1e-6)
+
+
+@needs_bin
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,csv,table", [("iris", "iris.data", "iris"), ("xornet", "xorgate.csv", "xornet")])
+def test_csv_to_trained_network_matches_fixture(name, csv, table):
+    """The reference's nn-test flow end to end: NumberInput::import(csv) + NNetwork::load(table) +
+    glades::train, started from the fixture's initial weights: the numbers of the fixture run."""
+    print("case", name, flush=True)
+    c = load_case(name)
+    with tempfile.TemporaryDirectory() as td:
+        cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
+        write_case(cin, c)
+        subprocess.check_call([BIN, "traincsv", os.path.join(DATASETS, csv), os.path.join(NETS, table), str(c["epochs"]), "0", "1",
+                               cout, cin], stdout=subprocess.DEVNULL)
+        head, res, Ws, bs, cls = read_out(cout, c)
+    d = c["d"]
+    assert int(head[0]) == c["epochs"]
+    np.testing.assert_allclose(head[1], d["epochs"][-1, 1], rtol=1e-4)
+    np.testing.assert_allclose(head[2], d["epochs"][-1, 0], rtol=1e-4)
+    np.testing.assert_allclose(res[1::2], d["preds"][-1], rtol=1e-4, atol=1e-6)
+    for l in range(c["nl"]):
+        np.testing.assert_allclose(Ws[l], d[f"W_{l}"], rtol=1e-4, atol=1e-4 * np.abs(d[f"W_{l}"]).max())
+    if name == "iris":
+        assert np.array_equal(cls[1], po.cmatrix(c["Y"], d["preds"]))
+
+
+@needs_bin
+@pytest.mark.gpu
+def test_text_dataset_trains_with_sampled_weights():
+    """xorgateText.csv + its table with weights from the sampler (srand): runs to the epoch limit."""
+    c = dict(nl=2, sizes=[4, 3, 2])
+    with tempfile.TemporaryDirectory() as td:
+        cout = os.path.join(td, "o.bin")
+        subprocess.check_call([BIN, "traincsv", os.path.join(DATASETS, "xorgateText.csv"), os.path.join(NETS, "xorgateText"), "50", "0", "7", cout],
+                              stdout=subprocess.DEVNULL)
+        head, res, Ws, bs, cls = read_out(cout, c)
+    assert int(head[0]) == 50 and np.isfinite(head[1]) and np.isfinite(head[2])
+    assert Ws[0].shape == (3, 4) and np.all(np.isfinite(Ws[0]))
+
+
 def write_case(path, c, wd2_layer0_from_wd1=True):
     s = c["spec"]
     nl = c["nl"]
