@@ -649,6 +649,44 @@ int ghip_net_get_params(ghip_net* n, int layer, float* host_W, float* host_bias,
     return 0;
 }
 
+// direction 0: device -> host, 1: host -> device
+static int move_state(ghip_net* n, int layer, float* a, float* b, int to_device)
+{
+    if (!n || layer < 0 || layer >= n->L) return fail(GHIP_EINVAL, "bad net or layer");
+    const ghip_net_spec& s = n->spec;
+    const int ni = s.sizes[layer], no = s.sizes[layer + 1];
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    if (s.mode == GHIP_MODE_EXACT) {
+        const int ld = n->ex.ld[layer];
+        float* dev[2] = {n->exSum + n->ex.woff[layer], n->exLast + n->ex.woff[layer]};
+        float* host[2] = {a, b};
+        std::vector<float> pad((size_t)ld * no, 0.0f);
+        for (int k = 0; k < 2; ++k) {
+            if (!host[k]) continue;
+            if (to_device) {
+                for (int o = 0; o < no; ++o) memcpy(&pad[(size_t)o * ld], host[k] + (size_t)o * ni, sizeof(float) * ni);
+                HIP_TRY(hipMemcpy(dev[k], pad.data(), pad.size() * 4, hipMemcpyHostToDevice));
+            } else {
+                HIP_TRY(hipMemcpy(pad.data(), dev[k], pad.size() * 4, hipMemcpyDeviceToHost));
+                for (int o = 0; o < no; ++o) memcpy(host[k] + (size_t)o * ni, &pad[(size_t)o * ld], sizeof(float) * ni);
+            }
+        }
+        return 0;
+    }
+    if (s.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "an inference-only network has no optimiser state");
+    if (a) HIP_TRY(to_device ? hipMemcpy(n->vW[layer], a, (size_t)ni * no * 4, hipMemcpyHostToDevice)
+                             : hipMemcpy(a, n->vW[layer], (size_t)ni * no * 4, hipMemcpyDeviceToHost));
+    if (b) HIP_TRY(to_device ? hipMemcpy(n->vb[layer], b, (size_t)no * 4, hipMemcpyHostToDevice)
+                             : hipMemcpy(b, n->vb[layer], (size_t)no * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int ghip_net_get_state(ghip_net* n, int layer, float* host_a, float* host_b) { return move_state(n, layer, host_a, host_b, 0); }
+int ghip_net_set_state(ghip_net* n, int layer, const float* host_a, const float* host_b)
+{
+    return move_state(n, layer, const_cast<float*>(host_a), const_cast<float*>(host_b), 1);
+}
+
 static int make_bf16_table(ghip_net* n)
 {
     const ghip_net_spec& s = n->spec;

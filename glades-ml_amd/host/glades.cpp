@@ -361,6 +361,95 @@ bool NNetwork::load(const std::string& path)
 
 bool NNetwork::save(const std::string& path) const { return skeleton ? skeleton->saveFile(path) : false; }
 
+// file: "GLCK" u32 version, i32 mode, i32 dtype, i32 epochs, i32 nLayers, i32 sizes[nLayers+1],
+//       u32 tableBytes, table text (the NNInfo CSV), then per layer: W, u32 biasLen, bias, u32 aLen, a, u32 bLen, b
+bool NNetwork::saveCheckpoint(const std::string& path)
+{
+    if (!skeleton || !dev) { lastError = "nothing to checkpoint: the network has not run"; return false; }
+    const int H = skeleton->numHiddenLayers(), L = H + 1;
+    std::vector<int32_t> sizes(L + 1);
+    sizes[0] = (int32_t)nFeat;
+    for (int i = 0; i < H; ++i) sizes[i + 1] = skeleton->getHiddenLayerSize(i);
+    sizes[L] = (int32_t)nOut;
+    const std::string tmp = path + ".table";
+    if (!skeleton->saveFile(tmp)) { lastError = "cannot write " + tmp; return false; }
+    std::string table;
+    {
+        FILE* t = fopen(tmp.c_str(), "rb");
+        if (!t) return false;
+        char buf[4096]; size_t got;
+        while ((got = fread(buf, 1, sizeof(buf), t)) > 0) table.append(buf, got);
+        fclose(t);
+        remove(tmp.c_str());
+    }
+    FILE* f = fopen(path.c_str(), "wb");
+    if (!f) { lastError = "cannot write " + path; return false; }
+    const uint32_t version = 1, tb = (uint32_t)table.size();
+    const int32_t head[4] = {mode, dtype, epochs, L};
+    fwrite("GLCK", 1, 4, f); fwrite(&version, 4, 1, f); fwrite(head, 4, 4, f); fwrite(sizes.data(), 4, sizes.size(), f);
+    fwrite(&tb, 4, 1, f); fwrite(table.data(), 1, table.size(), f);
+    bool ok = true;
+    for (int l = 0; l < L && ok; ++l) {
+        const size_t cnt = (size_t)sizes[l] * sizes[l + 1];
+        const uint32_t bl = mode == MODE_EXACT ? 1u : (uint32_t)sizes[l + 1];
+        const uint32_t al = (uint32_t)cnt, sl = mode == MODE_EXACT ? (uint32_t)cnt : (uint32_t)sizes[l + 1];
+        std::vector<float> W(cnt), b(bl), sa(al), sb(sl);
+        ok = ghip_net_get_params(dev, l, W.data(), b.data(), (int)bl) == 0 && ghip_net_get_state(dev, l, sa.data(), sb.data()) == 0;
+        if (!ok) { lastError = ghip_last_error(); break; }
+        fwrite(W.data(), 4, cnt, f);
+        fwrite(&bl, 4, 1, f); fwrite(b.data(), 4, bl, f);
+        fwrite(&al, 4, 1, f); fwrite(sa.data(), 4, al, f);
+        fwrite(&sl, 4, 1, f); fwrite(sb.data(), 4, sl, f);
+    }
+    fclose(f);
+    return ok;
+}
+
+bool NNetwork::loadCheckpoint(const std::string& path)
+{
+    FILE* f = fopen(path.c_str(), "rb");
+    if (!f) return false;
+    char magic[4];
+    uint32_t version = 0, tb = 0;
+    int32_t head[4];
+    bool ok = fread(magic, 1, 4, f) == 4 && memcmp(magic, "GLCK", 4) == 0 && fread(&version, 4, 1, f) == 1 && version == 1 &&
+              fread(head, 4, 4, f) == 4 && head[3] >= 1 && head[3] <= 16;
+    std::vector<int32_t> sizes;
+    std::string table;
+    if (ok) {
+        sizes.resize(head[3] + 1);
+        ok = fread(sizes.data(), 4, sizes.size(), f) == sizes.size() && fread(&tb, 4, 1, f) == 1 && tb < (1u << 20);
+    }
+    if (ok) { table.resize(tb); ok = fread(&table[0], 1, tb, f) == tb; }
+    std::vector<std::vector<float> > W, B, SA, SB;
+    for (int l = 0; ok && l < head[3]; ++l) {
+        const size_t cnt = (size_t)sizes[l] * sizes[l + 1];
+        std::vector<float> w(cnt), b, sa, sb;
+        uint32_t n1 = 0;
+        ok = fread(w.data(), 4, cnt, f) == cnt;
+        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { b.resize(n1); ok = fread(b.data(), 4, n1, f) == n1; }
+        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sa.resize(n1); ok = fread(sa.data(), 4, n1, f) == n1; }
+        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sb.resize(n1); ok = fread(sb.data(), 4, n1, f) == n1; }
+        W.push_back(w); B.push_back(b); SA.push_back(sa); SB.push_back(sb);
+    }
+    fclose(f);
+    if (!ok) { lastError = "not a checkpoint of this library: " + path; return false; }
+    const std::string tmp = path + ".table";
+    {
+        FILE* t = fopen(tmp.c_str(), "wb");
+        if (!t) return false;
+        fwrite(table.data(), 1, table.size(), t);
+        fclose(t);
+    }
+    const bool loaded = load(tmp);
+    remove(tmp.c_str());
+    if (!loaded) { lastError = "checkpoint holds no valid network table"; return false; }
+    clean();
+    mode = head[0]; dtype = head[1]; epochs = head[2];
+    initW = W; initB = B; initStateA = SA; initStateB = SB;
+    return true;
+}
+
 void NNetwork::train(DataInput* d) { run(d, RUN_TRAIN); }
 void NNetwork::test(DataInput* d) { run(d, RUN_TEST); }
 
@@ -449,6 +538,8 @@ bool NNetwork::build()
         int bl = 0;
         if ((size_t)l < initB.size() && !initB[l].empty()) { bp = initB[l].data(); bl = (int)initB[l].size(); }
         if (ghip_net_set_params(dev, l, W.data(), bp, bl) != 0) { lastError = ghip_last_error(); return false; }
+        if ((size_t)l < initStateA.size() && !initStateA[l].empty() && (size_t)l < initStateB.size() && !initStateB[l].empty())
+            if (ghip_net_set_state(dev, l, initStateA[l].data(), initStateB[l].data()) != 0) { lastError = ghip_last_error(); return false; }
     }
     if (ghip_net_set_dataset(dev, X.data(), Y.data(), (int64_t)nRows) != 0) { lastError = ghip_last_error(); return false; }
     // network.cpp:143-145: classification and KL runs keep a confusion matrix (counted on the device)
@@ -807,7 +898,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
     if (!newDataInput) return;
     di = newDataInput;
     if ((di->getTrainSize() <= 0) || (di->getFeatureCount() <= 0)) return;
-    if (epochs == 0 && !dev) {
+    if (!dev) {  // network.cpp:127-128 builds when epochs == 0; a restored checkpoint arrives with its epoch count
         if (!build()) {
             if (dev) ghip_net_destroy(dev);
             dev = NULL;

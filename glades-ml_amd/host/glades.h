@@ -331,6 +331,7 @@ class NNetwork
     std::vector<float> results;                 // (expected, predicted) pairs of the last row
     std::vector<std::vector<float> > initW;     // weights injected before the first run
     std::vector<std::vector<float> > initB;
+    std::vector<std::vector<float> > initStateA, initStateB;  // optimiser state of a restored checkpoint
     unsigned int nRows, nFeat, nOut;
     std::string lastError;
 
@@ -383,6 +384,12 @@ public:
     bool setBias(unsigned int layer, const std::vector<float>& bias);  // 1 value (exact) or n_out
     std::vector<float> getWeights(unsigned int layer);
     std::vector<float> getBias(unsigned int layer);
+    // Checkpoint = the skeleton's table + epochs run + every layer's weights, bias and optimiser state
+    // (exact mode: the pending delta windows; canonical: momentum), so that a restored network
+    // continues bit for bit.  The reference saves the table only (network.cpp:714-743: the weight
+    // part is a stub); the table text inside the file is its format, the rest is this build's.
+    bool saveCheckpoint(const std::string& path);
+    bool loadCheckpoint(const std::string& path);  // call train() afterwards with the same DataInput
     std::string getLastError() const { return lastError; }
 };
 

@@ -20,6 +20,7 @@ BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
 
 EXPORTS = [
     "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
+    "ghip_net_get_state", "ghip_net_set_state",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact",
     "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
@@ -76,6 +77,8 @@ def load():
             "ghip_net_destroy": (i, [vp]),
             "ghip_net_set_params": (i, [vp, i, vp, vp, i]),
             "ghip_net_get_params": (i, [vp, i, vp, vp, i]),
+            "ghip_net_get_state": (i, [vp, i, vp, vp]),
+            "ghip_net_set_state": (i, [vp, i, vp, vp]),
             "ghip_net_set_dataset": (i, [vp, vp, vp, i64]),
             "ghip_net_set_dataset_device": (i, [vp, vp, vp, i64]),
             "ghip_net_run_epochs_exact": (i, [vp, i, i, f, vp, C.POINTER(i), vp]),
@@ -176,6 +179,18 @@ class Net:
         b = np.zeros((blen,), np.float32)
         _check(self.lib.ghip_net_get_params(self.h, l, _ptr(W), _ptr(b), blen))
         return W, b
+
+    def get_state(self, l):
+        """exact: (pending-delta sums, last pending delta); canonical: (weight momentum, bias momentum)."""
+        a = np.empty((self.sizes[l + 1], self.sizes[l]), np.float32)
+        b = np.empty((self.sizes[l + 1], self.sizes[l]) if self.spec.mode == MODE_EXACT else (self.sizes[l + 1],), np.float32)
+        _check(self.lib.ghip_net_get_state(self.h, l, _ptr(a), _ptr(b)))
+        return a, b
+
+    def set_state(self, l, a, b):
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(b, np.float32)
+        _check(self.lib.ghip_net_set_state(self.h, l, _ptr(a), _ptr(b)))
 
     # ---- data
     def set_dataset(self, X, Y):

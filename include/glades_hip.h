@@ -107,6 +107,18 @@ int ghip_net_destroy(ghip_net* net);
 int ghip_net_set_params(ghip_net* net, int layer, const float* host_W, const float* host_bias, int bias_len);
 int ghip_net_get_params(ghip_net* net, int layer, float* host_W, float* host_bias, int bias_len);
 
+/* What a checkpoint needs beyond the parameters, so that a restored network continues exactly as the
+ * original would have (the reference's NNetwork::save writes the NNInfo table only and leaves the
+ * weights to a stub, ML/Networks/network.cpp:714-743, so there is no reference format to follow).
+ * exact mode:     a = pending-delta running sums, b = last pending delta, each sizes[layer+1] x
+ *                 sizes[layer] row-major: the content of the reference's Edge::prevDelta windows
+ *                 (ML/State/edge.cpp:54-101), which survive from one epoch into the next.
+ * canonical mode: a = weight momentum (previous update) sizes[layer+1] x sizes[layer],
+ *                 b = bias momentum sizes[layer+1].
+ * Either pointer may be NULL.  ghip_net_set_params clears this state: set the parameters first. */
+int ghip_net_get_state(ghip_net* net, int layer, float* host_a, float* host_b);
+int ghip_net_set_state(ghip_net* net, int layer, const float* host_a, const float* host_b);
+
 /* Uploads the training table once: replaces LayerBuilder::buildInputLayers
  * (ML/State/LayerBuilder.cpp:100-190) and DataInput::getTrainRow / getTrainExpectedRow
  * (ML/DataObjects/DataInput.h:39-40).  X is N x sizes[0], Y is N x sizes[n_layers]. */

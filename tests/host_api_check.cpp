@@ -9,6 +9,7 @@
 //   host_api_check ohe                                                   (no GPU needed)
 //   host_api_check numberinput <file.csv> <minmax|zscore> <out.bin>      (no GPU needed)
 //   host_api_check traincsv <file.csv> <nninfo table> <stop_epoch> <stop_accuracy> <seed> <out.bin> [case.bin with the initial weights]
+//   host_api_check checkpoint <case.bin> <mode> <E1> <E2> <file.ckpt> <out.bin>
 //   host_api_check train  <case.bin> <out.bin> <stop_epoch> <stop_accuracy> <mode>
 #include <stdio.h>
 #include <stdlib.h>
@@ -238,10 +239,70 @@ static int do_traincsv(const char* csv, const char* table, long stop_epoch, floa
     return train_and_dump(net, &di, nl, out);
 }
 
+static NNInfo* case_info(const Case& c)
+{
+    InputLayerInfo* il = new InputLayerInfo(c.batch, c.lr[0], c.mom[0], c.wd1[0], c.wd2[0], 0.0f, c.act[0], c.par[0]);
+    std::vector<HiddenLayerInfo*> hidden;
+    for (int k = 1; k < c.nl; ++k) hidden.push_back(new HiddenLayerInfo(c.sizes[k], c.lr[k], c.mom[k], c.wd1[k], c.wd2[k], 0.0f, c.act[k], c.par[k]));
+    return new NNInfo("check", il, hidden, new OutputLayerInfo(c.sizes[c.nl], c.cost));
+}
+
+static void seed_net(NNetwork& net, const Case& c, int mode)
+{
+    net.setMode(mode);
+    for (int l = 0; l < c.nl; ++l) {
+        net.setWeights(l, c.W[l]);
+        if (mode == NNetwork::MODE_EXACT) net.setBias(l, std::vector<float>(1, c.bias[l]));
+    }
+}
+
+// A trains E1 epochs and saves; B restores and trains on to E1 + E2; C trains E1 + E2 in one go.
+// out: epochs of B and C, then every layer's weights and bias of B, then of C.
+static int do_checkpoint(const char* in, int mode, int e1, int e2, const char* ckpt, const char* out)
+{
+    Case c;
+    int rc = read_case(in, c);
+    if (rc) return rc;
+    glades::init();
+    DenseInput di(c.X.data(), c.Y.data(), c.N, c.sizes[0], c.sizes[c.nl]);
+    NNInfo* ia = case_info(c);
+    NNInfo* ic = case_info(c);
+    {
+        NNetwork a(ia);
+        seed_net(a, c, mode);
+        a.terminator.setEpoch(e1);
+        a.train(&di);
+        if (a.getEpochs() != e1 || !a.saveCheckpoint(ckpt)) { fprintf(stderr, "save: %s\n", a.getLastError().c_str()); return 3; }
+    }
+    NNetwork b;
+    if (!b.loadCheckpoint(ckpt)) { fprintf(stderr, "load: %s\n", b.getLastError().c_str()); return 4; }
+    if (b.getEpochs() != e1) return 5;
+    b.terminator.setEpoch(e1 + e2);
+    b.train(&di);
+    NNetwork cn(ic);
+    seed_net(cn, c, mode);
+    cn.terminator.setEpoch(e1 + e2);
+    cn.train(&di);
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    float head[4] = {(float)b.getEpochs(), (float)cn.getEpochs(), b.getLoss(), cn.getLoss()};
+    fwrite(head, 4, 4, fo);
+    NNetwork* nets[2] = {&b, &cn};
+    for (int k = 0; k < 2; ++k)
+        for (int l = 0; l < c.nl; ++l) {
+            std::vector<float> w = nets[k]->getWeights(l), bb = nets[k]->getBias(l);
+            fwrite(w.data(), 4, w.size(), fo);
+            fwrite(bb.data(), 4, bb.size(), fo);
+        }
+    fclose(fo);
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
+    if (argc >= 8 && !strcmp(argv[1], "checkpoint")) return do_checkpoint(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7]);
     if (argc >= 2 && !strcmp(argv[1], "ohe")) return do_ohe();
     if (argc >= 5 && !strcmp(argv[1], "numberinput")) return do_numberinput(argv[2], argv[3], argv[4]);
     if (argc >= 8 && !strcmp(argv[1], "traincsv")) return do_traincsv(argv[2], argv[3], atol(argv[4]), (float)atof(argv[5]), atoi(argv[6]), argv[7], argc >= 9 ? argv[8] : NULL);

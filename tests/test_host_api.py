@@ -309,3 +309,30 @@ def test_canonical_mode_through_class_api():
         Wo, bo = o.get_params(l)
         np.testing.assert_allclose(Ws[l], Wo, rtol=1e-4, atol=2e-6)
         np.testing.assert_allclose(bs[l], bo, rtol=1e-4, atol=2e-6)
+
+
+@needs_bin
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,mode", [("window_4_5_3_1", 0), ("cfg1_shape_4_16_3", 0), ("iris", 1)])
+def test_checkpoint_resume_is_bit_identical(name, mode):
+    """saveCheckpoint after E1 epochs + loadCheckpoint + E2 more epochs = E1 + E2 epochs in one go:
+    weights, biases and loss bit for bit (exact mode carries its pending delta windows across the
+    epoch boundary; canonical mode its momentum)."""
+    print("case", name, "mode", mode, flush=True)
+    c = load_case(name)
+    if mode == 1:
+        c = dict(c)
+        c["spec"].mom[0] = c["spec"].mom[1] = 0.9
+        c["mb"] = 32
+    with tempfile.TemporaryDirectory() as td:
+        cin, ck, cout = os.path.join(td, "c.bin"), os.path.join(td, "n.ckpt"), os.path.join(td, "o.bin")
+        write_case(cin, c)
+        subprocess.check_call([BIN, "checkpoint", cin, str(mode), "3", "2", ck, cout], stdout=subprocess.DEVNULL)
+        raw = np.fromfile(cout, np.float32)
+        assert os.path.getsize(ck) > 64
+    assert raw[0] == 5 and raw[1] == 5
+    assert bits_equal(raw[2:3], raw[3:4])
+    body = raw[4:]
+    assert body.size % 2 == 0
+    assert bits_equal(body[:body.size // 2], body[body.size // 2:])
+    assert np.all(np.isfinite(body))
