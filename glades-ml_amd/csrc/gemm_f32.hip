@@ -7,11 +7,15 @@
 //   back-prop e = W^T d                          network.cpp:660-662  -> C = D * W
 //   gradient  dW = d (x) a, summed over the batch  node.cpp:278-292   -> C = D^T * A
 //
-// Tile: 64 x 64 x 16 per workgroup of 4 wavefronts, each wavefront owns one 32x32 accumulator
-// (16 VGPRs).  Operands are staged through LDS K-major ([k][row]) so that the per-lane operand
-// fetch of the 32x32x2 instruction (lane -> row = lane%32, k = lane/32) reads 32 consecutive
-// words: conflict free.  Two LDS buffers: the next K-slab is fetched from global memory into
-// registers while the current one feeds the matrix cores.
+// Tile: 64 x 64 per workgroup of 8 wavefronts, K in slabs of 64.  Wavefront w owns the 32x32
+// accumulator (w/2)%2, w%2 of the tile and half of every slab's K (w/4): these products are small
+// (batch 512, layers ~1024 wide), so splitting K inside the workgroup is what gives all four SIMDs
+// of a CU a matrix instruction stream; the two halves are added through LDS in a fixed order.
+// Each operand keeps in LDS the orientation it has in global memory, so that staging never
+// transposes: [k][row] with pitch 68 (16-byte stores) for a K-major operand, [row][k] with the odd
+// pitch 65 otherwise; the per-lane operand fetch of the 32x32x2 instruction (lane -> row = lane%32,
+// k = lane/32) is conflict free in both (consecutive words, or a stride of 65 words).  Three LDS slabs: slab kt+2 travels from global memory into registers while slab kt feeds
+// the matrix cores and slab kt+1 already waits in LDS.
 
 #include "ghip_internal.h"
 
@@ -19,94 +23,131 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 64, BN = 64, BK = 16, LDT = 64 + 4;
+constexpr int BM = 64, BN = 64, BK = 64, LDT = 64 + 4, NST = 3, NTHR = 512, UNITS = BM * BK / 4 / NTHR;
 
-struct Frag { float v[4]; };
+struct Frag { float4 v[UNITS]; bool ok[UNITS]; };  // ok: the unit lies inside the operand (FAST path)
 
-// Fetch this lane's 4 elements of a 64(row) x 16(k) operand tile.
-//   kmajor == 0: P is [rows][K]  (ld = row stride): lane -> row = t/4, k = (t%4)*4 .. +3
-//   kmajor == 1: P is [K][rows]  (ld = k stride):   lane -> k = t/16, row = (t%16)*4 .. +3
-__device__ __forceinline__ Frag fetch(const float* __restrict__ P, int ld, int kmajor, int vec_ok,
-                                      int r0, int k0, int R, int K, int t)
+// Fetch this thread's UNITS float4 of a 64(row) x 64(k) operand tile.
+//   kmajor == 0: P is [rows][K]  (ld = row stride): unit u -> row = u/16, k = (u%16)*4 .. +3
+//   kmajor == 1: P is [K][rows]  (ld = k stride):   unit u -> k = u/16, row = (u%16)*4 .. +3
+// FAST: the minor extent is a multiple of 4 and rows are 16-byte aligned, so a unit is wholly
+// inside or wholly outside the operand: one unconditional 16-byte load from a clamped address and
+// a select, no control flow (loads inside branches are waited for where the branches join, which
+// serialises the slab's fetch with its use).
+template <bool FAST>
+__device__ __forceinline__ Frag fetch(const float* __restrict__ P, int ld, int kmajor, int r0, int k0, int R, int K, int t)
 {
     Frag f;
-    if (!kmajor) {
-        const int row = r0 + (t >> 2), k = k0 + ((t & 3) << 2);
-        const float* src = P + (long long)row * ld + k;
-        if (row < R && k + 3 < K && vec_ok) {
-            float4 q = *reinterpret_cast<const float4*>(src);
-            f.v[0] = q.x; f.v[1] = q.y; f.v[2] = q.z; f.v[3] = q.w;
-        } else {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.v[j] = (row < R && k + j < K) ? src[j] : 0.0f;
-        }
-    } else {
-        const int k = k0 + (t >> 4), row = r0 + ((t & 15) << 2);
-        const float* src = P + (long long)k * ld + row;
-        if (k < K && row + 3 < R && vec_ok) {
-            float4 q = *reinterpret_cast<const float4*>(src);
-            f.v[0] = q.x; f.v[1] = q.y; f.v[2] = q.z; f.v[3] = q.w;
+    for (int i = 0; i < UNITS; ++i) {
+        const int u = t + i * NTHR;
+        const int major = u >> 4, minor = (u & 15) << 2;
+        if constexpr (FAST) {
+            const int mj = (kmajor ? k0 : r0) + major, mn = (kmajor ? r0 : k0) + minor;
+            const bool ok = mj < (kmajor ? K : R) && mn < (kmajor ? R : K);
+            // the value is not touched here: zeroing it now would wait for the load before the slab's MFMAs
+            f.v[i] = *reinterpret_cast<const float4*>(P + (ok ? (long long)mj * ld + mn : 0ll));
+            f.ok[i] = ok;
         } else {
+            const int row = kmajor ? r0 + minor : r0 + major;
+            const int k = kmajor ? k0 + major : k0 + minor;
+            const float* src = P + (kmajor ? (long long)k * ld + row : (long long)row * ld + k);
+            float e[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) f.v[j] = (k < K && row + j < R) ? src[j] : 0.0f;
+            for (int j = 0; j < 4; ++j) {
+                const bool ok = kmajor ? (k < K && row + j < R) : (row < R && k + j < K);
+                e[j] = ok ? src[j] : 0.0f;
+            }
+            f.v[i] = make_float4(e[0], e[1], e[2], e[3]);
+            f.ok[i] = true;
         }
     }
     return f;
 }
 
-__device__ __forceinline__ void stage(float (*dst)[LDT], const Frag& f, int kmajor, int t)
+constexpr int SLAB = BK * LDT;  // floats of one operand slab (covers both orientations)
+constexpr int PITCH_ROWS = 65;  // [row][k] orientation
+
+__device__ __forceinline__ void stage(float* dst, const Frag& f, int kmajor, int t)
 {
-    if (!kmajor) {
-        const int row = t >> 2, k = (t & 3) << 2;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) dst[k + j][row] = f.v[j];
-    } else {
-        const int k = t >> 4, row = (t & 15) << 2;
-        *reinterpret_cast<float4*>(&dst[k][row]) = make_float4(f.v[0], f.v[1], f.v[2], f.v[3]);
+    for (int i = 0; i < UNITS; ++i) {
+        const int u = t + i * NTHR;
+        const int major = u >> 4, minor = (u & 15) << 2;
+        const float4 q = f.ok[i] ? f.v[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (!kmajor) {
+            float* d = dst + major * PITCH_ROWS + minor;   // row major, k minor .. +3
+            d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
+        } else {
+            *reinterpret_cast<float4*>(dst + major * LDT + minor) = q;   // k major, row minor .. +3
+        }
     }
 }
 
-__global__ void __launch_bounds__(256) gemm_f32_kernel(GemmF32Args g)
+template <bool FAST>
+__global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
 {
-    __shared__ __attribute__((aligned(16))) float As[2][BK][LDT];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK][LDT];
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float* const As = lds;
+    float* const Bs = lds + NST * SLAB;
+    // word index of (k, row) in a slab: k * sk + row * sr
+    const int ska = g.a_kmajor ? LDT : 1, sra = g.a_kmajor ? 1 : PITCH_ROWS;
+    const int skb = g.b_kmajor ? LDT : 1, srb = g.b_kmajor ? 1 : PITCH_ROWS;
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
     const int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
-    const int wm = (w >> 1) * 32, wn = (w & 1) * 32;
-    const int a_vec = ((g.lda & 3) == 0) && ((((uintptr_t)g.A) & 15) == 0);
-    const int b_vec = ((g.ldb & 3) == 0) && ((((uintptr_t)g.B) & 15) == 0);
+    const int wm = ((w >> 1) & 1) * 32, wn = (w & 1) * 32, kh = (w >> 2) * (BK / 2);
 
     v16f acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
-    Frag fa = fetch(g.A, g.lda, g.a_kmajor, a_vec, bm, 0, g.M, g.K, t);
-    Frag fb = fetch(g.B, g.ldb, g.b_kmajor, b_vec, bn, 0, g.N, g.K, t);
-    stage(As[0], fa, g.a_kmajor, t);
-    stage(Bs[0], fb, g.b_kmajor, t);
+    const int nk = (g.K + BK - 1) / BK;
+    Frag fa = fetch<FAST>(g.A, g.lda, g.a_kmajor, bm, 0, g.M, g.K, t);
+    Frag fb = fetch<FAST>(g.B, g.ldb, g.b_kmajor, bn, 0, g.N, g.K, t);
+    stage(As, fa, g.a_kmajor, t);
+    stage(Bs, fb, g.b_kmajor, t);
+    if (nk > 1) {
+        fa = fetch<FAST>(g.A, g.lda, g.a_kmajor, bm, BK, g.M, g.K, t);
+        fb = fetch<FAST>(g.B, g.ldb, g.b_kmajor, bn, BK, g.N, g.K, t);
+        stage(As + SLAB, fa, g.a_kmajor, t);
+        stage(Bs + SLAB, fb, g.b_kmajor, t);
+    }
     __syncthreads();
 
-    const int nk = (g.K + BK - 1) / BK;
     const int lr = lane & 31, lk = lane >> 5;
     for (int kt = 0; kt < nk; ++kt) {
-        const int cur = kt & 1;
-        if (kt + 1 < nk) {
-            fa = fetch(g.A, g.lda, g.a_kmajor, a_vec, bm, (kt + 1) * BK, g.M, g.K, t);
-            fb = fetch(g.B, g.ldb, g.b_kmajor, b_vec, bn, (kt + 1) * BK, g.N, g.K, t);
+        const int cur = kt % NST, nxt = (kt + 2) % NST;
+        const bool more = kt + 2 < nk;
+        if (more) {
+            fa = fetch<FAST>(g.A, g.lda, g.a_kmajor, bm, (kt + 2) * BK, g.M, g.K, t);
+            fb = fetch<FAST>(g.B, g.ldb, g.b_kmajor, bn, (kt + 2) * BK, g.N, g.K, t);
         }
+        const float* pa = As + cur * SLAB + (kh + lk) * ska + (wm + lr) * sra;
+        const float* pb = Bs + cur * SLAB + (kh + lk) * skb + (wn + lr) * srb;
+        float av[BK / 4], bv[BK / 4];  // this wavefront's 16 operand pairs of the slab, requested together
 #pragma unroll
-        for (int kk = 0; kk < BK; kk += 2) {
-            const float a = As[cur][kk + lk][wm + lr];
-            const float b = Bs[cur][kk + lk][wn + lr];
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc, 0, 0, 0);
-        }
-        if (kt + 1 < nk) {
-            stage(As[cur ^ 1], fa, g.a_kmajor, t);
-            stage(Bs[cur ^ 1], fb, g.b_kmajor, t);
+        for (int i = 0; i < BK / 4; ++i) { av[i] = pa[2 * i * ska]; bv[i] = pb[2 * i * skb]; }
+        __builtin_amdgcn_sched_barrier(0);  // keep the reads together: sunk next to their MFMA each would be waited for alone
+#pragma unroll
+        for (int i = 0; i < BK / 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[i], acc, 0, 0, 0);
+        if (more) {  // slab kt-1's buffer: every wavefront left it before the barrier that ended kt-1
+            stage(As + nxt * SLAB, fa, g.a_kmajor, t);
+            stage(Bs + nxt * SLAB, fb, g.b_kmajor, t);
         }
         __syncthreads();
     }
+
+    // the upper K halves go to LDS ([wavefront][register][lane]) and are added by the lower ones
+    float* red = lds;
+    if (w >= 4) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) red[((w - 4) * 16 + i) * 64 + lane] = acc[i];
+    }
+    __syncthreads();
+    if (w >= 4) return;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] += red[(w * 16 + i) * 64 + lane];
 
     // accumulator layout of the 32x32 tile: lane -> column lane%32; register i -> row
     // 8*(i/4) + 4*(lane/32) + i%4
@@ -134,6 +175,17 @@ hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s)
 {
     if (a.M <= 0 || a.N <= 0 || a.K <= 0) return hipErrorInvalidValue;
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM);
-    hipLaunchKernelGGL(gemm_f32_kernel, grid, dim3(256), 0, s, a);
+    constexpr size_t lds_bytes = sizeof(float) * 2 * NST * SLAB;  // 104 448 B: above the 64 KiB default
+    static bool raised = false;
+    if (!raised) {
+        hipError_t e = hipFuncSetAttribute((const void*)gemm_f32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemm_f32_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        raised = true;
+    }
+    const bool a_fast = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((a.a_kmajor ? a.M : a.K) % 4) == 0;
+    const bool b_fast = (a.ldb % 4) == 0 && ((uintptr_t)a.B % 16) == 0 && ((a.b_kmajor ? a.N : a.K) % 4) == 0;
+    if (a_fast && b_fast) hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(NTHR), lds_bytes, s, a);
+    else hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(NTHR), lds_bytes, s, a);
     return hipGetLastError();
 }
