@@ -73,6 +73,7 @@ struct ghip_net {
     float* act[GHIP_MAX_LAYERS + 1] = {};
     float* dlt[GHIP_MAX_LAYERS + 1] = {};
     float* stageX = nullptr;
+    float* bpart = nullptr;   // fp32 path: bias-gradient partial sums [16][widest layer]
     int cap_batch = 0;
     double* dAcc = nullptr;
     int last_batch = 0;
@@ -289,7 +290,7 @@ void free_batch_buffers(ghip_net* n)
         if (l > 0) dfree(n->H[l]);
         dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]); dfree(n->csum[l]);
     }
-    dfree(n->stageX); dfree(n->logits);
+    dfree(n->stageX); dfree(n->logits); dfree(n->bpart);
     dfree(n->Aq[0]); dfree(n->Aq[1]); dfree(n->ascale[0]); dfree(n->ascale[1]);
     dfree(n->amax_bits); dfree(n->Hq); dfree(n->out8);
     n->cap_batch = 0;
@@ -306,6 +307,7 @@ int reserve_batch(ghip_net* n, int B)
     for (int l = 0; l <= L; ++l) if (s.sizes[l] > maxw) maxw = s.sizes[l];
     if (s.dtype == GHIP_F32) {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
+        TRY(dalloc(&n->bpart, (size_t)16 * maxw));
         for (int l = 1; l <= L; ++l) {
             TRY(dalloc(&n->act[l], (size_t)B * s.sizes[l]));
             TRY(dalloc(&n->dlt[l], (size_t)B * s.sizes[l]));
@@ -419,7 +421,11 @@ int step_f32(ghip_net* n, int64_t row0, int B)
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1]; g.alpha = 1.0f;
             LAUNCH(n, "gemm_f32_dgrad", ghip_gemm_f32(g, n->stream));
         }
-        LAUNCH(n, "bias_update", ghip_bias_update_f32(n->dlt[l + 1], B, no, no, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+        {   // bias gradient = column sums of the delta, over row chunks that are then added in order
+            const int chunks = B >= 1024 ? 16 : (B >= 128 ? 8 : 1);
+            LAUNCH(n, "bias_colsum", ghip_colsum_f32(n->dlt[l + 1], B, no, no, chunks, n->bpart, n->stream));
+            LAUNCH(n, "bias_update", ghip_bias_update_partials(n->bpart, chunks, no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+        }
         LAUNCH(n, "sgd_update_f32", ghip_sgd_update_f32(n->W[l], n->vW[l], n->gW[l], (long long)ni * no, s.lr[l], s.mom[l],
                                                        s.wd1[l], s.wd2[l], 1.0f, n->stream));
     }

@@ -267,6 +267,25 @@ bias_update_f32_kernel(const float* __restrict__ D, int B, int n, int ldd, float
     }
 }
 
+// column sums of a slice of rows: partial[blockIdx.y][o] = sum over rows [y*rpc, (y+1)*rpc) of D[b][o]
+// (the bias gradient of the fp32 path, split over row chunks so that small batches still fill the
+// device; the chunks are added in order by bias_update_partials_kernel)
+__global__ void __launch_bounds__(256)
+colsum_f32_kernel(const float* __restrict__ D, int B, int n, int ldd, int rows_per_chunk, float* __restrict__ partial)
+{
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int o = blockIdx.x * 64 + lane;
+    const int b0 = blockIdx.y * rows_per_chunk;
+    const int b1 = (b0 + rows_per_chunk) < B ? (b0 + rows_per_chunk) : B;
+    float s = 0.0f;
+    if (o < n)
+        for (int b = b0 + w; b < b1; b += 4) s += D[(long long)b * ldd + o];
+    __shared__ float red[4][64];
+    red[w][lane] = s;
+    __syncthreads();
+    if (w == 0 && o < n) partial[(long long)blockIdx.y * n + o] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+}
+
 // bf16 delta^T [n][B]: one wavefront per channel, 16-byte loads (B is a multiple of 8)
 __global__ void __launch_bounds__(256)
 bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* __restrict__ bias,
@@ -538,6 +557,13 @@ hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bi
                                 float mom, hipStream_t s)
 {
     hipLaunchKernelGGL(bias_update_f32_kernel, dim3((n + 63) / 64), dim3(256), 0, s, D, B, n, ldd, bias, vb, lr, mom);
+    return hipGetLastError();
+}
+
+hipError_t ghip_colsum_f32(const float* D, int B, int n, int ldd, int chunks, float* partial, hipStream_t s)
+{
+    const int rpc = (B + chunks - 1) / chunks;
+    hipLaunchKernelGGL(colsum_f32_kernel, dim3((n + 63) / 64, chunks), dim3(256), 0, s, D, B, n, ldd, rpc, partial);
     return hipGetLastError();
 }
 

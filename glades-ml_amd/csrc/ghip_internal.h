@@ -275,6 +275,8 @@ hipError_t ghip_sgd_update_f32(float* W, float* V, const float* G, long long n, 
 // gb[o] = sum_b D[b][o] (fp32 D [B][n]) fused with the bias update (no decay)
 hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bias, float* vbias,
                                 float lr, float mom, hipStream_t s);
+// partial[c][o] = column sums of D over row chunk c (chunks of ceil(B / chunks) rows)
+hipError_t ghip_colsum_f32(const float* D, int B, int n, int ldd, int chunks, float* partial, hipStream_t s);
 hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s);
 hipError_t ghip_fill_f64(double* p, long long n, double v, hipStream_t s);
 
