@@ -12,9 +12,10 @@
 // (batch 512, layers ~1024 wide), so splitting K inside the workgroup is what gives all four SIMDs
 // of a CU a matrix instruction stream; the two halves are added through LDS in a fixed order.
 // Each operand keeps in LDS the orientation it has in global memory, so that staging never
-// transposes: [k][row] with pitch 68 (16-byte stores) for a K-major operand, [row][k] with the odd
-// pitch 65 otherwise; the per-lane operand fetch of the 32x32x2 instruction (lane -> row = lane%32,
-// k = lane/32) is conflict free in both (consecutive words, or a stride of 65 words).  Three LDS slabs: slab kt+2 travels from global memory into registers while slab kt feeds
+// transposes: [k][row] for a K-major operand, [row][k] otherwise, both with pitch 68 (16-byte
+// stores).  A lane of the 32x32x2 instruction supplies one row and one of the two k of an MFMA; here
+// lane half lk takes k = 16*lk + i of its wavefront's half slab for MFMA i, so a [row][k] operand is
+// fetched with four 16-byte reads per slab (a [k][row] operand with sixteen 4-byte reads).  Three LDS slabs: slab kt+2 travels from global memory into registers while slab kt feeds
 // the matrix cores and slab kt+1 already waits in LDS.
 
 #include "ghip_internal.h"
@@ -66,7 +67,7 @@ __device__ __forceinline__ Frag fetch(const float* __restrict__ P, int ld, int k
 }
 
 constexpr int SLAB = BK * LDT;  // floats of one operand slab (covers both orientations)
-constexpr int PITCH_ROWS = 65;  // [row][k] orientation
+constexpr int PITCH_ROWS = 68;  // [row][k] orientation: 16-byte aligned rows; 16 lanes x 4 words step over all 64 banks
 
 __device__ __forceinline__ void stage(float* dst, const Frag& f, int kmajor, int t)
 {
@@ -76,23 +77,22 @@ __device__ __forceinline__ void stage(float* dst, const Frag& f, int kmajor, int
         const int major = u >> 4, minor = (u & 15) << 2;
         const float4 q = f.ok[i] ? f.v[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if (!kmajor) {
-            float* d = dst + major * PITCH_ROWS + minor;   // row major, k minor .. +3
-            d[0] = q.x; d[1] = q.y; d[2] = q.z; d[3] = q.w;
+            *reinterpret_cast<float4*>(dst + major * PITCH_ROWS + minor) = q;   // row major, k minor .. +3
         } else {
             *reinterpret_cast<float4*>(dst + major * LDT + minor) = q;   // k major, row minor .. +3
         }
     }
 }
 
-template <bool FAST>
+template <bool FAST, bool AKM, bool BKM>
 __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
 {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     float* const As = lds;
     float* const Bs = lds + NST * SLAB;
     // word index of (k, row) in a slab: k * sk + row * sr
-    const int ska = g.a_kmajor ? LDT : 1, sra = g.a_kmajor ? 1 : PITCH_ROWS;
-    const int skb = g.b_kmajor ? LDT : 1, srb = g.b_kmajor ? 1 : PITCH_ROWS;
+    constexpr int ska = AKM ? LDT : 1, sra = AKM ? 1 : PITCH_ROWS;
+    constexpr int skb = BKM ? LDT : 1, srb = BKM ? 1 : PITCH_ROWS;
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
     const int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
@@ -103,15 +103,15 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
     const int nk = (g.K + BK - 1) / BK;
-    Frag fa = fetch<FAST>(g.A, g.lda, g.a_kmajor, bm, 0, g.M, g.K, t);
-    Frag fb = fetch<FAST>(g.B, g.ldb, g.b_kmajor, bn, 0, g.N, g.K, t);
-    stage(As, fa, g.a_kmajor, t);
-    stage(Bs, fb, g.b_kmajor, t);
+    Frag fa = fetch<FAST>(g.A, g.lda, AKM, bm, 0, g.M, g.K, t);
+    Frag fb = fetch<FAST>(g.B, g.ldb, BKM, bn, 0, g.N, g.K, t);
+    stage(As, fa, AKM, t);
+    stage(Bs, fb, BKM, t);
     if (nk > 1) {
-        fa = fetch<FAST>(g.A, g.lda, g.a_kmajor, bm, BK, g.M, g.K, t);
-        fb = fetch<FAST>(g.B, g.ldb, g.b_kmajor, bn, BK, g.N, g.K, t);
-        stage(As + SLAB, fa, g.a_kmajor, t);
-        stage(Bs + SLAB, fb, g.b_kmajor, t);
+        fa = fetch<FAST>(g.A, g.lda, AKM, bm, BK, g.M, g.K, t);
+        fb = fetch<FAST>(g.B, g.ldb, BKM, bn, BK, g.N, g.K, t);
+        stage(As + SLAB, fa, AKM, t);
+        stage(Bs + SLAB, fb, BKM, t);
     }
     __syncthreads();
 
@@ -120,20 +120,22 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
         const int cur = kt % NST, nxt = (kt + 2) % NST;
         const bool more = kt + 2 < nk;
         if (more) {
-            fa = fetch<FAST>(g.A, g.lda, g.a_kmajor, bm, (kt + 2) * BK, g.M, g.K, t);
-            fb = fetch<FAST>(g.B, g.ldb, g.b_kmajor, bn, (kt + 2) * BK, g.N, g.K, t);
+            fa = fetch<FAST>(g.A, g.lda, AKM, bm, (kt + 2) * BK, g.M, g.K, t);
+            fb = fetch<FAST>(g.B, g.ldb, BKM, bn, (kt + 2) * BK, g.N, g.K, t);
         }
-        const float* pa = As + cur * SLAB + (kh + lk) * ska + (wm + lr) * sra;
-        const float* pb = Bs + cur * SLAB + (kh + lk) * skb + (wn + lr) * srb;
+        // lane half lk supplies k = kh + 16*lk + i to MFMA i (any pairing works as long as A and B agree):
+        // 16 consecutive k per lane, which a [row][k] operand delivers as four 16-byte reads
+        const float* pa = As + cur * SLAB + (kh + 16 * lk) * ska + (wm + lr) * sra;
+        const float* pb = Bs + cur * SLAB + (kh + 16 * lk) * skb + (wn + lr) * srb;
         float av[BK / 4], bv[BK / 4];  // this wavefront's 16 operand pairs of the slab, requested together
 #pragma unroll
-        for (int i = 0; i < BK / 4; ++i) { av[i] = pa[2 * i * ska]; bv[i] = pb[2 * i * skb]; }
+        for (int i = 0; i < BK / 4; ++i) { av[i] = pa[i * ska]; bv[i] = pb[i * skb]; }
         __builtin_amdgcn_sched_barrier(0);  // keep the reads together: sunk next to their MFMA each would be waited for alone
 #pragma unroll
         for (int i = 0; i < BK / 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[i], acc, 0, 0, 0);
         if (more) {  // slab kt-1's buffer: every wavefront left it before the barrier that ended kt-1
-            stage(As + nxt * SLAB, fa, g.a_kmajor, t);
-            stage(Bs + nxt * SLAB, fb, g.b_kmajor, t);
+            stage(As + nxt * SLAB, fa, AKM, t);
+            stage(Bs + nxt * SLAB, fb, BKM, t);
         }
         __syncthreads();
     }
@@ -176,16 +178,22 @@ hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s)
     if (a.M <= 0 || a.N <= 0 || a.K <= 0) return hipErrorInvalidValue;
     dim3 grid((a.N + BN - 1) / BN, (a.M + BM - 1) / BM);
     constexpr size_t lds_bytes = sizeof(float) * 2 * NST * SLAB;  // 104 448 B: above the 64 KiB default
-    static bool raised = false;
-    if (!raised) {
-        hipError_t e = hipFuncSetAttribute((const void*)gemm_f32_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void*)gemm_f32_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return e;
-        raised = true;
-    }
     const bool a_fast = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((a.a_kmajor ? a.M : a.K) % 4) == 0;
     const bool b_fast = (a.ldb % 4) == 0 && ((uintptr_t)a.B % 16) == 0 && ((a.b_kmajor ? a.N : a.K) % 4) == 0;
-    if (a_fast && b_fast) hipLaunchKernelGGL(gemm_f32_kernel<true>, grid, dim3(NTHR), lds_bytes, s, a);
-    else hipLaunchKernelGGL(gemm_f32_kernel<false>, grid, dim3(NTHR), lds_bytes, s, a);
+    typedef void (*kernel_t)(GemmF32Args);
+    static const kernel_t table[2][2][2] = {
+        {{gemm_f32_kernel<false, false, false>, gemm_f32_kernel<false, false, true>},
+         {gemm_f32_kernel<false, true, false>, gemm_f32_kernel<false, true, true>}},
+        {{gemm_f32_kernel<true, false, false>, gemm_f32_kernel<true, false, true>},
+         {gemm_f32_kernel<true, true, false>, gemm_f32_kernel<true, true, true>}}};
+    static bool raised = false;
+    if (!raised) {
+        for (int i = 0; i < 8; ++i) {
+            hipError_t e = hipFuncSetAttribute((const void*)table[i >> 2][(i >> 1) & 1][i & 1], hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return e;
+        }
+        raised = true;
+    }
+    hipLaunchKernelGGL(table[a_fast && b_fast][a.a_kmajor ? 1 : 0][a.b_kmajor ? 1 : 0], grid, dim3(NTHR), lds_bytes, s, a);
     return hipGetLastError();
 }
