@@ -50,13 +50,13 @@ def build_all(verbose=False):
     host_srcs = sorted(os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".cpp")) if os.path.isdir(HOST) else []
     if host_srcs:
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(HERE, "..", "include"),
-              "-o", HOST_LIB] + host_srcs + ["-L", HERE, "-lglades_hip", "-Wl,-rpath,$ORIGIN"])
+              "-pthread", "-o", HOST_LIB] + host_srcs + ["-L", HERE, "-lglades_hip", "-Wl,-rpath,$ORIGIN"])
         # driver of the C++ class API used by tests/test_host_api.py (built here, run on the GPU box)
         check_src = os.path.join(HERE, "..", "tests", "host_api_check.cpp")
         if os.path.exists(check_src):
             bindir = os.path.join(HERE, "..", "tests", "bin")
             os.makedirs(bindir, exist_ok=True)
-            _run(["g++", "-O2", "-std=c++17", "-Wall", "-I", HOST, "-I", os.path.join(HERE, "..", "include"),
+            _run(["g++", "-O2", "-std=c++17", "-Wall", "-pthread", "-I", HOST, "-I", os.path.join(HERE, "..", "include"),
                   "-o", os.path.join(bindir, "host_api_check"), check_src, "-L", HERE, "-lglades_host", "-lglades_hip",
                   "-Wl,-rpath,$ORIGIN/../../glades-ml_amd", "-Wl,-rpath-link," + HERE, "-L/opt/rocm/lib", "-Wl,-rpath-link,/opt/rocm/lib"])
     return LIB

@@ -61,6 +61,8 @@ struct ghip_net {
     int exMetricsCap = 0;
     int64_t exPredsCap = 0;
     int* exEpochs = nullptr;
+    ExactPointers* exMulti = nullptr;  // pointer list of a launch over several networks (held by the first one)
+    int exMultiCap = 0;
     int* cm = nullptr;              // confusion counters (both modes), n_out x n_out
     float* exClass = nullptr;       // exact mode: 5 floats per epoch of the last call
     int exClassCap = 0, exClassRan = 0;
@@ -249,7 +251,7 @@ int setup_exact(ghip_net* n)
     HIP_TRY(hipMemsetAsync(n->exSum, 0, sizeof(float) * woff, n->stream));
     HIP_TRY(hipMemsetAsync(n->exLast, 0, sizeof(float) * woff, n->stream));
     HIP_TRY(hipMemsetAsync(n->exBias, 0, sizeof(float) * GHIP_MAX_LAYERS, n->stream));
-    e.W = n->exW; e.wsum = n->exSum; e.wlast = n->exLast; e.bias = n->exBias; e.epochs_run = n->exEpochs;
+    e.ptr.W = n->exW; e.ptr.wsum = n->exSum; e.ptr.wlast = n->exLast; e.ptr.bias = n->exBias; e.ptr.epochs_run = n->exEpochs;
     return 0;
 }
 
@@ -563,6 +565,7 @@ int ghip_net_create(const ghip_net_spec* spec, ghip_net** out)
     if (!out) return fail(GHIP_EINVAL, "out is NULL");
     *out = nullptr;
     if (g_device < 0) TRY(ghip_init(0));
+    HIP_TRY(hipSetDevice(g_device));  // the calling thread may be a fresh one (one host thread per MetaNetwork subnet)
     TRY(check_spec(spec));
     ghip_net* n = new ghip_net();
     n->spec = *spec;
@@ -583,7 +586,7 @@ int ghip_net_destroy(ghip_net* n)
     free_batch_buffers(n);
     dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf);
     dfree(n->exW); dfree(n->exSum); dfree(n->exLast); dfree(n->exBias); dfree(n->exPreds);
-    dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass);
+    dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass); dfree(n->exMulti);
     for (int l = 0; l < GHIP_MAX_LAYERS; ++l) {
         dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]); dfree(n->gW[l]);
         dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
@@ -735,12 +738,9 @@ int ghip_net_set_dataset_device(ghip_net* n, const float* dev_X, const float* de
     return make_bf16_table(n);
 }
 
-int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_accuracy,
-                              ghip_metrics* host_metrics, int* epochs_run, float* host_preds)
+// buffers of one network for a call of n_epochs epochs; fills ptr
+static int exact_prepare(ghip_net* n, int n_epochs, bool want_preds, ExactPointers* ptr)
 {
-    if (!n || n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
-    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "network is not in exact mode");
-    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     const int nout = n->spec.sizes[n->L];
     if (n_epochs > n->exMetricsCap) {
         HIP_TRY(hipStreamSynchronize(n->stream));
@@ -748,19 +748,17 @@ int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_a
         TRY(dalloc(&n->exMetrics, (size_t)n_epochs));
         n->exMetricsCap = n_epochs;
     }
-    if (host_preds && n->n_rows * nout > n->exPredsCap) {
+    if (want_preds && n->n_rows * nout > n->exPredsCap) {
         HIP_TRY(hipStreamSynchronize(n->stream));
         dfree(n->exPreds);
         TRY(dalloc(&n->exPreds, (size_t)n->n_rows * nout));
         n->exPredsCap = n->n_rows * nout;
     }
-    ExactLaunch e = n->ex;
-    e.X = n->dX; e.Y = n->dY; e.n_rows = n->n_rows;
-    e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
-    e.preds = host_preds ? n->exPreds : nullptr;
-    e.metrics = (float*)n->exMetrics;
-    e.cm = n->cm;
-    e.class_metrics = nullptr;
+    *ptr = n->ex.ptr;
+    ptr->preds = want_preds ? n->exPreds : nullptr;
+    ptr->metrics = (float*)n->exMetrics;
+    ptr->cm = n->cm;
+    ptr->class_metrics = nullptr;
     if (n->cm && nout <= 64) {
         if (n_epochs > n->exClassCap) {
             HIP_TRY(hipStreamSynchronize(n->stream));
@@ -768,23 +766,86 @@ int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_a
             TRY(dalloc(&n->exClass, (size_t)n_epochs * 5));
             n->exClassCap = n_epochs;
         }
-        e.class_metrics = n->exClass;
+        ptr->class_metrics = n->exClass;
     }
     n->exClassRan = 0;
-    LAUNCH(n, "exact_epochs", ghip_launch_exact(e, n->ex_threads, n->ex_lds, n->stream));
+    return 0;
+}
+
+int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_accuracy,
+                              ghip_metrics* host_metrics, int* epochs_run, float* host_preds)
+{
+    if (!n || n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
+    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "network is not in exact mode");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
+    const int nout = n->spec.sizes[n->L];
+    ExactLaunch e = n->ex;
+    TRY(exact_prepare(n, n_epochs, host_preds != nullptr, &e.ptr));
+    e.X = n->dX; e.Y = n->dY; e.n_rows = n->n_rows;
+    e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
+    LAUNCH(n, "exact_epochs", ghip_launch_exact(e, nullptr, 1, n->ex_threads, n->ex_lds, n->stream));
     int ran = 0;
     HIP_TRY(hipMemcpyAsync(&ran, n->exEpochs, sizeof(int), hipMemcpyDeviceToHost, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
     if (epochs_run) *epochs_run = ran;
-    n->exClassRan = e.class_metrics ? ran : 0;
+    n->exClassRan = e.ptr.class_metrics ? ran : 0;
     if (host_metrics && ran > 0) HIP_TRY(hipMemcpy(host_metrics, n->exMetrics, sizeof(ghip_metrics) * ran, hipMemcpyDeviceToHost));
     if (host_preds) HIP_TRY(hipMemcpy(host_preds, n->exPreds, sizeof(float) * n->n_rows * nout, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epochs, int train, float stop_accuracy,
+                                    ghip_metrics* host_metrics, int* epochs_run)
+{
+    if (!nets || count < 1 || n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
+    ghip_net* lead = nets[0];
+    for (int k = 0; k < count; ++k) {
+        ghip_net* n = nets[k];
+        if (!n) return fail(GHIP_EINVAL, "network %d is NULL", k);
+        for (int j = 0; j < k; ++j)
+            if (nets[j] == n) return fail(GHIP_EINVAL, "network %d appears twice", k);
+        if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "network %d is not in exact mode", k);
+        if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "network %d has no dataset", k);
+        // one launch = one architecture, one schedule, one table: everything but the parameters is shared
+        if (memcmp(&n->spec, &lead->spec, sizeof(ghip_net_spec)) != 0) return fail(GHIP_EINVAL, "network %d differs from network 0 in its specification", k);
+        if (n->n_rows != lead->n_rows) return fail(GHIP_EINVAL, "network %d has a table of another length", k);
+    }
+    std::vector<ExactPointers> list(count);
+    for (int k = 0; k < count; ++k) {
+        TRY(exact_prepare(nets[k], n_epochs, false, &list[k]));
+        if (nets[k] != lead) HIP_TRY(hipStreamSynchronize(nets[k]->stream));  // its earlier work is done before lead's stream touches its arrays
+    }
+    if (count > lead->exMultiCap) {
+        HIP_TRY(hipStreamSynchronize(lead->stream));
+        dfree(lead->exMulti);
+        TRY(dalloc(&lead->exMulti, (size_t)count));
+        lead->exMultiCap = count;
+    }
+    HIP_TRY(hipMemcpyAsync(lead->exMulti, list.data(), sizeof(ExactPointers) * count, hipMemcpyHostToDevice, lead->stream));
+    ExactLaunch e = lead->ex;
+    // each network reads its own copy of the table (identical content is the caller's business: the
+    // reference trains every subnet of a MetaNetwork on the same DataInput, ML/main.cpp:137-160)
+    e.X = lead->dX; e.Y = lead->dY; e.n_rows = lead->n_rows;
+    e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
+    LAUNCH(lead, "exact_epochs_multi", ghip_launch_exact(e, lead->exMulti, count, lead->ex_threads, lead->ex_lds, lead->stream));
+    HIP_TRY(hipStreamSynchronize(lead->stream));
+    for (int k = 0; k < count; ++k) {
+        int ran = 0;
+        HIP_TRY(hipMemcpy(&ran, nets[k]->exEpochs, sizeof(int), hipMemcpyDeviceToHost));
+        if (epochs_run) epochs_run[k] = ran;
+        nets[k]->exClassRan = list[k].class_metrics ? ran : 0;
+        if (host_metrics && ran > 0)
+            HIP_TRY(hipMemcpy(host_metrics + (size_t)k * n_epochs, nets[k]->exMetrics, sizeof(ghip_metrics) * ran, hipMemcpyDeviceToHost));
+    }
     return 0;
 }
 
 int ghip_net_train_step(ghip_net* n, int64_t row0, int batch, ghip_metrics* host_metrics)
 {
     if (!n || batch < 1 || row0 < 0) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
     if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
     if (n->spec.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "fp8 networks are inference only");
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");

@@ -40,11 +40,16 @@ __device__ __forceinline__ float bias_chain(float b, const float* bs, int no, in
     return b;
 }
 
+// One workgroup per network: `p` describes the (shared) architecture, hyper-parameters and data
+// table; with `multi` each workgroup b takes its own parameter / result pointers from multi[b]
+// (the subnets of a MetaNetwork train at the same time, one per compute unit), without it the
+// single network's pointers are the ones in `p`.
 template <bool kLds>
 __global__ void __launch_bounds__(1024)
-exact_kernel(ExactLaunch p)
+exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 {
     extern __shared__ float smem[];
+    const ExactPointers own = multi ? multi[blockIdx.x] : p.ptr;
     const int tid = threadIdx.x;
     const int T = blockDim.x;
     const int serial = T - 1;  // lane that carries the order-dependent scalar chains
@@ -63,9 +68,9 @@ exact_kernel(ExactLaunch p)
         sLast = smem + 2 * S;
         nodes = smem + 3 * S;
     } else {
-        sW = p.W;
-        sSum = p.wsum;
-        sLast = p.wlast;
+        sW = own.W;
+        sSum = own.wsum;
+        sLast = own.wlast;
         nodes = smem;
     }
     float* sa = nodes;                      // node values, all layers
@@ -77,12 +82,12 @@ exact_kernel(ExactLaunch p)
 
     if (kLds) {
         for (int k = tid; k < S; k += T) {
-            sW[k] = p.W[k];
-            sSum[k] = p.wsum[k];
-            sLast[k] = p.wlast[k];
+            sW[k] = own.W[k];
+            sSum[k] = own.wsum[k];
+            sLast[k] = own.wlast[k];
         }
     }
-    if (tid < GHIP_MAX_LAYERS) sbias[tid] = p.bias[tid];
+    if (tid < GHIP_MAX_LAYERS) sbias[tid] = own.bias[tid];
     if (tid == 0) sflag[0] = 0;
 
     const float data_size = (float)((unsigned)p.n_rows * (unsigned)nout);
@@ -104,8 +109,8 @@ exact_kernel(ExactLaunch p)
         float tot_err = 0.0f, tot_acc = 0.0f;
         long long correct = 0;
         const bool last_epoch = (ep == p.n_epochs - 1) || (p.stop_accuracy > 0.0f);
-        if (p.cm) {  // CMatrix::reset at the head of every epoch (network.cpp:183-185)
-            for (int k = tid; k < nout * nout; k += T) p.cm[k] = 0;
+        if (own.cm) {  // CMatrix::reset at the head of every epoch (network.cpp:183-185)
+            for (int k = tid; k < nout * nout; k += T) own.cm[k] = 0;
             __threadfence();
             __syncthreads();
         }
@@ -154,8 +159,8 @@ exact_kernel(ExactLaunch p)
                 __syncthreads();
             }
             const float* pred = sa + p.aoff[L];
-            if (p.preds && last_epoch)
-                for (int o = tid; o < nout; o += T) p.preds[r * nout + o] = pred[o];
+            if (own.preds && last_epoch)
+                for (int o = tid; o < nout; o += T) own.preds[r * nout + o] = pred[o];
 
             // ---- output metrics in visiting order (network.cpp:519-559)
             if (tid == serial) {
@@ -170,7 +175,7 @@ exact_kernel(ExactLaunch p)
                 }
                 if (ip == iy) ++correct;
                 // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
-                if (p.cm && ip >= 0 && iy >= 0) atomicAdd(&p.cm[iy * nout + ip], 1);
+                if (own.cm && ip >= 0 && iy >= 0) atomicAdd(&own.cm[iy * nout + ip], 1);
             }
 
             if (p.train) {
@@ -274,13 +279,13 @@ exact_kernel(ExactLaunch p)
         // ---- end of epoch (network.cpp:193-195, Terminator.cpp:73-74)
         if (tid == serial) {
             float acc = __fdiv_rn(tot_acc, __fmul_rn((float)(unsigned)p.n_rows, (float)(unsigned)nout));
-            ghip_metrics* m = ((ghip_metrics*)p.metrics) + ep;
+            ghip_metrics* m = ((ghip_metrics*)own.metrics) + ep;
             m->loss = tot_err;
             m->accuracy = acc;
             m->correct = correct;
-            if (p.cm && p.class_metrics) {  // network.cpp:218-224, read back through the atomics' path
+            if (own.cm && own.class_metrics) {  // network.cpp:218-224, read back through the atomics' path
                 __threadfence();
-                ghip_cmatrix_overall(p.cm, nout, p.class_metrics + 5 * ep);
+                ghip_cmatrix_overall(own.cm, nout, own.class_metrics + 5 * ep);
             }
             if (p.stop_accuracy > 0.0f && acc >= p.stop_accuracy) sflag[0] = 1;
         }
@@ -290,13 +295,13 @@ exact_kernel(ExactLaunch p)
 
     if (kLds) {
         for (int k = tid; k < S; k += T) {
-            p.W[k] = sW[k];
-            p.wsum[k] = sSum[k];
-            p.wlast[k] = sLast[k];
+            own.W[k] = sW[k];
+            own.wsum[k] = sSum[k];
+            own.wlast[k] = sLast[k];
         }
     }
-    if (tid < GHIP_MAX_LAYERS) p.bias[tid] = sbias[tid];
-    if (tid == 0) p.epochs_run[0] = ep;
+    if (tid < GHIP_MAX_LAYERS) own.bias[tid] = sbias[tid];
+    if (tid == 0) own.epochs_run[0] = ep;
 }
 
 }  // namespace
@@ -308,16 +313,17 @@ size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds)
     return f * sizeof(float);
 }
 
-hipError_t ghip_launch_exact(const ExactLaunch& p, int threads, size_t lds_bytes, hipStream_t s)
+hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads, size_t lds_bytes,
+                             hipStream_t s)
 {
     hipError_t e;
     if (p.state_in_lds) {
         e = hipFuncSetAttribute((const void*)exact_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)lds_bytes);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(exact_kernel<true>, dim3(1), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(exact_kernel<true>, dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
     } else {
-        hipLaunchKernelGGL(exact_kernel<false>, dim3(1), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(exact_kernel<false>, dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
     }
     return hipGetLastError();
 }

@@ -200,6 +200,19 @@ __device__ __forceinline__ uint8_t ghip_f32_to_e4m3(float x)
 
 // ---------------------------------------------------------------- exact mode (exact_kernel.hip)
 
+// What differs between the networks of one launch: parameters, state and results.
+struct ExactPointers {
+    float* W;      // [state_floats] padded weights (global copy, read at start, written at end)
+    float* wsum;   // pending-delta running sums
+    float* wlast;  // last pending delta
+    float* bias;   // [GHIP_MAX_LAYERS] scalar layer biases
+    float* preds;  // n_rows x n_out or NULL
+    float* metrics;// per epoch: loss, accuracy, correct
+    int*   epochs_run;
+    int*   cm;            // n_out x n_out confusion counters of the running epoch, or NULL
+    float* class_metrics; // per epoch: overall accuracy, precision, recall, specificity, F1 (NULL with cm)
+};
+
 struct ExactLaunch {
     int   n_layers;
     int   sizes[GHIP_MAX_LAYERS + 1];
@@ -218,19 +231,13 @@ struct ExactLaunch {
     long long n_rows;
     const float* X;
     const float* Y;
-    float* W;      // [state_floats] padded weights (global copy, read at start, written at end)
-    float* wsum;   // pending-delta running sums
-    float* wlast;  // last pending delta
-    float* bias;   // [GHIP_MAX_LAYERS] scalar layer biases
-    float* preds;  // n_rows x n_out or NULL
-    float* metrics;// per epoch: loss, accuracy, correct (as float bits of an int), spare
-    int*   epochs_run;
+    ExactPointers ptr;  // this network's own arrays (a launch over several networks passes a list instead)
     int    state_in_lds;
-    int*   cm;            // n_out x n_out confusion counters of the running epoch, or NULL
-    float* class_metrics; // per epoch: overall accuracy, precision, recall, specificity, F1 (NULL with cm)
 };
 
-hipError_t ghip_launch_exact(const ExactLaunch& p, int threads, size_t lds_bytes, hipStream_t s);
+// count workgroups = count networks; dev_multi (device memory, count entries) or NULL for the one network in p.ptr
+hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads, size_t lds_bytes,
+                             hipStream_t s);
 size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds);
 
 // ---------------------------------------------------------------- canonical kernels

@@ -7,6 +7,7 @@
 #include <stdlib.h>
 #include <string.h>
 #include <time.h>
+#include <thread>
 
 #include "glades_hip.h"
 
@@ -326,7 +327,7 @@ static int64_t g_next_id = 1;
 
 NNetwork::NNetwork()
     : di(NULL), skeleton(NULL), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
-      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
+      dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
       minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
 {
@@ -334,7 +335,7 @@ NNetwork::NNetwork()
 
 NNetwork::NNetwork(NNInfo* newNNInfo)
     : di(NULL), skeleton(newNNInfo), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
-      dtype(DTYPE_F32), biasMode(0), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
+      dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
       minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
 {
@@ -891,24 +892,77 @@ void CMatrix::clean()
     matrix.clear(); truePositive.clear(); trueNegative.clear(); falsePositive.clear(); falseNegative.clear();
 }
 
-// NNetwork::run (ML/Networks/network.cpp:114-397)
-void NNetwork::run(DataInput* newDataInput, int runType)
+bool NNetwork::prepare(DataInput* newDataInput)
 {
-    if (!skeleton) return;
-    if (!newDataInput) return;
+    if (!skeleton) return false;
+    if (!newDataInput) return false;
     di = newDataInput;
-    if ((di->getTrainSize() <= 0) || (di->getFeatureCount() <= 0)) return;
+    if ((di->getTrainSize() <= 0) || (di->getFeatureCount() <= 0)) return false;
     if (!dev) {  // network.cpp:127-128 builds when epochs == 0; a restored checkpoint arrives with its epoch count
         if (!build()) {
             if (dev) ghip_net_destroy(dev);
             dev = NULL;
-            return;
+            return false;
         }
     }
-    if (!dev) return;
     minibatchSize = skeleton->getBatchSize();
-    if (runType == RUN_TRAIN) printf("[NN] Training...\n");
-    else if (runType == RUN_TEST) printf("[NN] Testing...\n");
+    return dev != NULL;
+}
+
+// what follows a batch of epochs (network.cpp:193-258): statistics of the last one, class figures, progress line
+void NNetwork::afterEpochs(const void* lastMetrics, int ran, int runType)
+{
+    const ghip_metrics* m = (const ghip_metrics*)lastMetrics;
+    epochs += ran;
+    overallTotalError = m->loss;
+    overallTotalAccuracy = m->accuracy;
+    overallCorrect = m->correct;
+    const bool classes = confusionMatrix.size() > 0;
+    if (classes) {
+        // network.cpp:218-224: the device counted the last epoch's cells; the ratios are CMatrix's
+        std::vector<int> cells((size_t)nOut * nOut);
+        if (ghip_net_confusion_get(dev, cells.data(), (int64_t)cells.size()) == 0) {
+            confusionMatrix.reset();
+            confusionMatrix.setMatrix(cells);
+            confusionMatrix.updateResultParams();
+            overallClassAccuracy = confusionMatrix.getOverallAccuracy() * 100.0f;
+            overallClassPrecision = confusionMatrix.getOverallPrecision() * 100.0f;
+            overallClassRecall = confusionMatrix.getOverallRecall() * 100.0f;
+            overallClassSpecificity = confusionMatrix.getOverallSpecificity() * 100.0f;
+            overallClassF1 = confusionMatrix.getOverallF1Score() * 100.0f;
+        }
+    }
+    if (verbose && runType == RUN_TRAIN) {
+        if (classes)
+            printf("\33[2K[NN] %d\t%s%f%%\t%f%%\t%f%%\t%f%%\t%f%%\r", epochs, epochs < 100 ? "\t" : "", overallClassAccuracy,
+                   overallClassPrecision, overallClassRecall, overallClassSpecificity, overallClassF1);
+        else
+            printf("\33[2K[NN] %d\t%f%%\r", epochs, overallTotalAccuracy);
+        fflush(stdout);
+    }
+}
+
+namespace {
+// several epochs per launch where the stop conditions allow it: up to the next epoch multiple,
+// 1 when a wall-clock condition has to be polled every epoch or for the test pass
+int epochChunk(const Terminator& t, int epochs, int runType)
+{
+    if (runType == NNetwork::RUN_TEST || t.getTimestamp() > 0) return 1;
+    if (t.getEpoch() > 0) {
+        const int64_t e = t.getEpoch();
+        const int64_t left = e - ((int64_t)epochs % e);
+        return (int)(left < 4096 ? left : 4096);
+    }
+    return 16;
+}
+}  // namespace
+
+// NNetwork::run (ML/Networks/network.cpp:114-397)
+void NNetwork::run(DataInput* newDataInput, int runType)
+{
+    if (!prepare(newDataInput)) return;
+    if (verbose && runType == RUN_TRAIN) printf("[NN] Training...\n");
+    else if (verbose && runType == RUN_TEST) printf("[NN] Testing...\n");
 
     const bool want_preds = (size_t)nRows * nOut <= (1u << 20);
     std::vector<float> preds(want_preds ? (size_t)nRows * nOut : 0);
@@ -916,15 +970,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
     running = true;
     while (running) {
         if (mode == MODE_EXACT) {
-            // several epochs per launch where the stop conditions allow it: up to the next epoch
-            // multiple, 1 when a wall-clock condition has to be polled every epoch
-            int chunk = 16;
-            if (runType == RUN_TEST || terminator.getTimestamp() > 0) chunk = 1;
-            else if (terminator.getEpoch() > 0) {
-                const int64_t e = terminator.getEpoch();
-                int64_t left = e - ((int64_t)epochs % e);
-                chunk = (int)(left < 4096 ? left : 4096);
-            }
+            const int chunk = epochChunk(terminator, epochs, runType);
             std::vector<ghip_metrics> ms(chunk);
             int ran = 0;
             if (ghip_net_run_epochs_exact(dev, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran,
@@ -933,10 +979,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
                 break;
             }
             if (ran <= 0) break;
-            epochs += ran;
-            overallTotalError = ms[ran - 1].loss;
-            overallTotalAccuracy = ms[ran - 1].accuracy;
-            overallCorrect = ms[ran - 1].correct;
+            afterEpochs(&ms[ran - 1], ran, runType);
         } else {
             if (confusionMatrix.size() > 0) ghip_net_confusion_reset(dev);  // network.cpp:183-185
             // canonical mode: batches [k*mb, (k+1)*mb), the last one averaged over its true size
@@ -952,33 +995,9 @@ void NNetwork::run(DataInput* newDataInput, int runType)
                 loss += (double)m.loss * b; acc += (double)m.accuracy * b; correct += m.correct;
             }
             if (failed) break;
-            ++epochs;
-            overallTotalError = (float)(loss / nRows);
-            overallTotalAccuracy = (float)(acc / nRows);
-            overallCorrect = correct;
-        }
-        const bool classes = confusionMatrix.size() > 0;
-        if (classes) {
-            // network.cpp:218-224: the device counted the last epoch's cells; the ratios are CMatrix's
-            std::vector<int> cells((size_t)nOut * nOut);
-            if (ghip_net_confusion_get(dev, cells.data(), (int64_t)cells.size()) == 0) {
-                confusionMatrix.reset();
-                confusionMatrix.setMatrix(cells);
-                confusionMatrix.updateResultParams();
-                overallClassAccuracy = confusionMatrix.getOverallAccuracy() * 100.0f;
-                overallClassPrecision = confusionMatrix.getOverallPrecision() * 100.0f;
-                overallClassRecall = confusionMatrix.getOverallRecall() * 100.0f;
-                overallClassSpecificity = confusionMatrix.getOverallSpecificity() * 100.0f;
-                overallClassF1 = confusionMatrix.getOverallF1Score() * 100.0f;
-            }
-        }
-        if (runType == RUN_TRAIN) {
-            if (classes)
-                printf("\33[2K[NN] %d\t%s%f%%\t%f%%\t%f%%\t%f%%\t%f%%\r", epochs, epochs < 100 ? "\t" : "", overallClassAccuracy,
-                       overallClassPrecision, overallClassRecall, overallClassSpecificity, overallClassF1);
-            else
-                printf("\33[2K[NN] %d\t%f%%\r", epochs, overallTotalAccuracy);
-            fflush(stdout);
+            ghip_metrics last;
+            last.loss = (float)(loss / nRows); last.accuracy = (float)(acc / nRows); last.correct = correct;
+            afterEpochs(&last, 1, runType);
         }
         if (terminator.triggered(time(NULL), epochs, overallTotalAccuracy)) break;
         if (runType == RUN_TEST) break;
@@ -990,9 +1009,60 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             results.push_back(preds[(size_t)(nRows - 1) * nOut + o]);
         }
     }
-    if (runType == RUN_TRAIN) printf("\n");
-    else if (runType == RUN_TEST) printf("[NN] %s Accuracy: %f%%\n", skeleton->getName().c_str(), overallTotalAccuracy);
+    if (verbose && runType == RUN_TRAIN) printf("\n");
+    else if (verbose && runType == RUN_TEST) printf("[NN] %s Accuracy: %f%%\n", skeleton->getName().c_str(), overallTotalAccuracy);
     running = false;
+}
+
+// Subnets that are the same network in everything but their parameters (exact mode, equal tables,
+// equal epoch counters and stop conditions) train in ONE kernel launch per chunk of epochs, a
+// workgroup each; a subnet that meets its stop condition leaves the group.
+bool MetaNetwork::runGroup(DataInput* d, int runType)
+{
+    std::vector<NNetwork*> act;
+    for (size_t i = 0; i < subnets.size(); ++i) {
+        NNetwork* n = subnets[i];
+        if (!n || !n->skeleton || n->mode != NNetwork::MODE_EXACT) return false;
+        NNetwork* a = subnets[0];
+        if (n->epochs != a->epochs || n->biasMode != a->biasMode || n->skeleton->toTable() != a->skeleton->toTable()) return false;
+        if (n->terminator.getEpoch() != a->terminator.getEpoch() || n->terminator.getAccuracy() != a->terminator.getAccuracy() ||
+            n->terminator.getTimestamp() != 0) return false;
+    }
+    for (size_t i = 0; i < subnets.size(); ++i) {
+        if (!subnets[i]->prepare(d)) return false;
+        subnets[i]->running = true;
+        act.push_back(subnets[i]);
+    }
+    while (!act.empty()) {
+        const int chunk = epochChunk(act[0]->terminator, act[0]->epochs, runType);
+        std::vector<ghip_net*> handles(act.size());
+        for (size_t i = 0; i < act.size(); ++i) handles[i] = act[i]->dev;
+        std::vector<ghip_metrics> ms((size_t)chunk * act.size());
+        std::vector<int> ran(act.size(), 0);
+        if (ghip_net_run_epochs_exact_multi(handles.data(), (int)act.size(), chunk, runType == NNetwork::RUN_TRAIN ? 1 : 0,
+                                            act[0]->terminator.getAccuracy(), ms.data(), ran.data()) != 0) {
+            for (size_t i = 0; i < act.size(); ++i) { act[i]->lastError = ghip_last_error(); act[i]->running = false; }
+            return true;
+        }
+        std::vector<NNetwork*> next;
+        for (size_t i = 0; i < act.size(); ++i) {
+            NNetwork* n = act[i];
+            if (ran[i] <= 0) { n->running = false; continue; }
+            n->afterEpochs(&ms[i * chunk + ran[i] - 1], ran[i], runType);
+            const bool done = !n->running || n->terminator.triggered(time(NULL), n->epochs, n->overallTotalAccuracy) || runType == NNetwork::RUN_TEST;
+            if (done) n->running = false;
+            else next.push_back(n);
+        }
+        // the survivors share a launch only while their epoch counters agree
+        for (size_t i = 1; i < next.size(); ++i)
+            if (next[i]->epochs != next[0]->epochs) {
+                for (size_t k = 0; k < next.size(); ++k) { next[k]->running = false; next[k]->run(d, runType); }
+                next.clear();
+                break;
+            }
+        act.swap(next);
+    }
+    return true;
 }
 
 // ------------------------------------------------------------------ facade (ML/main.cpp:51-243)
@@ -1013,12 +1083,47 @@ MetaNetwork* train(NNInfo* info, DataInput* d)
     return train(new NNetwork(info), d);
 }
 
+namespace {
+// runs fn(subnet) for every subnet: one host thread each when the MetaNetwork is concurrent (the
+// device work of different networks lives on different streams), else in order
+template <typename Fn>
+void for_each_subnet(MetaNetwork* m, Fn fn)
+{
+    const std::vector<NNetwork*>& nets = m->getSubnets();
+    if (!m->getConcurrent() || nets.size() < 2) {
+        for (size_t i = 0; i < nets.size(); ++i)
+            if (nets[i]) fn(nets[i]);
+        return;
+    }
+    std::vector<std::thread> pool;
+    for (size_t i = 0; i < nets.size(); ++i)
+        if (nets[i]) pool.push_back(std::thread(fn, nets[i]));
+    for (size_t i = 0; i < pool.size(); ++i) pool[i].join();
+}
+}  // namespace
+
 MetaNetwork* train(MetaNetwork* m, DataInput* d)
 {
     if (!m || !d) return NULL;
-    for (unsigned int i = 0; i < m->size(); ++i)
-        if (m->getSubnets()[i]) m->getSubnets()[i]->train(d);
+    if (m->getConcurrent() && m->size() > 1 && m->runGroup(d, NNetwork::RUN_TRAIN)) return m;
+    for_each_subnet(m, [d](NNetwork* n) { n->train(d); });
     return m;
+}
+
+float MetaNetwork::crossValidate(DataInput* newDataInput)
+{
+    if (!newDataInput || subnets.empty()) return 0.0f;
+    if (concurrent && subnets.size() > 1 && runGroup(newDataInput, NNetwork::RUN_TRAIN)) {
+        if (!runGroup(newDataInput, NNetwork::RUN_TEST))
+            for_each_subnet(this, [newDataInput](NNetwork* n) { n->test(newDataInput); });
+    } else {
+        for_each_subnet(this, [newDataInput](NNetwork* n) { n->train(newDataInput); n->test(newDataInput); });
+    }
+    float cvAccuracy = 0.0f;
+    for (size_t i = 0; i < subnets.size(); ++i)
+        if (subnets[i]) cvAccuracy += subnets[i]->getAccuracy();
+    printf("cvAccuracy: %f \t\n", cvAccuracy / subnets.size());
+    return cvAccuracy / subnets.size();
 }
 
 MetaNetwork* test(NNetwork* net, DataInput* d)
@@ -1038,8 +1143,8 @@ MetaNetwork* test(NNInfo* info, DataInput* d)
 MetaNetwork* test(MetaNetwork* m, DataInput* d)
 {
     if (!m || !d) return NULL;
-    for (unsigned int i = 0; i < m->size(); ++i)
-        if (m->getSubnets()[i]) m->getSubnets()[i]->test(d);
+    if (m->getConcurrent() && m->size() > 1 && m->runGroup(d, NNetwork::RUN_TEST)) return m;
+    for_each_subnet(m, [d](NNetwork* n) { n->test(d); });
     return m;
 }
 

@@ -322,6 +322,7 @@ class NNetwork
     ghip_net* dev;
     volatile bool running;
     int netType, epochs, mode, dtype, biasMode;
+    bool verbose;
     float overallTotalError, overallTotalAccuracy;
     float overallClassAccuracy, overallClassPrecision, overallClassRecall, overallClassSpecificity, overallClassF1;
     CMatrix confusionMatrix;
@@ -336,6 +337,8 @@ class NNetwork
     std::string lastError;
 
     void run(DataInput*, int);
+    bool prepare(DataInput*);                        // checks + build on first use
+    void afterEpochs(const void* lastMetrics, int ran, int runType);  // statistics, class figures, progress line
     bool build();
     void clean();
 
@@ -379,6 +382,7 @@ public:
     const CMatrix& getConfusionMatrix() const { return confusionMatrix; }
     void setMode(int newMode, int newDtype = DTYPE_F32) { mode = newMode; dtype = newDtype; }
     void setSequentialBias(bool faithful) { biasMode = faithful ? 0 : 1; }
+    void setVerbose(bool v) { verbose = v; }  // the per-epoch progress line and the [NN] banners
     // layer = weight layer 0..numHiddenLayers(); W is [n_out][n_in] row-major
     bool setWeights(unsigned int layer, const std::vector<float>& W);
     bool setBias(unsigned int layer, const std::vector<float>& bias);  // 1 value (exact) or n_out
@@ -397,9 +401,25 @@ class MetaNetwork
 {
     std::string name;
     std::vector<NNetwork*> subnets;
+    bool concurrent;
 
 public:
-    explicit MetaNetwork(const std::string& newName) : name(newName) {}
+    explicit MetaNetwork(const std::string& newName) : name(newName), concurrent(true) {}
+    // Subnets are independent networks (metanetwork.cpp:86-127): with `concurrent` (the default) train /
+    // test / crossValidate run them at the same time, one host thread and one HIP stream each, instead
+    // of one after the other as the reference's loop does (ML/main.cpp:137-160).  Results are the same.
+    void setConcurrent(bool v) { concurrent = v; }
+    bool getConcurrent() const { return concurrent; }
+    void addSubnet(NNInfo* info) { if (info) subnets.push_back(new NNetwork(info)); }  // metanetwork.cpp:95-102
+    NNetwork* getSubnet(unsigned int i) { return i < subnets.size() ? subnets[i] : NULL; }
+    void clearSubnets() { subnets.clear(); }
+    // metanetwork.cpp:216-251: every subnet trains on the data, then runs the test pass; prints and
+    // returns the mean test accuracy.  (The reference splits the file into k stratified folds with the
+    // un-vendored GTable::stratify and then passes the WHOLE DataInput to every subnet all the same;
+    // this does what that code does, without the unused split.)
+    float crossValidate(DataInput* newDataInput);
+    // one kernel launch for all subnets where they allow it (see glades.cpp); false = not applicable
+    bool runGroup(DataInput*, int runType);
     std::string getName() const { return name; }
     void addSubnet(NNetwork* n) { if (n) subnets.push_back(n); }
     const std::vector<NNetwork*>& getSubnets() const { return subnets; }

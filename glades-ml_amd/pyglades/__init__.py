@@ -21,7 +21,7 @@ BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
 EXPORTS = [
     "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
     "ghip_net_get_state", "ghip_net_set_state",
-    "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact",
+    "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
     "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
     "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
@@ -82,6 +82,7 @@ def load():
             "ghip_net_set_dataset": (i, [vp, vp, vp, i64]),
             "ghip_net_set_dataset_device": (i, [vp, vp, vp, i64]),
             "ghip_net_run_epochs_exact": (i, [vp, i, i, f, vp, C.POINTER(i), vp]),
+            "ghip_net_run_epochs_exact_multi": (i, [vp, i, i, i, f, vp, vp]),
             "ghip_net_train_step": (i, [vp, i64, i, vp]),
             "ghip_net_last_metrics": (i, [vp, C.POINTER(Metrics)]),
             "ghip_net_forward": (i, [vp, vp, i, vp]),
@@ -292,3 +293,17 @@ class Net:
             _check(self.lib.ghip_net_profile_entry(self.h, k, name, 96, C.byref(ms), C.byref(cnt)))
             out[name.value.decode()] = (ms.value, cnt.value)
         return out
+
+
+def run_epochs_exact_multi(nets, n_epochs, train=True, stop_accuracy=0.0):
+    """One launch for several exact-mode networks of one specification.  Returns per network the list
+    of (loss, accuracy, correct) per epoch run."""
+    lib = load()
+    k = len(nets)
+    handles = (C.c_void_p * k)(*[n.h for n in nets])
+    ms = (Metrics * (k * n_epochs))()
+    ran = (C.c_int * k)()
+    _check(lib.ghip_net_run_epochs_exact_multi(C.cast(handles, C.c_void_p), k, n_epochs, 1 if train else 0, float(stop_accuracy),
+                                               C.cast(ms, C.c_void_p), C.cast(ran, C.c_void_p)))
+    return [[(ms[j * n_epochs + e].loss, ms[j * n_epochs + e].accuracy, ms[j * n_epochs + e].correct) for e in range(ran[j])]
+            for j in range(k)]

@@ -136,6 +136,16 @@ int ghip_net_set_dataset_device(ghip_net* net, const float* dev_X, const float* 
 int ghip_net_run_epochs_exact(ghip_net* net, int n_epochs, int train, float stop_accuracy,
                               ghip_metrics* host_metrics, int* epochs_run, float* host_preds);
 
+/* The same for `count` networks of one specification and one table length at once, one workgroup
+ * each: the subnets of a MetaNetwork, which the reference trains one after the other on the same
+ * DataInput (ML/main.cpp:137-160, ML/Networks/metanetwork.cpp:216-251).  Narrow networks are bound
+ * by the latency of their sequential rows, so the device's answer is many of them side by side.
+ * All networks use the table of nets[0] (the caller has given every one the same data).
+ * host_metrics: count x n_epochs entries, row k for nets[k]; epochs_run: count entries.
+ * Every network stops on its own when it reaches stop_accuracy. */
+int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epochs, int train, float stop_accuracy,
+                                    ghip_metrics* host_metrics, int* epochs_run);
+
 /* Canonical mode: one training step (forward, backward, update) on rows [row0, row0+batch) of
  * the resident table.  host_metrics may be NULL (then the call does not synchronise). */
 int ghip_net_train_step(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);

@@ -10,10 +10,12 @@
 //   host_api_check numberinput <file.csv> <minmax|zscore> <out.bin>      (no GPU needed)
 //   host_api_check traincsv <file.csv> <nninfo table> <stop_epoch> <stop_accuracy> <seed> <out.bin> [case.bin with the initial weights]
 //   host_api_check checkpoint <case.bin> <mode> <E1> <E2> <file.ckpt> <out.bin>
+//   host_api_check meta <case.bin> <mode> <k subnets> <epochs> <out.bin>
 //   host_api_check train  <case.bin> <out.bin> <stop_epoch> <stop_accuracy> <mode>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #include <vector>
 
@@ -298,10 +300,65 @@ static int do_checkpoint(const char* in, int mode, int e1, int e2, const char* c
     return 0;
 }
 
+// k subnets with the case's weights in one MetaNetwork: trained one after the other, then (fresh
+// copies) at the same time.  out: k, seconds in order, seconds concurrent, cross-validation accuracy,
+// then per subnet and per run the final loss, and every layer's weights of both runs of subnet 0 and k-1.
+static int do_meta(const char* in, int mode, int k, int epochs, const char* out)
+{
+    Case c;
+    int rc = read_case(in, c);
+    if (rc) return rc;
+    glades::init();
+    DenseInput di(c.X.data(), c.Y.data(), c.N, c.sizes[0], c.sizes[c.nl]);
+    double secs[2];
+    std::vector<float> losses;
+    std::vector<std::vector<float> > keep;
+    float cv = 0.0f;
+    for (int run = 0; run < 2; ++run) {
+        MetaNetwork meta("meta");
+        meta.setConcurrent(run == 1);
+        for (int i = 0; i < k; ++i) {
+            meta.addSubnet(case_info(c));
+            NNetwork* n = meta.getSubnet(i);
+            seed_net(*n, c, mode);
+            n->setVerbose(false);
+            n->terminator.setEpoch(epochs);
+        }
+        struct timespec t0, t1;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        if (run == 0) { if (!glades::train(&meta, &di)) return 3; }
+        else cv = meta.crossValidate(&di);
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        secs[run] = (t1.tv_sec - t0.tv_sec) + 1e-9 * (t1.tv_nsec - t0.tv_nsec);
+        for (int i = 0; i < k; ++i) {
+            NNetwork* n = meta.getSubnet(i);
+            if (!n->getLastError().empty()) { fprintf(stderr, "subnet %d: %s\n", i, n->getLastError().c_str()); return 4; }
+            losses.push_back(n->getLoss());
+        }
+        for (int which = 0; which < 2; ++which) {
+            NNetwork* n = meta.getSubnet(which == 0 ? 0 : k - 1);
+            std::vector<float> all;
+            for (int l = 0; l < c.nl; ++l) { std::vector<float> w = n->getWeights(l); all.insert(all.end(), w.begin(), w.end()); }
+            keep.push_back(all);
+        }
+        for (int i = 0; i < k; ++i) delete meta.getSubnet(i);
+    }
+    printf("meta: %d subnets x %d epochs x %d rows: in order %.3f s, concurrent (train + test pass) %.3f s\n", k, epochs, c.N, secs[0], secs[1]);
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    float head[4] = {(float)k, (float)secs[0], (float)secs[1], cv};
+    fwrite(head, 4, 4, fo);
+    fwrite(losses.data(), 4, losses.size(), fo);
+    for (size_t i = 0; i < keep.size(); ++i) fwrite(keep[i].data(), 4, keep[i].size(), fo);
+    fclose(fo);
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
+    if (argc >= 7 && !strcmp(argv[1], "meta")) return do_meta(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 8 && !strcmp(argv[1], "checkpoint")) return do_checkpoint(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7]);
     if (argc >= 2 && !strcmp(argv[1], "ohe")) return do_ohe();
     if (argc >= 5 && !strcmp(argv[1], "numberinput")) return do_numberinput(argv[2], argv[3], argv[4]);

@@ -151,3 +151,48 @@ def test_error_paths():
     with pytest.raises(pg.GladesHipError):   # wrong mode
         net.train_step(0, 1)
     net.close()
+
+
+def test_many_networks_in_one_launch_equal_their_solo_runs():
+    """ghip_net_run_epochs_exact_multi: one workgroup per network; every network ends exactly where
+    it ends when it runs alone (metrics of every epoch, weights, biases, delta windows)."""
+    import pyglades as pg
+    c = load_case("window_4_5_3_1")
+    rng = np.random.default_rng(21)
+    K, E = 7, 5
+    solo, group = [], []
+    for k in range(K):
+        Ws = [(c["W0"][l] + rng.normal(0, 0.05, c["W0"][l].shape)).astype(np.float32) for l in range(c["nl"])]
+        for dst in (solo, group):
+            n = gpu_net(c)
+            for l in range(c["nl"]):
+                n.set_params(l, Ws[l], c["bias0"][l])
+            dst.append(n)
+    want = [n.run_epochs_exact(E)[0] for n in solo]
+    got = pg.run_epochs_exact_multi(group, E)
+    assert got == want
+    assert len({tuple(m) for ms in got for m in ms}) > K      # the networks really differ
+    for a, b in zip(solo, group):
+        for l in range(c["nl"]):
+            Wa, ba = a.get_params(l); Wb, bb = b.get_params(l)
+            assert np.array_equal(Wa, Wb) and np.array_equal(ba, bb)
+            sa, sb = a.get_state(l), b.get_state(l)
+            assert np.array_equal(sa[0], sb[0]) and np.array_equal(sa[1], sb[1])
+    # every network stops on its own: in a test pass (weights fixed) those at or above the target
+    # leave after one epoch, the others use all three
+    fresh = []
+    for k in range(K):
+        n = gpu_net(c)
+        for l in range(c["nl"]):
+            W, b = solo[k].get_params(l)
+            n.set_params(l, W, b)
+        fresh.append(n)
+    alone = [n.run_epochs_exact(1, train=False)[0][0][1] for n in fresh]
+    target = float(np.sort(alone)[K // 2])
+    test_pass = pg.run_epochs_exact_multi(fresh, 3, train=False, stop_accuracy=target)
+    assert [len(ms) for ms in test_pass] == [1 if a >= target else 3 for a in alone]
+    assert 1 in [len(ms) for ms in test_pass] and 3 in [len(ms) for ms in test_pass]
+    with pytest.raises(pg.GladesHipError):
+        pg.run_epochs_exact_multi([group[0], group[0]], 1)
+    for n in solo + group + fresh:
+        n.close()

@@ -336,3 +336,33 @@ def test_checkpoint_resume_is_bit_identical(name, mode):
     assert body.size % 2 == 0
     assert bits_equal(body[:body.size // 2], body[body.size // 2:])
     assert np.all(np.isfinite(body))
+
+
+@needs_bin
+@pytest.mark.gpu
+def test_meta_network_subnets_run_concurrently_with_equal_results():
+    """k subnets of one MetaNetwork, one host thread and one stream each: every subnet ends where
+    the same network trained alone ends, bit for bit; the run prints both wall-clock times."""
+    c = load_case("cfg1_shape_4_16_3")
+    k, epochs = 8, 40
+    with tempfile.TemporaryDirectory() as td:
+        cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
+        write_case(cin, c)
+        log = subprocess.check_output([BIN, "meta", cin, "0", str(k), str(epochs), cout], text=True)
+        raw = np.fromfile(cout, np.float32)
+    print(log.strip().splitlines()[-1], flush=True)
+    assert int(raw[0]) == k
+    losses = raw[4:4 + 2 * k]
+    # run 0 ends on the last training epoch, run 1 (crossValidate) on the test pass after it
+    assert bits_equal(losses[:k], np.full(k, losses[0], np.float32)) and bits_equal(losses[k:], np.full(k, losses[k], np.float32))
+    nw = sum(c["sizes"][l] * c["sizes"][l + 1] for l in range(c["nl"]))
+    W = raw[4 + 2 * k:].reshape(4, nw)
+    assert all(bits_equal(W[0], W[i]) for i in range(1, 4))
+    o = po.ExactNet(c["spec"])
+    for l in range(c["nl"]):
+        o.set_weights(l, c["W0"][l]); o.set_bias(l, float(c["bias0"][l]))
+    for _ in range(epochs):
+        m, _ = o.epoch(c["X"], c["Y"], train=True, want_preds=False)
+    np.testing.assert_allclose(losses[0], m.loss, rtol=1e-4)
+    m, _ = o.epoch(c["X"], c["Y"], train=False, want_preds=False)
+    np.testing.assert_allclose(raw[3], m.accuracy, rtol=1e-4)             # cross-validation accuracy = mean test accuracy
