@@ -190,28 +190,41 @@ def run_exact(w, args):
         acts, params, cost = [pg.SIGMOID, pg.SIGMOID], [0, 0], pg.CLASSIFICATION
     nl = len(sizes) - 1
     spec = pg.make_spec(sizes, acts, lr=0.01, mom=0.9, act_params=params, batch=mb, cost=cost, mode=pg.MODE_EXACT)
-    net = pg.Net(spec)
-    for l in range(nl):
-        lim = np.sqrt(6.0 / (sizes[l] + sizes[l + 1]))
-        net.set_params(l, rng.uniform(-lim, lim, (sizes[l + 1], sizes[l])).astype(np.float32), 0.0)
-    net.set_dataset(X, Y)
+    K = max(1, args.subnets)   # networks trained side by side (the subnets of a MetaNetwork), one workgroup each
+    nets = []
+    for _ in range(K):
+        net = pg.Net(spec)
+        for l in range(nl):
+            lim = np.sqrt(6.0 / (sizes[l] + sizes[l + 1]))
+            net.set_params(l, rng.uniform(-lim, lim, (sizes[l + 1], sizes[l])).astype(np.float32), 0.0)
+        net.set_dataset(X, Y)
+        nets.append(net)
+    net = nets[0]
+
+    def epochs(n):
+        if K == 1:
+            return net.run_epochs_exact(n)[0]
+        return pg.run_epochs_exact_multi(nets, n)[0]
+
     for _ in range(args.warmup):
-        net.run_epochs_exact(1)
+        epochs(1)
     net.sync()
     t0 = time.perf_counter()
-    ms, _ = net.run_epochs_exact(args.steps)   # one launch, `steps` epochs
+    ms = epochs(args.steps)   # one launch, `steps` epochs
     net.sync()
     el = time.perf_counter() - t0
-    prof = kernel_profile(net, lambda s: net.run_epochs_exact(1), 3)
-    net.close()
-    value = args.steps * N / el
-    k = prof["exact_epochs"]
+    kname = "exact_epochs" if K == 1 else "exact_epochs_multi"
+    prof = kernel_profile(net, lambda s: epochs(1), 3)
+    for n in nets:
+        n.close()
+    value = K * args.steps * N / el
+    k = prof[kname]
     bytes_per_sample = 4 * (sizes[0] + sizes[-1])
-    ach = bytes_per_sample * N / (k[0] / k[1] * 1e-3) / 1e9
-    roof = dict(bound="hbm", kernel="exact_epochs", achieved=round(ach, 4), peak=HBM_PEAK, unit="GB/s",
+    ach = K * bytes_per_sample * N / (k[0] / k[1] * 1e-3) / 1e9
+    roof = dict(bound="hbm", kernel=kname, achieved=round(ach, 4), peak=HBM_PEAK, unit="GB/s",
                 frac=round(ach / HBM_PEAK, 8), traffic=None, avg_launch_ms=round(k[0] / k[1], 4),
-                note="latency-bound: one persistent workgroup, rows strictly sequential")
-    extra = dict(final_loss=ms[-1][0], final_accuracy=ms[-1][1], flop_per_sample=train_flops_per_sample(sizes))
+                note="latency-bound: one persistent workgroup per network, rows strictly sequential")
+    extra = dict(final_loss=ms[-1][0], final_accuracy=ms[-1][1], flop_per_sample=train_flops_per_sample(sizes), subnets=K)
     return value, el, roof, extra
 
 
@@ -271,6 +284,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS) + ["copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--subnets", type=int, default=1,
+                    help="exact workloads: this many networks (MetaNetwork subnets) side by side in one launch; value is their sum")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -310,7 +325,8 @@ def main():
         "value": round(value, 1), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(el / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w['desc']}", "rows_per_step": unit_rows,
+        "config": {"workload": f"{args.workload}: {w['desc']}" + (f", {args.subnets} subnets side by side" if w["kind"] == "exact" and args.subnets > 1 else ""),
+                   "rows_per_step": unit_rows,
                    "flop_per_sample": train_flops_per_sample(w["sizes"]) if w["kind"] != "infer" else infer_flops_per_sample(w["sizes"])},
         "roofline": roof,
     }
