@@ -138,11 +138,12 @@ template <int Q>
 __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
 {
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int b = blockIdx.x * 4 + w;
     double loss = 0.0, accs = 0.0, corr = 0.0;
     const bool softmax = a.act == GHIP_SOFTMAX;
     const bool sig_bce = (a.act == GHIP_SIGMOID || a.act == GHIP_SIGMOIDP) && a.cost == GHIP_CLASSIFICATION;
-    if (b < a.B) {
+    // a bounded grid walks the rows: the three sums reach the accumulators once per workgroup (the
+    // same-address double atomics of one workgroup per 4 rows took longer than the rows themselves)
+    for (int b = blockIdx.x * 4 + w; b < a.B; b += gridDim.x * 4) {
         float* p = a.P + (long long)b * a.ldp;
         const float* y = a.Y ? a.Y + (long long)b * a.ldy : nullptr;
         float4 pr[Q], yr[Q];
@@ -215,9 +216,9 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
             ov = __shfl_xor(by, o, 64); oi = __shfl_xor(iy, o, 64);
             if (ov > by || (ov == by && oi < iy)) { by = ov; iy = oi; }
         }
-        loss = (double)wave_sum(l);
-        accs = (double)wave_sum(ac);
-        if (ip == iy) corr = 1.0;
+        loss += (double)wave_sum(l);
+        accs += (double)wave_sum(ac);
+        if (ip == iy) corr += 1.0;
         // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
         if (a.cm && lane == 0 && ip != 0x7fffffff && iy != 0x7fffffff) atomicAdd(&a.cm[(long long)iy * a.n + ip], 1);
     }
@@ -531,7 +532,8 @@ hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
     const bool vec_ok = (a.n % 4) == 0 && a.n <= 2048 && (a.ldp % 4) == 0 && (!a.Y || (a.ldy % 4) == 0) &&
                         ((uintptr_t)a.P % 16) == 0 && ((uintptr_t)a.Y % 16) == 0 && ((uintptr_t)a.D % 16) == 0 && ((uintptr_t)a.Dbf % 8) == 0;
     if (vec_ok) {
-        const dim3 grid4((a.B + 3) / 4);
+        const int groups = (a.B + 3) / 4;
+        const dim3 grid4(groups < 1024 ? groups : 1024);
         if (a.n <= 256) hipLaunchKernelGGL(output_delta_vec4_kernel<1>, grid4, dim3(256), 0, s, a);
         else if (a.n <= 512) hipLaunchKernelGGL(output_delta_vec4_kernel<2>, grid4, dim3(256), 0, s, a);
         else if (a.n <= 1024) hipLaunchKernelGGL(output_delta_vec4_kernel<4>, grid4, dim3(256), 0, s, a);

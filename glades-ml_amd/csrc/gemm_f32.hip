@@ -103,26 +103,27 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
     const int nk = (g.K + BK - 1) / BK;
-    Frag fa = fetch<FAST>(g.A, g.lda, AKM, bm, 0, g.M, g.K, t);
-    Frag fb = fetch<FAST>(g.B, g.ldb, BKM, bn, 0, g.N, g.K, t);
-    stage(As, fa, AKM, t);
-    stage(Bs, fb, BKM, t);
-    if (nk > 1) {
-        fa = fetch<FAST>(g.A, g.lda, AKM, bm, BK, g.M, g.K, t);
-        fb = fetch<FAST>(g.B, g.ldb, BKM, bn, BK, g.N, g.K, t);
-        stage(As + SLAB, fa, AKM, t);
-        stage(Bs + SLAB, fb, BKM, t);
-    }
+    // Slabs 0 and 1 go straight to LDS; from then on slab kt+2 is staged at the end of iteration kt from
+    // registers filled one iteration earlier, so a global load has a whole iteration to arrive
+    // (two register sets, alternating: the loop body is written out for even and odd kt).
+    Frag fa0 = fetch<FAST>(g.A, g.lda, AKM, bm, 0, g.M, g.K, t);
+    Frag fb0 = fetch<FAST>(g.B, g.ldb, BKM, bn, 0, g.N, g.K, t);
+    Frag fa1 = fetch<FAST>(g.A, g.lda, AKM, bm, BK, g.M, g.K, t);      // past K: zeros (FAST) / guarded loads
+    Frag fb1 = fetch<FAST>(g.B, g.ldb, BKM, bn, BK, g.N, g.K, t);
+    stage(As, fa0, AKM, t);
+    stage(Bs, fb0, BKM, t);
+    stage(As + SLAB, fa1, AKM, t);
+    stage(Bs + SLAB, fb1, BKM, t);
+    fa0 = fetch<FAST>(g.A, g.lda, AKM, bm, 2 * BK, g.M, g.K, t);       // slab 2, staged at the end of iteration 0
+    fb0 = fetch<FAST>(g.B, g.ldb, BKM, bn, 2 * BK, g.N, g.K, t);
     __syncthreads();
 
     const int lr = lane & 31, lk = lane >> 5;
-    for (int kt = 0; kt < nk; ++kt) {
+    auto iteration = [&](int kt, Frag& sa_, Frag& sb_, Frag& na_, Frag& nb_) {
         const int cur = kt % NST, nxt = (kt + 2) % NST;
-        const bool more = kt + 2 < nk;
-        if (more) {
-            fa = fetch<FAST>(g.A, g.lda, AKM, bm, (kt + 2) * BK, g.M, g.K, t);
-            fb = fetch<FAST>(g.B, g.ldb, BKM, bn, (kt + 2) * BK, g.N, g.K, t);
-        }
+        // slab kt+3 sets out now, into the register set that was staged one iteration ago
+        na_ = fetch<FAST>(g.A, g.lda, AKM, bm, (kt + 3) * BK, g.M, g.K, t);
+        nb_ = fetch<FAST>(g.B, g.ldb, BKM, bn, (kt + 3) * BK, g.N, g.K, t);
         // lane half lk supplies k = kh + 16*lk + i to MFMA i (any pairing works as long as A and B agree):
         // 16 consecutive k per lane, which a [row][k] operand delivers as four 16-byte reads
         const float* pa = As + cur * SLAB + (kh + 16 * lk) * ska + (wm + lr) * sra;
@@ -133,11 +134,14 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
         __builtin_amdgcn_sched_barrier(0);  // keep the reads together: sunk next to their MFMA each would be waited for alone
 #pragma unroll
         for (int i = 0; i < BK / 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av[i], bv[i], acc, 0, 0, 0);
-        if (more) {  // slab kt-1's buffer: every wavefront left it before the barrier that ended kt-1
-            stage(As + nxt * SLAB, fa, AKM, t);
-            stage(Bs + nxt * SLAB, fb, BKM, t);
-        }
+        // slab kt+2 (requested during iteration kt-1) into the buffer slab kt-1 has left
+        stage(As + nxt * SLAB, sa_, AKM, t);
+        stage(Bs + nxt * SLAB, sb_, BKM, t);
         __syncthreads();
+    };
+    for (int kt = 0; kt < nk; kt += 2) {
+        iteration(kt, fa0, fb0, fa1, fb1);
+        if (kt + 1 < nk) iteration(kt + 1, fa1, fb1, fa0, fb0);
     }
 
     // the upper K halves go to LDS ([wavefront][register][lane]) and are added by the lower ones
