@@ -255,6 +255,9 @@ struct go_exact {
     float  bias[GO_MAX_LAYERS];  /* scalar bias of layer l, added to layer l+1 (l >= 1) */
     float* a[GO_MAX_LAYERS + 1]; /* node values */
     float* e[GO_MAX_LAYERS + 1]; /* node error accumulators */
+    int32_t* wcnt[GO_MAX_LAYERS]; /* number of pending deltas of the edge (Edge::prevDelta.size()) */
+    const uint8_t* masks;        /* dropout flags of the coming epoch, N rows x mask_len, or NULL */
+    int mask_len, moff[GO_MAX_LAYERS + 1];
 };
 
 go_exact* go_exact_create(const go_spec* spec)
@@ -266,6 +269,9 @@ go_exact* go_exact_create(const go_spec* spec)
         n->W[l] = (float*)calloc(cnt, sizeof(float));
         n->wsum[l] = (float*)calloc(cnt, sizeof(float));
         n->wlast[l] = (float*)calloc(cnt, sizeof(float));
+        n->wcnt[l] = (int32_t*)calloc(cnt, sizeof(int32_t));
+        n->moff[l] = n->mask_len;
+        n->mask_len += spec->sizes[l];
     }
     for (int l = 0; l <= spec->n_layers; ++l) {
         n->a[l] = (float*)calloc(spec->sizes[l], sizeof(float));
@@ -277,7 +283,7 @@ go_exact* go_exact_create(const go_spec* spec)
 void go_exact_destroy(go_exact* n)
 {
     if (!n) return;
-    for (int l = 0; l < n->s.n_layers; ++l) { free(n->W[l]); free(n->wsum[l]); free(n->wlast[l]); }
+    for (int l = 0; l < n->s.n_layers; ++l) { free(n->W[l]); free(n->wsum[l]); free(n->wlast[l]); free(n->wcnt[l]); }
     for (int l = 0; l <= n->s.n_layers; ++l) { free(n->a[l]); free(n->e[l]); }
     free(n);
 }
@@ -295,9 +301,16 @@ void go_exact_get_window(const go_exact* n, int l, float* sum, float* last)
     memcpy(last, n->wlast[l], cnt * sizeof(float));
 }
 
-/* network.cpp:457-575 for one row (no dropout). */
+/* Layer::possiblePath (layer.cpp:136-150): nodes of the output layer are never dropped. */
+static int valid_node(const go_exact* n, const uint8_t* m, int layer, int i)
+{
+    if (!m || layer >= n->s.n_layers) return 1;
+    return !m[n->moff[layer] + i];
+}
+
+/* network.cpp:457-575 for one row; m = the row's dropout flags or NULL. */
 static void exact_forward(go_exact* n, const float* x, const float* y, int64_t N,
-                          float* tot_err, float* tot_acc)
+                          float* tot_err, float* tot_acc, const uint8_t* m)
 {
     const go_spec* s = &n->s;
     const int H1 = s->n_layers;
@@ -308,9 +321,13 @@ static void exact_forward(go_exact* n, const float* x, const float* y, int64_t N
         for (int o = 0; o < no; ++o) {
             float z = 0.0f; /* node.cpp:82-93: sum of edge activations, i ascending */
             for (int i = 0; i < ni; ++i) {
+                /* network.cpp:480-488: a dropped pair sets no edge activation */
+                if (!(valid_node(n, m, l, i) && valid_node(n, m, l + 1, o))) continue;
                 float ea = W[(size_t)o * ni + i] * n->a[l][i]; /* network.cpp:485-487 */
                 z += ea;
             }
+            /* network.cpp:491-516 runs at the last valid input node for EVERY output node: a dropped
+               output node still becomes squash(bias) */
             if (l != 0) z += n->bias[l]; /* network.cpp:501-502 */
             n->a[l + 1][o] = go_squash(z, s->act[l], s->act_param[l]);
             if (l == H1 - 1) { /* network.cpp:519-559 */
@@ -326,8 +343,8 @@ static void exact_forward(go_exact* n, const float* x, const float* y, int64_t N
     }
 }
 
-/* network.cpp:577-668 for one row `r` (no dropout); node.cpp:278-307 inlined. */
-static void exact_backward(go_exact* n, const float* y, int64_t r)
+/* network.cpp:577-668 for one row `r`; node.cpp:278-307 inlined; m = the row's dropout flags or NULL. */
+static void exact_backward(go_exact* n, const float* y, int64_t r, const uint8_t* m)
 {
     const go_spec* s = &n->s;
     const int H1 = s->n_layers;
@@ -338,6 +355,7 @@ static void exact_backward(go_exact* n, const float* y, int64_t r)
         float* W = n->W[l];
         float* ws = n->wsum[l];
         float* wl = n->wlast[l];
+        int32_t* wc = n->wcnt[l];
         const float lr = s->lr[l], mom = s->mom[l], wd1 = s->wd1[l], wd2 = s->wd2[l];
         for (int i = 0; i < ni; ++i) {
             const float ain = n->a[l][i];
@@ -349,25 +367,34 @@ static void exact_backward(go_exact* n, const float* y, int64_t r)
                 } else {
                     der = go_act_der(n->a[L][o], s->act[l], 0.01f); /* network.cpp:616-618 */
                 }
+                /* network.cpp:621-625 */
+                const int dropout = !(valid_node(n, m, l, i) && valid_node(n, m, L, o));
                 float d = n->e[L][o];
-                d *= der;
-                if (i == ni - 1) n->e[L][o] = 0;
-                float base = lr * d;
                 size_t k = (size_t)o * ni + i;
-                /* node.cpp:285-288 */
-                float dW = ((base * ain) + (mom * wl[k]) + (wd1 * lr * fabsf(ain)) +
-                            (wd2 * lr * ain));
-                ws[k] += dW; /* same order as node.cpp:299-301 summing the window from 0 */
-                wl[k] = dW;
-                if ((r % mb) == 0) { /* network.cpp:647-651 */
-                    float dsum = ws[k];
-                    dsum /= mb;
-                    W[k] = W[k] - dsum;
-                    ws[k] = 0.0f;
-                    wl[k] = 0.0f;
+                if (!dropout) {
+                    d *= der;
+                    if (i == ni - 1) n->e[L][o] = 0;
+                    float base = lr * d;
+                    /* node.cpp:285-288 */
+                    float dW = ((base * ain) + (mom * wl[k]) + (wd1 * lr * fabsf(ain)) +
+                                (wd2 * lr * ain));
+                    /* node.cpp:299-301 sums the window's first minibatchSize entries from 0; an edge
+                       that sat out an applying row can hold more than that */
+                    if (wc[k] < mb) ws[k] += dW;
+                    wc[k] += 1;
+                    wl[k] = dW;
+                    if ((r % mb) == 0) { /* network.cpp:647-651 */
+                        float dsum = ws[k];
+                        dsum /= mb;
+                        W[k] = W[k] - dsum;
+                        ws[k] = 0.0f;
+                        wl[k] = 0.0f;
+                        wc[k] = 0;
+                    }
+                    if (l != 0) n->bias[l] = n->bias[l] - base; /* network.cpp:654-656 */
                 }
-                if (l != 0) n->bias[l] = n->bias[l] - base; /* network.cpp:654-656 */
-                /* network.cpp:660-662 + node.cpp:173-176 */
+                /* network.cpp:660-662 + node.cpp:173-176: runs for dropped pairs too, with the
+                   accumulator of the output node taken as it stands (no derivative factor) */
                 float cin = n->e[l][i] + (d * W[k]);
                 n->e[l][i] += cin;
             }
@@ -387,14 +414,64 @@ void go_exact_epoch(go_exact* n, const float* X, const float* Y, int64_t N, int 
     for (int64_t r = 0; r < N; ++r) {
         const float* x = X + r * nf;
         const float* y = Y + r * no;
-        exact_forward(n, x, y, N, &tot_err, &tot_acc);
+        const uint8_t* m = n->masks ? n->masks + (size_t)r * n->mask_len : NULL;
+        exact_forward(n, x, y, N, &tot_err, &tot_acc, m);
         const float* p = n->a[s->n_layers];
         if (preds) memcpy(preds + r * no, p, sizeof(float) * no);
         if (go_argmax_ref(p, no) == go_argmax_ref(y, no)) ++correct;
-        if (train) exact_backward(n, y, r);
+        if (train) exact_backward(n, y, r, m);
     }
     tot_acc /= ((float)(unsigned)N) * ((float)(unsigned)no); /* network.cpp:194-195 */
     if (m) { m->loss = tot_err; m->accuracy = tot_acc; m->correct = correct; }
+}
+
+/* ---- dropout (layer.cpp:102-134, LayerBuilder.cpp:497-523) ---- */
+
+int go_exact_mask_len(const go_exact* n) { return n->mask_len; }
+void go_exact_set_dropout(go_exact* n, const uint8_t* masks) { n->masks = masks; }
+void go_exact_get_pending(const go_exact* n, int l, int32_t* cnt)
+{ memcpy(cnt, n->wcnt[l], sizeof(int32_t) * n->s.sizes[l] * n->s.sizes[l + 1]); }
+void go_exact_get_errder(const go_exact* n, int layer, float* e)
+{ memcpy(e, n->e[layer], sizeof(float) * n->s.sizes[layer]); }
+
+/* Layer::generateDropout: one dart rand()%100+1 per node, node dropped when dart <= int(p*100);
+   the whole layer is drawn again while every node came out dropped; a rate below 0 or from 100
+   up draws nothing and leaves the flags as they are. */
+static void draw_layer(float p, int n, uint8_t* flag)
+{
+    int rate = p * 100.0f;
+    if (rate < 0) return;
+    if (rate >= 100) return;
+    int all_dropped;
+    do {
+        all_dropped = 1;
+        for (int i = 0; i < n; ++i) {
+            int dropped = 0;
+            int dart = (rand() % 100) + 1;
+            if (dart <= rate) dropped = 1;
+            else all_dropped = 0;
+            flag[i] = (uint8_t)dropped;
+        }
+    } while (all_dropped);
+}
+
+/* One epoch's flags in the order SGDHelper draws them (network.cpp:407-411): for every row, the
+   row's input layer, then each hidden layer.  p[l] is the probability of node layer l (0 = input);
+   masks is N x sum(sizes[0..n_layers-1]) bytes, 1 = dropped, and must hold the previous row's flags
+   of the hidden layers and the previous epoch's flags of the row's input layer on entry for layers
+   whose rate draws nothing (all zero for a fresh network). */
+void go_dropout_draw(const go_spec* s, const float* p, int64_t N, uint8_t* masks)
+{
+    int len = 0;
+    for (int l = 0; l < s->n_layers; ++l) len += s->sizes[l];
+    for (int64_t r = 0; r < N; ++r) {
+        uint8_t* m = masks + (size_t)r * len;
+        int off = 0;
+        for (int l = 0; l < s->n_layers; ++l) {
+            draw_layer(p[l], s->sizes[l], m + off);
+            off += s->sizes[l];
+        }
+    }
 }
 
 /* ------------------------------------------------------------------ canonical mode */

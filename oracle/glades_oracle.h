@@ -36,6 +36,11 @@
  *       be compiled here (it needs the un-vendored shmea library); its order is
  *       restated from the source text in both the harness and this file:
  *       for that ordering alone -- parity unpinned by execution.
+ *   go_dropout_draw / the dropout branches of go_exact_*  (layer.cpp:102-183, network.cpp:480-488,
+ *       621-662)  pinned: the flags, the rand() stream position afterwards and the trained state
+ *       are bit-compared with the reference's compiled Layer::generateDropout / possiblePath /
+ *       lastValidPath and Node/Edge objects run through the same harness (fixtures
+ *       tests/golden/dropout_*.npz); the loop nest is restated as above.
  *   go_canon_*  no counterpart in the reference (the reference has no batched
  *       training, softmax or per-channel bias): pinned against torch autograd +
  *       torch.optim.SGD and finite differences; forward pinned against go_exact
@@ -114,6 +119,18 @@ void  go_exact_get_window(const go_exact* n, int layer, float* sum, float* last)
    preds (N*n_out) may be NULL. */
 void  go_exact_epoch(go_exact* n, const float* X, const float* Y, int64_t N, int train,
                      go_metrics* m, float* preds);
+
+/* dropout: flags for one epoch, N rows x go_exact_mask_len() bytes (1 = dropped), the node layers
+   0..n_layers-1 of a row side by side; NULL = nothing dropped.  The pointer is kept, not copied. */
+int   go_exact_mask_len(const go_exact* n);
+void  go_exact_set_dropout(go_exact* n, const uint8_t* masks);
+/* draws one epoch's flags with libc rand() in the reference's order (layer.cpp:102-134,
+   LayerBuilder.cpp:497-523, network.cpp:407-411); p[l] = probability of node layer l */
+void  go_dropout_draw(const go_spec* s, const float* p, int64_t N, uint8_t* masks);
+/* what dropout leaves behind between rows: pending-delta counts per edge and the error
+   accumulators of a hidden layer's nodes */
+void  go_exact_get_pending(const go_exact* n, int layer, int32_t* cnt);
+void  go_exact_get_errder(const go_exact* n, int layer, float* e);
 
 /* ---- canonical mode ---- */
 typedef struct go_canon go_canon;

@@ -77,6 +77,13 @@ def lib():
             "go_exact_get_bias": (C.c_float, [vp, C.c_int]),
             "go_exact_get_window": (None, [vp, C.c_int, f32p, f32p]),
             "go_exact_epoch": (None, [vp, f32p, f32p, C.c_int64, C.c_int, C.POINTER(Metrics), vp]),
+            "go_exact_mask_len": (C.c_int, [vp]),
+            "go_exact_set_dropout": (None, [vp, vp]),
+            "go_dropout_draw": (None, [C.POINTER(Spec), f32p, C.c_int64, u8p]),
+            "go_exact_get_pending": (None, [vp, C.c_int, i32p]),
+            "go_exact_get_errder": (None, [vp, C.c_int, f32p]),
+            "srand": (None, [C.c_uint]),
+            "rand": (C.c_int, []),
             "go_canon_create": (vp, [C.POINTER(Spec)]),
             "go_canon_destroy": (None, [vp]),
             "go_canon_set_params": (None, [vp, C.c_int, f32p, vp]),
@@ -165,11 +172,26 @@ class ExactNet:
         lib().go_exact_get_window(self.h, l, s, t)
         return s, t
 
-    def epoch(self, X, Y, train=True, want_preds=True):
+    def get_pending(self, l):
+        c = np.empty((self.sizes[l + 1], self.sizes[l]), np.int32)
+        lib().go_exact_get_pending(self.h, l, c)
+        return c
+
+    def get_errder(self, layer):
+        e = np.empty(self.sizes[layer], np.float32)
+        lib().go_exact_get_errder(self.h, layer, e)
+        return e
+
+    def epoch(self, X, Y, train=True, want_preds=True, masks=None):
+        """masks: N x sum(sizes[:-1]) uint8 dropout flags of this epoch (1 = dropped) or None."""
         X = np.ascontiguousarray(X, np.float32)
         Y = np.ascontiguousarray(Y, np.float32)
         N = X.shape[0]
         assert X.shape == (N, self.sizes[0]) and Y.shape == (N, self.sizes[-1])
+        if masks is not None:
+            masks = np.ascontiguousarray(masks, np.uint8)
+            assert masks.shape == (N, sum(self.sizes[:-1]))
+        lib().go_exact_set_dropout(self.h, _vp(masks))
         preds = np.empty((N, self.sizes[-1]), np.float32) if want_preds else None
         m = Metrics()
         lib().go_exact_epoch(self.h, X, Y, N, 1 if train else 0, C.byref(m), _vp(preds))
@@ -270,9 +292,31 @@ def have_ref():
     return os.path.exists(REF_HARNESS)
 
 
-def ref_train(spec, weights, biases, X, Y, epochs, tmpdir):
+def libc_srand(seed):
+    """Seeds the libc rand() stream that go_dropout_draw and go_ref_xavier_layer consume."""
+    lib().srand(int(seed))
+
+
+def libc_rand():
+    return lib().rand()
+
+
+def dropout_draw(spec, p, N):
+    """One epoch's dropout flags drawn from libc rand() in the reference's order: N x sum(sizes[:-1])."""
+    nl = spec.n_layers
+    p = np.ascontiguousarray(p, np.float32)
+    assert p.shape == (nl,)
+    m = np.zeros((N, sum(spec.sizes[i] for i in range(nl))), np.uint8)
+    lib().go_dropout_draw(C.byref(spec), p, N, m)
+    return m
+
+
+def ref_train(spec, weights, biases, X, Y, epochs, tmpdir, dropout=None):
     """Run the harness built from the reference's compiled objects.  Returns a dict with
-    per-epoch (loss, accuracy), final weights, biases, last-epoch predictions and windows."""
+    per-epoch (loss, accuracy), final weights, biases, last-epoch predictions and windows.
+    dropout = (seed, [p per non-output layer]) also returns the flags the reference drew
+    ("masks": epochs x N x sum(sizes[:-1])), the window lengths ("wcnt"), the hidden nodes'
+    error accumulators ("errder") and the next rand() % 65536 ("rand_after")."""
     nl = spec.n_layers
     sizes = [spec.sizes[i] for i in range(nl + 1)]
     X = np.ascontiguousarray(X, np.float32)
@@ -291,6 +335,9 @@ def ref_train(spec, weights, biases, X, Y, epochs, tmpdir):
         f.write(np.array([biases[l] for l in range(nl)], np.float32).tobytes())
         f.write(X.tobytes())
         f.write(Y.tobytes())
+        if dropout is not None:
+            f.write(np.array([dropout[0]], np.int32).tobytes())
+            f.write(np.asarray(dropout[1], np.float32).tobytes())
     with open(os.devnull, "w") as dn:
         subprocess.check_call([REF_HARNESS, "train", cin, cout], stdout=dn)
     raw = np.fromfile(cout, np.float32)
@@ -313,6 +360,21 @@ def ref_train(spec, weights, biases, X, Y, epochs, tmpdir):
         out["wsum"].append(w[..., 0].copy())
         out["wlast"].append(w[..., 1].copy())
         pos += 2 * cnt
+    if dropout is not None:
+        ml = sum(sizes[:-1])
+        out["masks"] = raw[pos : pos + epochs * N * ml].reshape(epochs, N, ml).astype(np.uint8)
+        pos += epochs * N * ml
+        out["wcnt"] = []
+        for l in range(nl):
+            cnt = sizes[l] * sizes[l + 1]
+            out["wcnt"].append(raw[pos : pos + cnt].reshape(sizes[l + 1], sizes[l]).astype(np.int32))
+            pos += cnt
+        out["errder"] = []
+        for l in range(1, nl):
+            out["errder"].append(raw[pos : pos + sizes[l]].copy())
+            pos += sizes[l]
+        out["rand_after"] = int(raw[pos])
+        pos += 1
     assert pos == raw.size
     return out
 

@@ -164,7 +164,14 @@ static int do_train(const char* in, const char* out)
     std::vector<float> X((size_t)c.N * nf), Y((size_t)c.N * no);
     if (fread(&X[0], 4, X.size(), f) != X.size()) return 2;
     if (fread(&Y[0], 4, Y.size(), f) != Y.size()) return 2;
+    /* optional trailer: srand() seed and one dropout probability per non-output layer */
+    int32_t seed = 0;
+    std::vector<float> pdrop(H1, 0.0f);
+    const bool with_dropout = fread(&seed, 4, 1, f) == 1;
+    if (with_dropout && fread(&pdrop[0], 4, H1, f) != (size_t)H1) return 2;
     fclose(f);
+    std::vector<float> flags; /* every row's flags of every epoch, in drawing order */
+    if (with_dropout) srand((unsigned)seed);
 
     /* one input Layer per row, as LayerBuilder::buildInputLayers does */
     std::vector<Layer*> inputLayers(c.N);
@@ -189,8 +196,13 @@ static int do_train(const char* in, const char* out)
         float overallTotalError = 0.0f, overallTotalAccuracy = 0.0f;
         for (unsigned int r = 0; r < (unsigned)c.N; ++r) {
             layers[0] = inputLayers[r];
-            /* scrambleDropout with p = 0 (flags all false); consumes rand() only */
-            for (int L = 0; L < H1; ++L) layers[L]->generateDropout(0.0f);
+            /* scrambleDropout (LayerBuilder.cpp:497-523): the row's input layer, then the hidden
+               layers; with p = 0 the flags stay false and only rand() is consumed */
+            for (int L = 0; L < H1; ++L) layers[L]->generateDropout(pdrop[L]);
+            if (with_dropout)
+                for (int L = 0; L < H1; ++L)
+                    for (unsigned i = 0; i < layers[L]->size(); ++i)
+                        flags.push_back(layers[L]->possiblePath(i) ? 0.0f : 1.0f);
             /* ---- ForwardPass ---- */
             for (int cl = 0; cl < H1; ++cl) {
                 Layer* inL = layers[cl];
@@ -280,10 +292,22 @@ static int do_train(const char* in, const char* out)
             for (int i = 0; i < c.sizes[L - 1]; ++i) {
                 std::vector<float> pd = (*layers[L])[o]->getPrevDeltas(i);
                 float s = 0.0f;
-                for (size_t k = 0; k < pd.size(); ++k) s += pd[k];
+                /* the entries applyDeltas would read (node.cpp:299-301: the first minibatchSize) */
+                for (size_t k = 0; k < pd.size() && k < (size_t)minibatchSize; ++k) s += pd[k];
                 wrf(fo, s);
                 wrf(fo, pd.empty() ? 0.0f : pd.back());
             }
+    if (with_dropout) {
+        wr(fo, &flags[0], flags.size() * 4);
+        /* what is left behind between rows: window lengths and the hidden nodes' accumulators */
+        for (int L = 1; L <= H1; ++L)
+            for (int o = 0; o < c.sizes[L]; ++o)
+                for (int i = 0; i < c.sizes[L - 1]; ++i)
+                    wrf(fo, (float)(*layers[L])[o]->getPrevDeltas(i).size());
+        for (int L = 1; L < H1; ++L)
+            for (int o = 0; o < c.sizes[L]; ++o) wrf(fo, (*layers[L])[o]->getErrDer());
+        wrf(fo, (float)(rand() % 65536)); /* where the rand() stream stands afterwards */
+    }
     fclose(fo);
     return 0;
 }

@@ -37,6 +37,23 @@ CASES = [
     ("iris", [4, 5, 3], [po.SIGMOID, po.SIGMOID], po.CLASSIFICATION, 150, 1, 30, 0.01, 0, 0, 0, 0, 12, "iris"),
 ]
 
+# dropout runs: (name, sizes, acts, cost, N, mb, epochs, lr, mom, wd1, wd2, act_params, seed, p per non-output layer)
+# The reference's error accumulators are not cleared for rows whose last input node is dropped
+# (network.cpp:621-631), so wide upper layers overflow within a few rows: the cases keep the upper
+# layers narrow and the numbers finite (if wild), which is the harsher bit-for-bit test.
+DROPOUT_CASES = [
+    ("window_4_5_3_1", [4, 5, 3, 1], [po.TANH] * 3, po.REGRESSION, 11, 3, 4, 0.05, 0.5, 0, 0, 0, 2, [0.2, 0.5, 0.3]),
+    ("decay_3_4_2", [3, 4, 2], [po.SIGMOID] * 2, po.CLASSIFICATION, 10, 4, 3, 0.05, 0.9, 0.01, 0.01, 0, 3, [0.0, 0.5]),
+    ("out_of_range_6_8_2", [6, 8, 2], [po.TANH, po.TANH], po.REGRESSION, 40, 7, 5, 0.02, 0.8, 0, 0, 0, 9, [-0.5, 1.0]),
+    ("heavy_6_8_2", [6, 8, 2], [po.TANH, po.TANH], po.REGRESSION, 40, 7, 5, 0.02, 0.8, 0, 0, 0, 9, [0.5, 0.9]),
+    ("batch1_5_7_6_4", [5, 7, 6, 4], [po.TANH, po.SIGMOID, po.SIGMOID], po.CLASSIFICATION, 23, 1, 3, 0.001, 0.3,
+     0.001, 0.002, 0, 6, [0.1, 0.25, 0.4]),
+    ("deep_64_48_6_2", [64, 48, 6, 2], [po.TANH, po.TANH, po.SIGMOID], po.CLASSIFICATION, 40, 8, 3, 0.001, 0.5, 0, 0, 0,
+     8, [0.3, 0.3, 0.2]),
+    ("wide_1100_12_2", [1100, 12, 2], [po.RELU, po.LINEAR], po.REGRESSION, 12, 4, 2, 0.0005, 0.5, 0, 0, [0, 1.0], 8,
+     [0.5, 0.25]),
+]
+
 IRIS = os.path.join(HERE, "iris_measurements.csv")
 
 
@@ -127,6 +144,33 @@ def main():
                 d[f"wlast_{l}"] = ref["wlast"][l]
             np.savez_compressed(os.path.join(HERE, f"train_{name}.npz"), **d)
             print(name, "epochs", epochs, "last", ref["epochs"][-1])
+        # dropout runs: the flags come from the reference's compiled Layer::generateDropout under srand(seed)
+        for (name, sizes, acts, cost, N, mb, epochs, lr, mom, wd1, wd2, params, seed, pd) in DROPOUT_CASES:
+            rng = np.random.default_rng(seed)
+            nl = len(sizes) - 1
+            spec = po.make_spec(sizes, acts, lr=lr, mom=mom, wd1=wd1, wd2=wd2, act_params=params, batch=mb, cost=cost)
+            Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * 0.5).astype(np.float32) for l in range(nl)]
+            bs = [0.0] + [float(np.float32(rng.standard_normal() * 0.1)) for _ in range(nl - 1)]
+            X = rng.random((N, sizes[0])).astype(np.float32)
+            Y = rng.random((N, sizes[-1])).astype(np.float32)
+            ref = po.ref_train(spec, Ws, bs, X, Y, epochs, td, dropout=(seed, pd))
+            assert all(np.isfinite(w).all() for w in ref["W"]), name
+            d = dict(sizes=np.array(sizes, np.int32), acts=np.array(acts, np.int32),
+                     hyper=np.array([lr, mom, wd1, wd2], np.float32),
+                     act_params=np.array(params if isinstance(params, list) else [params] * nl, np.float32),
+                     ints=np.array([cost, N, mb, epochs], np.int32), X=X, Y=Y, seed=np.int32(seed),
+                     p=np.array(pd, np.float32), masks=ref["masks"], rand_after=np.int32(ref["rand_after"]),
+                     bias0=np.array(bs, np.float32), epochs=ref["epochs"], bias=ref["bias"], preds=ref["preds"])
+            for l in range(nl):
+                d[f"W0_{l}"] = Ws[l]
+                d[f"W_{l}"] = ref["W"][l]
+                d[f"wsum_{l}"] = ref["wsum"][l]
+                d[f"wlast_{l}"] = ref["wlast"][l]
+                d[f"wcnt_{l}"] = ref["wcnt"][l]
+            for l in range(1, nl):
+                d[f"errder_{l}"] = ref["errder"][l - 1]
+            np.savez_compressed(os.path.join(HERE, f"dropout_{name}.npz"), **d)
+            print("dropout", name, "dropped %.2f" % ref["masks"].mean(), "last", ref["epochs"][-1])
 
 
 if __name__ == "__main__":

@@ -10,8 +10,14 @@ TRAIN_CASES = ["one_sample_2_3_2", "window_4_5_3_1", "decay_3_4_2", "cfg1_shape_
                "cfg2_shape_32_64_64_1", "mixed_5_7_6_4", "kl_3_5_4_2", "xornet", "iris"]
 
 
-def load_case(name):
-    d = np.load(os.path.join(GOLDEN, f"train_{name}.npz"), allow_pickle=False)
+DROPOUT_CASES = ["window_4_5_3_1", "decay_3_4_2", "out_of_range_6_8_2", "heavy_6_8_2", "batch1_5_7_6_4",
+                 "deep_64_48_6_2", "wide_1100_12_2"]
+
+
+def load_case(name, kind="train"):
+    """kind "train": runs without dropout; "dropout": runs whose flags the reference's compiled
+    Layer::generateDropout drew (d["masks"]: epochs x N x sum(sizes[:-1]), d["seed"], d["p"])."""
+    d = np.load(os.path.join(GOLDEN, f"{kind}_{name}.npz"), allow_pickle=False)
     sizes = [int(v) for v in d["sizes"]]
     nl = len(sizes) - 1
     cost, N, mb, epochs = [int(v) for v in d["ints"]]

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import pyoracle as po
-from helpers import GOLDEN, TRAIN_CASES, bits_equal, load_case
+from helpers import DROPOUT_CASES, GOLDEN, TRAIN_CASES, bits_equal, load_case
 
 
 def test_elementwise_grid_bit_exact():
@@ -64,6 +64,69 @@ def test_exact_training_bit_exact(name):
         assert bits_equal(s, d[f"wsum_{l}"]) and bits_equal(t, d[f"wlast_{l}"]), l
         if l >= 1:
             assert bits_equal(net.get_bias(l), d["bias"][l]), l
+
+
+@pytest.mark.parametrize("name", DROPOUT_CASES)
+def test_dropout_draw_and_training_bit_exact(name):
+    """Flags, rand() stream position and trained state against the reference's compiled
+    Layer::generateDropout / possiblePath / lastValidPath and Node/Edge objects."""
+    c = load_case(name, "dropout")
+    d = c["d"]
+    net = po.ExactNet(c["spec"])
+    for l in range(c["nl"]):
+        net.set_weights(l, c["W0"][l])
+        net.set_bias(l, c["bias0"][l])
+    po.libc_srand(int(d["seed"]))
+    eps = []
+    for ep in range(c["epochs"]):
+        masks = po.dropout_draw(c["spec"], d["p"], c["N"])
+        assert np.array_equal(masks, d["masks"][ep]), ep
+        m, preds = net.epoch(c["X"], c["Y"], masks=masks)
+        eps.append((m.loss, m.accuracy))
+    assert po.libc_rand() % 65536 == int(d["rand_after"])
+    assert bits_equal(np.array(eps, np.float32), d["epochs"])
+    assert bits_equal(preds, d["preds"])
+    for l in range(c["nl"]):
+        assert bits_equal(net.get_weights(l), d[f"W_{l}"]), l
+        s, t = net.get_window(l)
+        assert bits_equal(s, d[f"wsum_{l}"]) and bits_equal(t, d[f"wlast_{l}"]), l
+        assert np.array_equal(net.get_pending(l), d[f"wcnt_{l}"]), l
+        if l:
+            assert bits_equal(net.get_bias(l), d["bias"][l]), l
+            assert bits_equal(net.get_errder(l), d[f"errder_{l}"]), l
+
+
+def test_dropout_flags_change_the_result_and_zero_flags_do_not():
+    """All-zero flags reproduce the run without dropout; the fixture's flags do not (the test
+    above would pass vacuously if the flags were ignored)."""
+    c = load_case("window_4_5_3_1", "dropout")
+    outs = []
+    for masks in (None, np.zeros_like(c["d"]["masks"][0]), c["d"]["masks"][0]):
+        net = po.ExactNet(c["spec"])
+        for l in range(c["nl"]):
+            net.set_weights(l, c["W0"][l])
+            net.set_bias(l, c["bias0"][l])
+        net.epoch(c["X"], c["Y"], masks=masks)
+        outs.append([net.get_weights(l) for l in range(c["nl"])])
+    assert all(bits_equal(a, b) for a, b in zip(outs[0], outs[1]))
+    assert not all(bits_equal(a, b) for a, b in zip(outs[0], outs[2]))
+
+
+def test_dropped_hidden_node_outputs_squash_of_bias():
+    """network.cpp:491-516 finalises every output node at the last valid input: a dropped hidden
+    node still takes squash(0 + bias) (squash(0) in the first hidden layer), and feeds nothing on."""
+    spec = po.make_spec([2, 3, 1], [po.SIGMOID, po.LINEAR], act_params=[0, 1.0], lr=0.0)
+    net = po.ExactNet(spec)
+    net.set_weights(0, np.array([[1, 2], [3, 4], [5, 6]], np.float32))
+    net.set_weights(1, np.array([[1, 10, 100]], np.float32))
+    net.set_bias(1, 0.5)
+    X = np.array([[1.0, 1.0]], np.float32)
+    Y = np.zeros((1, 1), np.float32)
+    sig = lambda z: np.float32(po.lib().go_squash(float(z), po.SIGMOID, 0.0))
+    # drop input 1 and hidden node 1
+    _, p = net.epoch(X, Y, train=False, masks=np.array([[0, 1, 0, 1, 0]], np.uint8))
+    want = np.float32(np.float32(sig(1.0) * np.float32(1)) + np.float32(sig(5.0) * np.float32(100))) + np.float32(0.5)
+    assert bits_equal(p, np.array([[want]], np.float32))
 
 
 @pytest.mark.skipif(not po.have_ref(), reason="reference harness only exists in the build container")
