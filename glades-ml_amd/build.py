@@ -18,6 +18,11 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rd
              "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
              "-Wno-option-ignored", "-Wno-unused-result", "-Wno-inline-asm"]
 
+# Exact mode repeats the reference's fp32 arithmetic operation by operation: a product must be
+# rounded before it is added, so nothing in that file may be contracted into a fused multiply-add
+# (hipcc contracts by default, across the inlined __fmul_rn / __fadd_rn helpers too).
+PER_FILE_FLAGS = {"exact_kernel.hip": ["-ffp-contract=off"]}
+
 
 def _run(cmd):
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -38,7 +43,7 @@ def build_all(verbose=False):
 
     def one(pair):
         src, obj = pair
-        return _run([HIPCC] + HIP_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
+        return _run([HIPCC] + HIP_FLAGS + PER_FILE_FLAGS.get(src, []) + ["-c", os.path.join(CSRC, src), "-o", obj])
 
     with ThreadPoolExecutor(max_workers=min(6, len(srcs))) as ex:
         outs = list(ex.map(one, zip(srcs, objs)))

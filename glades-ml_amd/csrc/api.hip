@@ -61,6 +61,19 @@ struct ghip_net {
     int exMetricsCap = 0;
     int64_t exPredsCap = 0;
     int* exEpochs = nullptr;
+    // dropout: flags of the coming epochs, window lengths, error accumulators; once a run has used
+    // flags the accumulators may be non-zero between rows, so every later run keeps them too
+    unsigned char* exMasks = nullptr;
+    int exMaskEpochs = 0;
+    int64_t exMasksCap = 0;
+    int* exCnt = nullptr;
+    float* exErr = nullptr;
+    bool exDropState = false;
+    // the launches without dropout do not keep window lengths: there every edge of a layer holds
+    // the same number of pending deltas, noted here and written out when dropout state is first needed
+    int exUniformCnt[GHIP_MAX_LAYERS] = {};
+    size_t ex_lds_drop = 0;
+    int ex_drop_in_lds = 0;
     ExactPointers* exMulti = nullptr;  // pointer list of a launch over several networks (held by the first one)
     int exMultiCap = 0;
     int* cm = nullptr;              // confusion counters (both modes), n_out x n_out
@@ -237,21 +250,28 @@ int setup_exact(ghip_net* n)
         if (tw > T) tw = T;
         e.tw_log2[l] = ilog2(tw);
     }
-    size_t lds_full = ghip_exact_lds_bytes(e, true);
+    size_t lds_full = ghip_exact_lds_bytes(e, true, false);
     e.state_in_lds = lds_full <= (size_t)g_max_lds ? 1 : 0;
-    n->ex_lds = ghip_exact_lds_bytes(e, e.state_in_lds != 0);
+    n->ex_lds = ghip_exact_lds_bytes(e, e.state_in_lds != 0, false);
     if (n->ex_lds > (size_t)g_max_lds)
         return fail(GHIP_EINVAL, "exact mode: layers too wide (%zu bytes of node state exceed LDS)", n->ex_lds);
+    n->ex_drop_in_lds = ghip_exact_lds_bytes(e, true, true) <= (size_t)g_max_lds ? 1 : 0;
+    n->ex_lds_drop = ghip_exact_lds_bytes(e, n->ex_drop_in_lds != 0, true);
     TRY(dalloc(&n->exW, (size_t)woff));
     TRY(dalloc(&n->exSum, (size_t)woff));
     TRY(dalloc(&n->exLast, (size_t)woff));
     TRY(dalloc(&n->exBias, GHIP_MAX_LAYERS));
     TRY(dalloc(&n->exEpochs, 1));
+    TRY(dalloc(&n->exCnt, (size_t)woff));
+    TRY(dalloc(&n->exErr, (size_t)aoff));
+    HIP_TRY(hipMemsetAsync(n->exCnt, 0, sizeof(int) * woff, n->stream));
+    HIP_TRY(hipMemsetAsync(n->exErr, 0, sizeof(float) * aoff, n->stream));
     HIP_TRY(hipMemsetAsync(n->exW, 0, sizeof(float) * woff, n->stream));
     HIP_TRY(hipMemsetAsync(n->exSum, 0, sizeof(float) * woff, n->stream));
     HIP_TRY(hipMemsetAsync(n->exLast, 0, sizeof(float) * woff, n->stream));
     HIP_TRY(hipMemsetAsync(n->exBias, 0, sizeof(float) * GHIP_MAX_LAYERS, n->stream));
     e.ptr.W = n->exW; e.ptr.wsum = n->exSum; e.ptr.wlast = n->exLast; e.ptr.bias = n->exBias; e.ptr.epochs_run = n->exEpochs;
+    e.ptr.wcnt = n->exCnt; e.ptr.errder = n->exErr;
     return 0;
 }
 
@@ -587,6 +607,7 @@ int ghip_net_destroy(ghip_net* n)
     dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf);
     dfree(n->exW); dfree(n->exSum); dfree(n->exLast); dfree(n->exBias); dfree(n->exPreds);
     dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass); dfree(n->exMulti);
+    dfree(n->exMasks); dfree(n->exCnt); dfree(n->exErr);
     for (int l = 0; l < GHIP_MAX_LAYERS; ++l) {
         dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]); dfree(n->gW[l]);
         dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
@@ -611,6 +632,8 @@ int ghip_net_set_params(ghip_net* n, int layer, const float* host_W, const float
             HIP_TRY(hipMemcpyAsync(n->exW + n->ex.woff[layer], pad.data(), pad.size() * 4, hipMemcpyHostToDevice, n->stream));
             HIP_TRY(hipMemsetAsync(n->exSum + n->ex.woff[layer], 0, pad.size() * 4, n->stream));
             HIP_TRY(hipMemsetAsync(n->exLast + n->ex.woff[layer], 0, pad.size() * 4, n->stream));
+            HIP_TRY(hipMemsetAsync(n->exCnt + n->ex.woff[layer], 0, pad.size() * 4, n->stream));
+            n->exUniformCnt[layer] = 0;
             HIP_TRY(hipStreamSynchronize(n->stream));
         }
         if (host_bias && bias_len == 1) {
@@ -696,6 +719,93 @@ int ghip_net_set_state(ghip_net* n, int layer, const float* host_a, const float*
     return move_state(n, layer, const_cast<float*>(host_a), const_cast<float*>(host_b), 1);
 }
 
+int ghip_net_set_dropout_masks(ghip_net* n, const uint8_t* host_masks, int n_epochs)
+{
+    if (!n) return fail(GHIP_EINVAL, "bad net");
+    HIP_TRY(hipSetDevice(g_device));
+    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "dropout flags belong to exact mode");
+    if (!host_masks) {
+        n->exMaskEpochs = 0;
+        return 0;
+    }
+    if (n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset (the flags are per row of the table)");
+    const int64_t len = (int64_t)n_epochs * n->n_rows * n->ex.aoff[n->L];
+    for (int64_t k = 0; k < len; ++k)
+        if (host_masks[k] > 1) return fail(GHIP_EINVAL, "flag %lld is %d, not 0 or 1", (long long)k, (int)host_masks[k]);
+    // a layer with every node dropped would never finalise the next layer (Layer::lastValidPath,
+    // ML/State/layer.cpp:168-183); the reference redraws such a layer (layer.cpp:114-133)
+    {
+        const uint8_t* m = host_masks;
+        for (int64_t row = 0; row < (int64_t)n_epochs * n->n_rows; ++row)
+            for (int l = 0; l < n->L; ++l) {
+                int valid = 0;
+                for (int i = 0; i < n->spec.sizes[l]; ++i) valid += m[i] ? 0 : 1;
+                if (!valid) return fail(GHIP_EINVAL, "row %lld drops every node of layer %d", (long long)row, l);
+                m += n->spec.sizes[l];
+            }
+    }
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    if (len > n->exMasksCap) {
+        dfree(n->exMasks);
+        TRY(dalloc(&n->exMasks, (size_t)len));
+        n->exMasksCap = len;
+    }
+    HIP_TRY(hipMemcpy(n->exMasks, host_masks, (size_t)len, hipMemcpyHostToDevice));
+    n->exMaskEpochs = n_epochs;
+    return 0;
+}
+
+// Window lengths of a network that has only run without dropout: the same for every edge of a layer.
+static int materialize_counts(ghip_net* n)
+{
+    if (n->exDropState) return 0;
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    for (int l = 0; l < n->L; ++l) {
+        std::vector<int32_t> pad((size_t)n->ex.ld[l] * n->spec.sizes[l + 1], n->exUniformCnt[l]);
+        HIP_TRY(hipMemcpy(n->exCnt + n->ex.woff[l], pad.data(), pad.size() * 4, hipMemcpyHostToDevice));
+    }
+    return 0;
+}
+
+// direction 0: device -> host, 1: host -> device
+static int move_dropout_state(ghip_net* n, int layer, int32_t* counts, float* errder, int to_device)
+{
+    if (!n || layer < 0 || layer >= n->L) return fail(GHIP_EINVAL, "bad net or layer");
+    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "dropout state belongs to exact mode");
+    HIP_TRY(hipSetDevice(g_device));
+    const int ni = n->spec.sizes[layer], no = n->spec.sizes[layer + 1], ld = n->ex.ld[layer];
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    TRY(materialize_counts(n));
+    if (counts) {
+        std::vector<int32_t> pad((size_t)ld * no, 0);
+        int* dev = n->exCnt + n->ex.woff[layer];
+        if (to_device) {
+            for (int o = 0; o < no; ++o) memcpy(&pad[(size_t)o * ld], counts + (size_t)o * ni, sizeof(int32_t) * ni);
+            HIP_TRY(hipMemcpy(dev, pad.data(), pad.size() * 4, hipMemcpyHostToDevice));
+        } else {
+            HIP_TRY(hipMemcpy(pad.data(), dev, pad.size() * 4, hipMemcpyDeviceToHost));
+            for (int o = 0; o < no; ++o) memcpy(counts + (size_t)o * ni, &pad[(size_t)o * ld], sizeof(int32_t) * ni);
+        }
+    }
+    if (errder) {
+        float* dev = n->exErr + n->ex.aoff[layer + 1];
+        HIP_TRY(to_device ? hipMemcpy(dev, errder, (size_t)no * 4, hipMemcpyHostToDevice)
+                          : hipMemcpy(errder, dev, (size_t)no * 4, hipMemcpyDeviceToHost));
+    }
+    if (to_device) n->exDropState = true;
+    return 0;
+}
+
+int ghip_net_get_dropout_state(ghip_net* n, int layer, int32_t* host_counts, float* host_errder)
+{
+    return move_dropout_state(n, layer, host_counts, host_errder, 0);
+}
+int ghip_net_set_dropout_state(ghip_net* n, int layer, const int32_t* host_counts, const float* host_errder)
+{
+    return move_dropout_state(n, layer, const_cast<int32_t*>(host_counts), const_cast<float*>(host_errder), 1);
+}
+
 static int make_bf16_table(ghip_net* n)
 {
     const ghip_net_spec& s = n->spec;
@@ -755,6 +865,12 @@ static int exact_prepare(ghip_net* n, int n_epochs, bool want_preds, ExactPointe
         n->exPredsCap = n->n_rows * nout;
     }
     *ptr = n->ex.ptr;
+    ptr->masks = nullptr;
+    if (n->exMaskEpochs > 0) {
+        if (n_epochs > n->exMaskEpochs)
+            return fail(GHIP_EINVAL, "%d epochs asked for, dropout flags for %d", n_epochs, n->exMaskEpochs);
+        ptr->masks = n->exMasks;
+    }
     ptr->preds = want_preds ? n->exPreds : nullptr;
     ptr->metrics = (float*)n->exMetrics;
     ptr->cm = n->cm;
@@ -784,7 +900,20 @@ int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_a
     TRY(exact_prepare(n, n_epochs, host_preds != nullptr, &e.ptr));
     e.X = n->dX; e.Y = n->dY; e.n_rows = n->n_rows;
     e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
-    LAUNCH(n, "exact_epochs", ghip_launch_exact(e, nullptr, 1, n->ex_threads, n->ex_lds, n->stream));
+    size_t lds = n->ex_lds;
+    if (e.ptr.masks || n->exDropState) {
+        TRY(materialize_counts(n));
+        e.dropout = 1;
+        e.state_in_lds = n->ex_drop_in_lds;
+        lds = n->ex_lds_drop;
+        n->exDropState = true;
+        n->exMaskEpochs = 0;  // flags are used once
+    }
+    else if (e.train) {
+        // rows after the last applying one each pushed a delta (network.cpp:647-651)
+        for (int l = 0; l < n->L; ++l) n->exUniformCnt[l] = (int)((n->n_rows - 1) % n->spec.batch);
+    }
+    LAUNCH(n, e.dropout ? "exact_epochs_dropout" : "exact_epochs", ghip_launch_exact(e, nullptr, 1, n->ex_threads, lds, n->stream));
     int ran = 0;
     HIP_TRY(hipMemcpyAsync(&ran, n->exEpochs, sizeof(int), hipMemcpyDeviceToHost, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
@@ -829,7 +958,24 @@ int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epoc
     // reference trains every subnet of a MetaNetwork on the same DataInput, ML/main.cpp:137-160)
     e.X = lead->dX; e.Y = lead->dY; e.n_rows = lead->n_rows;
     e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
-    LAUNCH(lead, "exact_epochs_multi", ghip_launch_exact(e, lead->exMulti, count, lead->ex_threads, lead->ex_lds, lead->stream));
+    size_t lds = lead->ex_lds;
+    bool any_drop = false;
+    for (int k = 0; k < count; ++k) any_drop = any_drop || list[k].masks || nets[k]->exDropState;
+    if (any_drop) {
+        e.dropout = 1;
+        e.state_in_lds = lead->ex_drop_in_lds;
+        lds = lead->ex_lds_drop;
+        for (int k = 0; k < count; ++k) {
+            TRY(materialize_counts(nets[k]));
+            nets[k]->exDropState = true;
+            nets[k]->exMaskEpochs = 0;
+        }
+    } else if (e.train) {
+        for (int k = 0; k < count; ++k)
+            for (int l = 0; l < lead->L; ++l) nets[k]->exUniformCnt[l] = (int)((lead->n_rows - 1) % lead->spec.batch);
+    }
+    LAUNCH(lead, any_drop ? "exact_epochs_multi_dropout" : "exact_epochs_multi",
+           ghip_launch_exact(e, lead->exMulti, count, lead->ex_threads, lds, lead->stream));
     HIP_TRY(hipStreamSynchronize(lead->stream));
     for (int k = 0; k < count; ++k) {
         int ran = 0;

@@ -10,12 +10,25 @@
 //   back-prop    one lane per input node, outputs visited in ascending order with the
 //                reference's doubling accumulator  e <- e + (e + d*w)   (network.cpp:660-662)
 //   bias, loss   one wavefront / one designated lane, in the reference's visiting order
-// Every fp32 operation is written with explicit round-to-nearest intrinsics so that nothing is
-// contracted into an FMA or re-associated: the arithmetic order is the reference's.
+// Every fp32 operation is written as a separate round-to-nearest step in the reference's order, and
+// the file is compiled with contraction off (the pragma below and -ffp-contract=off in the build):
+// hipcc would otherwise fuse a product with the addition that follows it, also through the
+// __fmul_rn / __fadd_rn helpers, which are plain operators.
+//
+// Dropout (the kDrop instantiation) takes the flags of every row from a table the host drew
+// (LayerBuilder::scrambleDropout, "Backend/Machine Learning/State/LayerBuilder.cpp":497-523) and
+// follows what the reference does with them: a dropped pair sets no edge activation and gets no
+// delta, the output node is finalised regardless (a dropped hidden node becomes squash(bias)), a
+// dropped pair still hands the output node's error accumulator down (without the derivative
+// factor), and the accumulator of an output node is only cleared by a valid pair with the LAST
+// input node -- so it can survive into the next row, the next epoch and the next call
+// (network.cpp:480-516, 621-662).
 //
 // Weights, pending-delta sums and last deltas live in LDS for the whole call (3 floats per edge,
 // rows padded to an odd stride so that lane-per-row and lane-per-column walks are both free of
 // bank conflicts); networks too large for LDS keep them in global memory (L2 resident).
+
+#pragma clang fp contract(off)
 
 #include "ghip_internal.h"
 
@@ -27,12 +40,14 @@ constexpr int kPrefetch = 4;  // values per lane of the next row held in registe
 // bias -= lr*d[o] for o = 0..n_out-1, repeated n_in times -- one dependent chain of n_in*n_out fp32
 // subtractions whose rounding order must be kept.  The n_out values sit in NP registers (padded
 // with zeros: b - 0 is exact), so a step is a single subtract with no memory access.
+// With dropout only valid pairs take part: dropped output nodes (mo[k] != 0) subtract an exact zero
+// and ni counts the valid input nodes.
 template <int NP>
-__device__ __forceinline__ float bias_chain(float b, const float* bs, int no, int ni)
+__device__ __forceinline__ float bias_chain(float b, const float* bs, int no, int ni, const int* mo = nullptr)
 {
     float x[NP];
 #pragma unroll
-    for (int k = 0; k < NP; ++k) x[k] = (k < no) ? bs[k] : 0.0f;
+    for (int k = 0; k < NP; ++k) x[k] = (k < no && !(mo && mo[k])) ? bs[k] : 0.0f;
     for (int i = 0; i < ni; ++i) {
 #pragma unroll
         for (int k = 0; k < NP; ++k) b = __fsub_rn(b, x[k]);
@@ -44,7 +59,7 @@ __device__ __forceinline__ float bias_chain(float b, const float* bs, int no, in
 // table; with `multi` each workgroup b takes its own parameter / result pointers from multi[b]
 // (the subnets of a MetaNetwork train at the same time, one per compute unit), without it the
 // single network's pointers are the ones in `p`.
-template <bool kLds>
+template <bool kLds, bool kDrop>
 __global__ void __launch_bounds__(1024)
 exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 {
@@ -79,7 +94,18 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     float* sy = nodes + 3 * p.node_floats;  // expected row
     float* sbias = sy + nout;               // GHIP_MAX_LAYERS scalars
     int* sflag = (int*)(sbias + GHIP_MAX_LAYERS);
+    // dropout only: the row's flags (1 = dropped; output layer always 0) and the nodes' error
+    // accumulators (Node::errorDer), which outlive the row
+    int* sm = sflag + 4;
+    float* sE = (float*)(sm + p.node_floats);
+    const int mask_len = p.aoff[L];  // flags of one row: the non-output layers side by side
 
+    if (kDrop) {
+        for (int k = tid; k < p.node_floats; k += T) {
+            sm[k] = 0;
+            sE[k] = own.errder[k];
+        }
+    }
     if (kLds) {
         for (int k = tid; k < S; k += T) {
             sW[k] = own.W[k];
@@ -137,6 +163,10 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 for (int i = tid; i < n0; i += T) sa[i] = p.X[r * n0 + i];
                 for (int i = tid; i < nout; i += T) sy[i] = p.Y[r * nout + i];
             }
+            if (kDrop && own.masks) {
+                const unsigned char* mr = own.masks + ((long long)ep * p.n_rows + r) * mask_len;
+                for (int k = tid; k < mask_len; k += T) sm[k] = mr[k];
+            }
             __syncthreads();
 
             // ---- ForwardPass (network.cpp:457-516)
@@ -148,11 +178,22 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 const int act = p.act[l];
                 const float par = p.act_param[l];
                 const float bl = sbias[l];
+                const int* mi = sm + p.aoff[l];
+                const int* mo = sm + p.aoff[l + 1];
                 for (int o = tid; o < no; o += T) {
                     const float* w = Wl + o * ld;
                     float z = 0.0f;
+                    if (kDrop) {
+                        // the sum starts at +0 and never becomes -0, so adding +0 for a dropped
+                        // pair leaves it as skipping the pair does
+                        const bool vo = !mo[o];
+#pragma unroll 8
+                        for (int i = 0; i < ni; ++i)
+                            z = __fadd_rn(z, (vo && !mi[i]) ? __fmul_rn(w[i], ain[i]) : 0.0f);
+                    } else {
 #pragma unroll 16
-                    for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
+                        for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
+                    }
                     if (l != 0) z = __fadd_rn(z, bl);
                     aout[o] = ghip_squash<true>(z, act, par);
                 }
@@ -188,6 +229,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         float e = __fadd_rn(0.0f, ghip_cost_der(sy[o], pred[o], p.cost));
                         dl[o] = e;
                         bs[o] = __fmul_rn(lr, e);
+                        if (kDrop) sE[p.aoff[L] + o] = e;
                     }
                 }
                 __syncthreads();
@@ -203,21 +245,34 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     const float* bs = sbase + p.aoff[Lo];
                     const float lr = p.lr[l], mom = p.mom[l];
                     const float w1 = __fmul_rn(p.wd1[l], lr), w2 = __fmul_rn(p.wd2[l], lr);
+                    const int* mi = sm + p.aoff[l];
+                    const int* mo = sm + p.aoff[Lo];
+                    const float* raw = sE + p.aoff[Lo];  // the out-layer's accumulators as they stand
                     // ---- per-edge delta push and conditional apply (node.cpp:278-307)
                     {
                         const int sh = p.tw_log2[l];
                         const int tw = 1 << sh;
                         const int i0 = tid & (tw - 1), o0 = tid >> sh, rpp = T >> sh;
+                        // an edge that sat out an applying row can hold more than mb pending deltas;
+                        // applyDeltas reads the first mb only (node.cpp:299-301), so their number is kept
+                        int* Cl = (kDrop && p.mb > 1) ? own.wcnt + p.woff[l] : nullptr;
                         for (int i = i0; i < ni; i += tw) {
+                            if (kDrop && mi[i]) continue;
                             const float a = ain[i];
                             const float t1 = __fmul_rn(w1, fabsf(a));
                             const float t2 = __fmul_rn(w2, a);
                             for (int o = o0; o < no; o += rpp) {
+                                if (kDrop && mo[o]) continue;
                                 const int k = o * ld + i;
                                 float dW = __fadd_rn(__fmul_rn(bs[o], a), __fmul_rn(mom, Ll[k]));
                                 dW = __fadd_rn(dW, t1);
                                 dW = __fadd_rn(dW, t2);
                                 float s = __fadd_rn(Sl[k], dW);
+                                if (Cl) {
+                                    const int c = Cl[k];
+                                    if (c >= p.mb) s = Sl[k];
+                                    Cl[k] = apply ? 0 : c + 1;
+                                }
                                 if (apply) {
                                     Wl[k] = __fsub_rn(Wl[k], __fdiv_rn(s, fmb));
                                     Sl[k] = 0.0f;
@@ -234,22 +289,29 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     // wavefront with the lr*d values held in registers (bias_chain below).
                     if ((tid >> 6) == (T >> 6) - 1 && l != 0) {
                         float b = sbias[l];
+                        int nv = ni;  // input nodes taking part
+                        const int* mk = nullptr;
+                        if (kDrop) {
+                            nv = 0;
+                            for (int i = 0; i < ni; ++i) nv += mi[i] ? 0 : 1;
+                            mk = mo;
+                        }
                         if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
-                            if (no <= 4) b = bias_chain<4>(b, bs, no, ni);
-                            else if (no <= 8) b = bias_chain<8>(b, bs, no, ni);
-                            else if (no <= 16) b = bias_chain<16>(b, bs, no, ni);
-                            else if (no <= 32) b = bias_chain<32>(b, bs, no, ni);
-                            else if (no <= 64) b = bias_chain<64>(b, bs, no, ni);
+                            if (no <= 4) b = bias_chain<4>(b, bs, no, nv, mk);
+                            else if (no <= 8) b = bias_chain<8>(b, bs, no, nv, mk);
+                            else if (no <= 16) b = bias_chain<16>(b, bs, no, nv, mk);
+                            else if (no <= 32) b = bias_chain<32>(b, bs, no, nv, mk);
+                            else if (no <= 64) b = bias_chain<64>(b, bs, no, nv, mk);
                             else {
-                                for (int i = 0; i < ni; ++i) {
+                                for (int i = 0; i < nv; ++i) {
 #pragma unroll 8
-                                    for (int o = 0; o < no; ++o) b = __fsub_rn(b, bs[o]);
+                                    for (int o = 0; o < no; ++o) b = __fsub_rn(b, (mk && mk[o]) ? 0.0f : bs[o]);
                                 }
                             }
                         } else {
                             float s = 0.0f;
-                            for (int o = 0; o < no; ++o) s = __fadd_rn(s, bs[o]);
-                            b = __fsub_rn(b, __fmul_rn((float)ni, s));
+                            for (int o = 0; o < no; ++o) s = __fadd_rn(s, (mk && mk[o]) ? 0.0f : bs[o]);
+                            b = __fsub_rn(b, __fmul_rn((float)nv, s));
                         }
                         if (tid == serial) sbias[l] = b;
                     }
@@ -263,14 +325,35 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         const float lrn = p.lr[l - 1];
                         for (int i = tid; i < ni; i += T) {
                             float e = 0.0f;
+                            if (kDrop) {
+                                // starts from what earlier rows left; a dropped pair hands down the
+                                // out-node's accumulator without the derivative factor
+                                e = sE[p.aoff[l] + i];
+                                const bool di = mi[i] != 0;
+#pragma unroll 8
+                                for (int o = 0; o < no; ++o) {
+                                    const float c = (di || mo[o]) ? raw[o] : dl[o];
+                                    e = __fadd_rn(e, __fadd_rn(e, __fmul_rn(c, Wl[o * ld + i])));
+                                }
+                                sE[p.aoff[l] + i] = e;
+                            } else {
 #pragma unroll 16
-                            for (int o = 0; o < no; ++o)
-                                e = __fadd_rn(e, __fadd_rn(e, __fmul_rn(dl[o], Wl[o * ld + i])));
+                                for (int o = 0; o < no; ++o)
+                                    e = __fadd_rn(e, __fadd_rn(e, __fmul_rn(dl[o], Wl[o * ld + i])));
+                            }
                             // the reference always passes 0.01 here (network.cpp:617-618)
                             float d = __fmul_rn(e, ghip_act_der_ref(ain[i], actp, 0.01f));
                             dn[i] = d;
                             bn[i] = __fmul_rn(lrn, d);
                         }
+                        __syncthreads();
+                    }
+                    if (kDrop && Lo < L) {
+                        // clearErrDer of the out-layer's nodes: only by a valid pair with the last
+                        // input node (network.cpp:629-631)
+                        if (!mi[ni - 1])
+                            for (int o = tid; o < no; o += T)
+                                if (!mo[o]) sE[p.aoff[Lo] + o] = 0.0f;
                         __syncthreads();
                     }
                 }
@@ -302,28 +385,40 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     }
     if (tid < GHIP_MAX_LAYERS) own.bias[tid] = sbias[tid];
     if (tid == 0) own.epochs_run[0] = ep;
+    if (kDrop)
+        for (int k = tid; k < p.node_floats; k += T) own.errder[k] = sE[k];
 }
 
 }  // namespace
 
-size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds)
+size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropout)
 {
     size_t f = (size_t)3 * p.node_floats + p.sizes[p.n_layers] + GHIP_MAX_LAYERS + 4;
+    if (dropout) f += (size_t)2 * p.node_floats;
     if (state_in_lds) f += (size_t)3 * p.state_floats;
     return f * sizeof(float);
+}
+
+template <bool kLds, bool kDrop>
+static hipError_t launch_variant(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads,
+                                 size_t lds_bytes, hipStream_t s)
+{
+    if (kLds) {
+        hipError_t e = hipFuncSetAttribute((const void*)exact_kernel<kLds, kDrop>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((exact_kernel<kLds, kDrop>), dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
+    return hipGetLastError();
 }
 
 hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads, size_t lds_bytes,
                              hipStream_t s)
 {
-    hipError_t e;
-    if (p.state_in_lds) {
-        e = hipFuncSetAttribute((const void*)exact_kernel<true>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds_bytes);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(exact_kernel<true>, dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
-    } else {
-        hipLaunchKernelGGL(exact_kernel<false>, dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
+    if (p.dropout) {
+        if (p.state_in_lds) return launch_variant<true, true>(p, dev_multi, count, threads, lds_bytes, s);
+        return launch_variant<false, true>(p, dev_multi, count, threads, lds_bytes, s);
     }
-    return hipGetLastError();
+    if (p.state_in_lds) return launch_variant<true, false>(p, dev_multi, count, threads, lds_bytes, s);
+    return launch_variant<false, false>(p, dev_multi, count, threads, lds_bytes, s);
 }

@@ -211,6 +211,10 @@ struct ExactPointers {
     int*   epochs_run;
     int*   cm;            // n_out x n_out confusion counters of the running epoch, or NULL
     float* class_metrics; // per epoch: overall accuracy, precision, recall, specificity, F1 (NULL with cm)
+    // dropout launches only
+    const unsigned char* masks; // n_epochs x n_rows x aoff[n_layers] flags (1 = dropped) or NULL = none dropped
+    int*   wcnt;                // [state_floats] number of pending deltas per edge
+    float* errder;              // [node_floats] the nodes' error accumulators between rows
 };
 
 struct ExactLaunch {
@@ -233,12 +237,13 @@ struct ExactLaunch {
     const float* Y;
     ExactPointers ptr;  // this network's own arrays (a launch over several networks passes a list instead)
     int    state_in_lds;
+    int    dropout;     // run the instantiation that reads flags and keeps accumulators / window lengths
 };
 
 // count workgroups = count networks; dev_multi (device memory, count entries) or NULL for the one network in p.ptr
 hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads, size_t lds_bytes,
                              hipStream_t s);
-size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds);
+size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropout);
 
 // ---------------------------------------------------------------- canonical kernels
 

@@ -21,6 +21,7 @@ BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
 EXPORTS = [
     "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
     "ghip_net_get_state", "ghip_net_set_state",
+    "ghip_net_set_dropout_masks", "ghip_net_get_dropout_state", "ghip_net_set_dropout_state",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
     "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
@@ -79,6 +80,9 @@ def load():
             "ghip_net_get_params": (i, [vp, i, vp, vp, i]),
             "ghip_net_get_state": (i, [vp, i, vp, vp]),
             "ghip_net_set_state": (i, [vp, i, vp, vp]),
+            "ghip_net_set_dropout_masks": (i, [vp, vp, i]),
+            "ghip_net_get_dropout_state": (i, [vp, i, vp, vp]),
+            "ghip_net_set_dropout_state": (i, [vp, i, vp, vp]),
             "ghip_net_set_dataset": (i, [vp, vp, vp, i64]),
             "ghip_net_set_dataset_device": (i, [vp, vp, vp, i64]),
             "ghip_net_run_epochs_exact": (i, [vp, i, i, f, vp, C.POINTER(i), vp]),
@@ -192,6 +196,27 @@ class Net:
         a = np.ascontiguousarray(a, np.float32)
         b = np.ascontiguousarray(b, np.float32)
         _check(self.lib.ghip_net_set_state(self.h, l, _ptr(a), _ptr(b)))
+
+    def set_dropout_masks(self, masks):
+        """masks: epochs x n_rows x sum(sizes[:-1]) uint8 (1 = dropped) for the next exact run, or None."""
+        if masks is None:
+            _check(self.lib.ghip_net_set_dropout_masks(self.h, None, 0))
+            return
+        masks = np.ascontiguousarray(masks, np.uint8)
+        assert masks.ndim == 3 and masks.shape[1:] == (self.n_rows, sum(self.sizes[:-1])), masks.shape
+        _check(self.lib.ghip_net_set_dropout_masks(self.h, _ptr(masks), masks.shape[0]))
+
+    def get_dropout_state(self, l):
+        """(pending-delta counts of weight layer l, error accumulators of the nodes of layer l+1)."""
+        c = np.empty((self.sizes[l + 1], self.sizes[l]), np.int32)
+        e = np.empty(self.sizes[l + 1], np.float32)
+        _check(self.lib.ghip_net_get_dropout_state(self.h, l, _ptr(c), _ptr(e)))
+        return c, e
+
+    def set_dropout_state(self, l, counts, errder):
+        c = None if counts is None else np.ascontiguousarray(counts, np.int32)
+        e = None if errder is None else np.ascontiguousarray(errder, np.float32)
+        _check(self.lib.ghip_net_set_dropout_state(self.h, l, _ptr(c), _ptr(e)))
 
     # ---- data
     def set_dataset(self, X, Y):

@@ -119,6 +119,27 @@ int ghip_net_get_params(ghip_net* net, int layer, float* host_W, float* host_bia
 int ghip_net_get_state(ghip_net* net, int layer, float* host_a, float* host_b);
 int ghip_net_set_state(ghip_net* net, int layer, const float* host_a, const float* host_b);
 
+/* Dropout (exact mode): replaces LayerBuilder::scrambleDropout (ML/State/LayerBuilder.cpp:497-523)
+ * as the source of the per-row flags and Layer::possiblePath / lastValidPath
+ * (ML/State/layer.cpp:136-183) as their readers.  The caller draws the flags -- the reference draws
+ * them from libc rand() (Layer::generateDropout, ML/State/layer.cpp:102-134), a stream that lives on
+ * the host -- and hands over n_epochs x n_rows x (sizes[0] + ... + sizes[n_layers-1]) bytes: for
+ * every epoch and row the node layers 0..n_layers-1 side by side, 1 = dropped.  The next
+ * ghip_net_run_epochs_exact / _multi call (train or test: the reference scrambles in both,
+ * ML/Networks/network.cpp:407-411) consumes them and must not ask for more epochs; later calls run
+ * without dropout until flags are set again.  A row that drops every node of a layer is refused
+ * (the reference redraws such a layer).  Needs the table (ghip_net_set_dataset) first.
+ * NULL forgets flags that were set. */
+int ghip_net_set_dropout_masks(ghip_net* net, const uint8_t* host_masks, int n_epochs);
+/* What dropout leaves behind between rows, for checkpoints: the number of pending deltas of every
+ * edge of weight layer `layer` (Edge::prevDelta.size(), ML/State/edge.cpp:64-67; sizes[layer+1] x
+ * sizes[layer]: an edge that sat out an applying row keeps its window, and Node::applyDeltas reads
+ * the first minibatchSize entries only, ML/State/node.cpp:294-307) and the error accumulators of
+ * the nodes of layer `layer`+1 (Node::errorDer, cleared only by a valid pair with the last input
+ * node, ML/Networks/network.cpp:629-631; sizes[layer+1]).  Either pointer may be NULL. */
+int ghip_net_get_dropout_state(ghip_net* net, int layer, int32_t* host_counts, float* host_errder);
+int ghip_net_set_dropout_state(ghip_net* net, int layer, const int32_t* host_counts, const float* host_errder);
+
 /* Uploads the training table once: replaces LayerBuilder::buildInputLayers
  * (ML/State/LayerBuilder.cpp:100-190) and DataInput::getTrainRow / getTrainExpectedRow
  * (ML/DataObjects/DataInput.h:39-40).  X is N x sizes[0], Y is N x sizes[n_layers]. */

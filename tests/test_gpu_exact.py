@@ -139,6 +139,30 @@ def test_edge_shapes_against_oracle(sizes, N, mb):
     net.close()
 
 
+@pytest.mark.parametrize("name", ["mixed_5_7_6_4", "one_sample_2_3_2"])
+def test_fixtures_without_libm_calls_are_bit_exact(name):
+    """Where the trained state depends on no libm routine the device must reproduce the reference's
+    compiled objects bit for bit: every product is rounded before it is added (no fused
+    multiply-add), in the reference's order.  mixed_5_7_6_4: RELU / LEAKY / SIGMOIDP whose sigmoid
+    branch the data never reaches, momentum, both decays, minibatch 5; the loss goes through logf
+    and is held to the tolerance only."""
+    from helpers import bits_equal
+    c = load_case(name)
+    d = c["d"]
+    net = gpu_net(c)
+    ms, preds = net.run_epochs_exact(c["epochs"], want_preds=True)
+    assert bits_equal(preds, d["preds"])
+    assert bits_equal([m[1] for m in ms], d["epochs"][:, 1])
+    for l in range(c["nl"]):
+        W, b = net.get_params(l)
+        assert bits_equal(W, d[f"W_{l}"]), l
+        s, t = net.get_state(l)
+        assert bits_equal(s, d[f"wsum_{l}"]) and bits_equal(t, d[f"wlast_{l}"]), l
+        if l >= 1:
+            assert bits_equal(b[0], d["bias"][l]), l
+    net.close()
+
+
 def test_error_paths():
     import pyglades as pg
     with pytest.raises(pg.GladesHipError):   # BATCH_FULL = 0 is "row % 0" in the reference
