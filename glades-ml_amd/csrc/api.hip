@@ -576,6 +576,20 @@ int ghip_init(int device_ordinal)
     int lds = 0;
     if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, device_ordinal) == hipSuccess && lds > 0)
         g_max_lds = lds;
+    // The runtime completes its own set-up inside the first stream creation / allocation, and that
+    // set-up draws from libc rand().  The reference's weight sampler and dropout read the same
+    // stream, so it is done here: a caller who seeds rand() after this call finds the stream
+    // untouched by the calls that follow.
+    {
+        hipStream_t s = nullptr;
+        void* p = nullptr;
+        HIP_TRY(hipStreamCreate(&s));
+        HIP_TRY(hipMalloc(&p, 256));
+        HIP_TRY(hipMemsetAsync(p, 0, 256, s));
+        HIP_TRY(hipStreamSynchronize(s));
+        HIP_TRY(hipFree(p));
+        HIP_TRY(hipStreamDestroy(s));
+    }
     g_device = device_ordinal;
     return 0;
 }

@@ -329,7 +329,7 @@ NNetwork::NNetwork()
     : di(NULL), skeleton(NULL), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
       dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
-      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false)
 {
 }
 
@@ -337,7 +337,7 @@ NNetwork::NNetwork(NNInfo* newNNInfo)
     : di(NULL), skeleton(newNNInfo), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
       dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
-      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0)
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false)
 {
 }
 
@@ -363,7 +363,8 @@ bool NNetwork::load(const std::string& path)
 bool NNetwork::save(const std::string& path) const { return skeleton ? skeleton->saveFile(path) : false; }
 
 // file: "GLCK" u32 version, i32 mode, i32 dtype, i32 epochs, i32 nLayers, i32 sizes[nLayers+1],
-//       u32 tableBytes, table text (the NNInfo CSV), then per layer: W, u32 biasLen, bias, u32 aLen, a, u32 bLen, b
+//       u32 tableBytes, table text (the NNInfo CSV), then per layer: W, u32 biasLen, bias, u32 aLen, a, u32 bLen, b,
+//       and from version 2 on u32 cLen, window lengths (i32), u32 eLen, node error accumulators (exact mode; else 0, 0)
 bool NNetwork::saveCheckpoint(const std::string& path)
 {
     if (!skeleton || !dev) { lastError = "nothing to checkpoint: the network has not run"; return false; }
@@ -385,7 +386,7 @@ bool NNetwork::saveCheckpoint(const std::string& path)
     }
     FILE* f = fopen(path.c_str(), "wb");
     if (!f) { lastError = "cannot write " + path; return false; }
-    const uint32_t version = 1, tb = (uint32_t)table.size();
+    const uint32_t version = 2, tb = (uint32_t)table.size();
     const int32_t head[4] = {mode, dtype, epochs, L};
     fwrite("GLCK", 1, 4, f); fwrite(&version, 4, 1, f); fwrite(head, 4, 4, f); fwrite(sizes.data(), 4, sizes.size(), f);
     fwrite(&tb, 4, 1, f); fwrite(table.data(), 1, table.size(), f);
@@ -401,6 +402,12 @@ bool NNetwork::saveCheckpoint(const std::string& path)
         fwrite(&bl, 4, 1, f); fwrite(b.data(), 4, bl, f);
         fwrite(&al, 4, 1, f); fwrite(sa.data(), 4, al, f);
         fwrite(&sl, 4, 1, f); fwrite(sb.data(), 4, sl, f);
+        const uint32_t cl = mode == MODE_EXACT ? (uint32_t)cnt : 0u, el = mode == MODE_EXACT ? (uint32_t)sizes[l + 1] : 0u;
+        std::vector<int32_t> wc(cl);
+        std::vector<float> ed(el);
+        if (cl && ghip_net_get_dropout_state(dev, l, wc.data(), ed.data()) != 0) { ok = false; lastError = ghip_last_error(); break; }
+        fwrite(&cl, 4, 1, f); fwrite(wc.data(), 4, cl, f);
+        fwrite(&el, 4, 1, f); fwrite(ed.data(), 4, el, f);
     }
     fclose(f);
     return ok;
@@ -413,7 +420,7 @@ bool NNetwork::loadCheckpoint(const std::string& path)
     char magic[4];
     uint32_t version = 0, tb = 0;
     int32_t head[4];
-    bool ok = fread(magic, 1, 4, f) == 4 && memcmp(magic, "GLCK", 4) == 0 && fread(&version, 4, 1, f) == 1 && version == 1 &&
+    bool ok = fread(magic, 1, 4, f) == 4 && memcmp(magic, "GLCK", 4) == 0 && fread(&version, 4, 1, f) == 1 && (version == 1 || version == 2) &&
               fread(head, 4, 4, f) == 4 && head[3] >= 1 && head[3] <= 16;
     std::vector<int32_t> sizes;
     std::string table;
@@ -422,7 +429,8 @@ bool NNetwork::loadCheckpoint(const std::string& path)
         ok = fread(sizes.data(), 4, sizes.size(), f) == sizes.size() && fread(&tb, 4, 1, f) == 1 && tb < (1u << 20);
     }
     if (ok) { table.resize(tb); ok = fread(&table[0], 1, tb, f) == tb; }
-    std::vector<std::vector<float> > W, B, SA, SB;
+    std::vector<std::vector<float> > W, B, SA, SB, ED;
+    std::vector<std::vector<int32_t> > WC;
     for (int l = 0; ok && l < head[3]; ++l) {
         const size_t cnt = (size_t)sizes[l] * sizes[l + 1];
         std::vector<float> w(cnt), b, sa, sb;
@@ -431,7 +439,13 @@ bool NNetwork::loadCheckpoint(const std::string& path)
         ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { b.resize(n1); ok = fread(b.data(), 4, n1, f) == n1; }
         ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sa.resize(n1); ok = fread(sa.data(), 4, n1, f) == n1; }
         ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sb.resize(n1); ok = fread(sb.data(), 4, n1, f) == n1; }
-        W.push_back(w); B.push_back(b); SA.push_back(sa); SB.push_back(sb);
+        std::vector<int32_t> wc;
+        std::vector<float> ed;
+        if (version >= 2) {
+            ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { wc.resize(n1); ok = fread(wc.data(), 4, n1, f) == n1; }
+            ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { ed.resize(n1); ok = fread(ed.data(), 4, n1, f) == n1; }
+        }
+        W.push_back(w); B.push_back(b); SA.push_back(sa); SB.push_back(sb); WC.push_back(wc); ED.push_back(ed);
     }
     fclose(f);
     if (!ok) { lastError = "not a checkpoint of this library: " + path; return false; }
@@ -447,7 +461,7 @@ bool NNetwork::loadCheckpoint(const std::string& path)
     if (!loaded) { lastError = "checkpoint holds no valid network table"; return false; }
     clean();
     mode = head[0]; dtype = head[1]; epochs = head[2];
-    initW = W; initB = B; initStateA = SA; initStateB = SB;
+    initW = W; initB = B; initStateA = SA; initStateB = SB; initCounts = WC; initErrDer = ED;
     return true;
 }
 
@@ -497,6 +511,55 @@ std::vector<float> NNetwork::getBias(unsigned int layer)
 
 // LayerBuilder::build (ML/State/LayerBuilder.cpp:54-267): table to the device, weights sampled
 // in the reference's order (hidden layers, then the output layer, node by node) unless injected.
+bool NNetwork::hasDropout() const
+{
+    if (!skeleton) return false;
+    const int H = skeleton->numHiddenLayers();
+    for (int l = 0; l <= H; ++l) {
+        const float p = l == 0 ? skeleton->getPInput() : skeleton->getPDropout(l - 1);
+        const int rate = p * 100.0f;  // layer.cpp:107
+        if (rate >= 1 && rate < 100) return true;
+    }
+    return false;
+}
+
+// Layer::generateDropout (ML/State/layer.cpp:102-134) for every row in SGDHelper's order
+// (network.cpp:407-411): the row's input layer, then the hidden layers; one dart rand()%100+1 per
+// node, the layer drawn again while every node came out dropped; a rate outside 0..99 draws nothing.
+void NNetwork::drawDropout()
+{
+    const int H = skeleton->numHiddenLayers();
+    std::vector<int> sizes(H + 1);
+    sizes[0] = (int)nFeat;
+    size_t len = nFeat;
+    for (int h = 0; h < H; ++h) { sizes[h + 1] = skeleton->getHiddenLayerSize(h); len += sizes[h + 1]; }
+    if (dropFlags.size() != (size_t)nRows * len) dropFlags.assign((size_t)nRows * len, 0);
+    std::vector<unsigned char> hidden(len - nFeat, 0);  // the hidden layers are shared by all rows
+    if (nRows > 0) memcpy(hidden.data(), &dropFlags[(size_t)(nRows - 1) * len + nFeat], hidden.size());
+    for (unsigned int r = 0; r < nRows; ++r) {
+        unsigned char* m = &dropFlags[(size_t)r * len];
+        memcpy(m + nFeat, hidden.data(), hidden.size());
+        size_t off = 0;
+        for (int l = 0; l <= H; ++l) {
+            const int rate = pNode[l] * 100.0f;
+            if (rate >= 0 && rate < 100) {
+                bool all;
+                do {
+                    all = true;
+                    for (int i = 0; i < sizes[l]; ++i) {
+                        const int dart = (rand() % 100) + 1;
+                        const bool dropped = dart <= rate;
+                        if (!dropped) all = false;
+                        m[off + i] = dropped ? 1 : 0;
+                    }
+                } while (all);
+            }
+            off += sizes[l];
+        }
+        memcpy(hidden.data(), m + nFeat, hidden.size());
+    }
+}
+
 bool NNetwork::build()
 {
     std::vector<float> X, Y;
@@ -516,8 +579,15 @@ bool NNetwork::build()
         s.lr[l] = skeleton->getLearningRate(l); s.mom[l] = skeleton->getMomentumFactor(l);
         s.wd1[l] = skeleton->getWeightDecay1(l); s.wd2[l] = skeleton->getWeightDecay2(l);
         s.act[l] = skeleton->getActivationType(l); s.act_param[l] = skeleton->getActivationParam(l);
-        if (skeleton->getPDropout(l) != 0.0f) { lastError = "dropout is not supported on this path"; return false; }
     }
+    // network.cpp:407-411: the input layer takes getPInput(), hidden layer h takes getPDropout(h), whose
+    // index 0 is the input row again (nninfo.cpp:321-333): the last hidden row's rate is never used
+    pNode.assign(H + 1, 0.0f);
+    pNode[0] = skeleton->getPInput();
+    for (int h = 0; h < H; ++h) pNode[h + 1] = skeleton->getPDropout(h);
+    dropoutOn = hasDropout();
+    if (dropoutOn && mode != MODE_EXACT) { lastError = "dropout follows the reference's per-row algorithm: exact mode only"; return false; }
+    dropFlags.clear();
     s.batch = skeleton->getBatchSize();
     s.cost = skeleton->getOutputType();
     s.mode = mode == MODE_EXACT ? GHIP_MODE_EXACT : GHIP_MODE_CANONICAL;
@@ -541,6 +611,9 @@ bool NNetwork::build()
         if (ghip_net_set_params(dev, l, W.data(), bp, bl) != 0) { lastError = ghip_last_error(); return false; }
         if ((size_t)l < initStateA.size() && !initStateA[l].empty() && (size_t)l < initStateB.size() && !initStateB[l].empty())
             if (ghip_net_set_state(dev, l, initStateA[l].data(), initStateB[l].data()) != 0) { lastError = ghip_last_error(); return false; }
+        if ((size_t)l < initCounts.size() && initCounts[l].size() == (size_t)ni * no && (size_t)l < initErrDer.size() &&
+            initErrDer[l].size() == (size_t)no)
+            if (ghip_net_set_dropout_state(dev, l, initCounts[l].data(), initErrDer[l].data()) != 0) { lastError = ghip_last_error(); return false; }
     }
     if (ghip_net_set_dataset(dev, X.data(), Y.data(), (int64_t)nRows) != 0) { lastError = ghip_last_error(); return false; }
     // network.cpp:143-145: classification and KL runs keep a confusion matrix (counted on the device)
@@ -970,9 +1043,14 @@ void NNetwork::run(DataInput* newDataInput, int runType)
     running = true;
     while (running) {
         if (mode == MODE_EXACT) {
-            const int chunk = epochChunk(terminator, epochs, runType);
+            // with dropout one epoch per launch: the flags come from libc rand() as the epoch starts
+            const int chunk = dropoutOn ? 1 : epochChunk(terminator, epochs, runType);
             std::vector<ghip_metrics> ms(chunk);
             int ran = 0;
+            if (dropoutOn) {
+                drawDropout();
+                if (ghip_net_set_dropout_masks(dev, dropFlags.data(), 1) != 0) { lastError = ghip_last_error(); break; }
+            }
             if (ghip_net_run_epochs_exact(dev, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran,
                                           want_preds ? preds.data() : NULL) != 0) {
                 lastError = ghip_last_error();
@@ -1023,6 +1101,7 @@ bool MetaNetwork::runGroup(DataInput* d, int runType)
     for (size_t i = 0; i < subnets.size(); ++i) {
         NNetwork* n = subnets[i];
         if (!n || !n->skeleton || n->mode != NNetwork::MODE_EXACT) return false;
+        if (n->hasDropout()) return false;  // the subnets draw from one rand() stream, in subnet order
         NNetwork* a = subnets[0];
         if (n->epochs != a->epochs || n->biasMode != a->biasMode || n->skeleton->toTable() != a->skeleton->toTable()) return false;
         if (n->terminator.getEpoch() != a->terminator.getEpoch() || n->terminator.getAccuracy() != a->terminator.getAccuracy() ||
@@ -1090,7 +1169,9 @@ template <typename Fn>
 void for_each_subnet(MetaNetwork* m, Fn fn)
 {
     const std::vector<NNetwork*>& nets = m->getSubnets();
-    if (!m->getConcurrent() || nets.size() < 2) {
+    bool dropout = false;  // libc rand() is one stream: the reference's order is subnet after subnet
+    for (size_t i = 0; i < nets.size(); ++i) dropout = dropout || (nets[i] && nets[i]->hasDropout());
+    if (!m->getConcurrent() || nets.size() < 2 || dropout) {
         for (size_t i = 0; i < nets.size(); ++i)
             if (nets[i]) fn(nets[i]);
         return;

@@ -333,8 +333,17 @@ class NNetwork
     std::vector<std::vector<float> > initW;     // weights injected before the first run
     std::vector<std::vector<float> > initB;
     std::vector<std::vector<float> > initStateA, initStateB;  // optimiser state of a restored checkpoint
+    std::vector<std::vector<int32_t> > initCounts;            // dropout leftovers of a restored checkpoint:
+    std::vector<std::vector<float> > initErrDer;              // window lengths, node error accumulators
     unsigned int nRows, nFeat, nOut;
     std::string lastError;
+    // dropout (LayerBuilder::scrambleDropout, ML/State/LayerBuilder.cpp:497-523): probability per node
+    // layer (0 = input) as the reference resolves it, and the flags of the last epoch drawn, which the
+    // layers whose rate draws nothing keep (Layer::generateDropout returns early, layer.cpp:107-112)
+    std::vector<float> pNode;
+    std::vector<unsigned char> dropFlags;
+    bool dropoutOn;
+    void drawDropout();                              // one epoch's flags from libc rand()
 
     void run(DataInput*, int);
     bool prepare(DataInput*);                        // checks + build on first use
@@ -343,6 +352,7 @@ class NNetwork
     void clean();
 
 public:
+    bool hasDropout() const;  // some layer's rate int(p*100) lies in 1..99
     static const int TYPE_DFF = 0, TYPE_RNN = 1;
     static const int RUN_TRAIN = 0, RUN_TEST = 1, RUN_VALIDATE = 2;
     static const int MODE_EXACT = 0, MODE_CANONICAL = 1;      // extension

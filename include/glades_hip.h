@@ -90,7 +90,10 @@ typedef struct {
 } ghip_metrics;
 
 /* Selects the device and checks that it is a gfx950.  Stands in for glades::init()
- * (ML/main.cpp:51-56) as the once-per-process set-up call. */
+ * (ML/main.cpp:51-56) as the once-per-process set-up call.  It also makes the HIP runtime finish
+ * its own lazy set-up (first stream, first allocation), which draws from libc rand(): seed rand()
+ * AFTER this call and the stream the reference's weight sampler (ML/State/node.cpp:241-276) and
+ * dropout (ML/State/layer.cpp:102-134) read stays reproducible. */
 int ghip_init(int device_ordinal);
 
 /* Builds the device-side network: replaces LayerBuilder::build (ML/State/LayerBuilder.cpp:54-98)

@@ -249,6 +249,15 @@ static NNInfo* case_info(const Case& c)
     return new NNInfo("check", il, hidden, new OutputLayerInfo(c.sizes[c.nl], c.cost));
 }
 
+// the rows of the table carry the dropout rates: pd[0] on the input row, pd[k] on hidden row k-1
+static NNInfo* case_info_dropout(const Case& c, const std::vector<float>& pd)
+{
+    InputLayerInfo* il = new InputLayerInfo(c.batch, c.lr[0], c.mom[0], c.wd1[0], c.wd2[0], pd[0], c.act[0], c.par[0]);
+    std::vector<HiddenLayerInfo*> hidden;
+    for (int k = 1; k < c.nl; ++k) hidden.push_back(new HiddenLayerInfo(c.sizes[k], c.lr[k], c.mom[k], c.wd1[k], c.wd2[k], pd[k], c.act[k], c.par[k]));
+    return new NNInfo("check", il, hidden, new OutputLayerInfo(c.sizes[c.nl], c.cost));
+}
+
 static void seed_net(NNetwork& net, const Case& c, int mode)
 {
     net.setMode(mode);
@@ -256,6 +265,59 @@ static void seed_net(NNetwork& net, const Case& c, int mode)
         net.setWeights(l, c.W[l]);
         if (mode == NNetwork::MODE_EXACT) net.setBias(l, std::vector<float>(1, c.bias[l]));
     }
+}
+
+// Dropout through the class API: srand(seed); A trains E1 epochs and saves; B restores and trains on to
+// E1 + E2 (the rand() stream runs on); srand(seed) again; C trains E1 + E2 in one go; then C's test pass.
+// out: epochs of B and C, their losses, C's test-pass accuracy and rand() % 65536 after it, then
+// every layer's weights and bias of B, then of C.
+static int do_dropout(const char* in, int seed, int e1, int e2, const char* ckpt, const char* out, const std::vector<float>& pd)
+{
+    Case c;
+    int rc = read_case(in, c);
+    if (rc) return rc;
+    if ((int)pd.size() != c.nl) return 6;
+    glades::init();
+    DenseInput di(c.X.data(), c.Y.data(), c.N, c.sizes[0], c.sizes[c.nl]);
+    NNInfo* ia = case_info_dropout(c, pd);
+    NNInfo* ic = case_info_dropout(c, pd);
+    srand(seed);
+    {
+        NNetwork a(ia);
+        seed_net(a, c, NNetwork::MODE_EXACT);
+        a.setVerbose(false);
+        if (!a.hasDropout()) return 7;
+        a.terminator.setEpoch(e1);
+        a.train(&di);
+        if (a.getEpochs() != e1 || !a.saveCheckpoint(ckpt)) { fprintf(stderr, "save: %s\n", a.getLastError().c_str()); return 3; }
+    }
+    NNetwork b;
+    if (!b.loadCheckpoint(ckpt)) { fprintf(stderr, "load: %s\n", b.getLastError().c_str()); return 4; }
+    b.setVerbose(false);
+    b.terminator.setEpoch(e1 + e2);
+    b.train(&di);
+    if (!b.getLastError().empty()) { fprintf(stderr, "b: %s\n", b.getLastError().c_str()); return 5; }
+    srand(seed);
+    NNetwork cn(ic);
+    seed_net(cn, c, NNetwork::MODE_EXACT);
+    cn.setVerbose(false);
+    cn.terminator.setEpoch(e1 + e2);
+    cn.train(&di);
+    if (!cn.getLastError().empty()) { fprintf(stderr, "c: %s\n", cn.getLastError().c_str()); return 5; }
+    const float train_loss = cn.getLoss();
+    const int trained_c = cn.getEpochs();
+    std::vector<std::vector<float> > w, bb;
+    NNetwork* nets[2] = {&b, &cn};
+    for (int k = 0; k < 2; ++k)
+        for (int l = 0; l < c.nl; ++l) { w.push_back(nets[k]->getWeights(l)); bb.push_back(nets[k]->getBias(l)); }
+    cn.test(&di);  // draws flags as well (network.cpp:407-411)
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    float head[6] = {(float)b.getEpochs(), (float)trained_c, b.getLoss(), train_loss, cn.getAccuracy(), (float)(rand() % 65536)};
+    fwrite(head, 4, 6, fo);
+    for (size_t k = 0; k < w.size(); ++k) { fwrite(w[k].data(), 4, w[k].size(), fo); fwrite(bb[k].data(), 4, bb[k].size(), fo); }
+    fclose(fo);
+    return 0;
 }
 
 // A trains E1 epochs and saves; B restores and trains on to E1 + E2; C trains E1 + E2 in one go.
@@ -360,6 +422,11 @@ int main(int argc, char** argv)
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
     if (argc >= 7 && !strcmp(argv[1], "meta")) return do_meta(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 8 && !strcmp(argv[1], "checkpoint")) return do_checkpoint(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7]);
+    if (argc >= 9 && !strcmp(argv[1], "dropout")) {
+        std::vector<float> pd;
+        for (int k = 8; k < argc; ++k) pd.push_back((float)atof(argv[k]));
+        return do_dropout(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7], pd);
+    }
     if (argc >= 2 && !strcmp(argv[1], "ohe")) return do_ohe();
     if (argc >= 5 && !strcmp(argv[1], "numberinput")) return do_numberinput(argv[2], argv[3], argv[4]);
     if (argc >= 8 && !strcmp(argv[1], "traincsv")) return do_traincsv(argv[2], argv[3], atol(argv[4]), (float)atof(argv[5]), atoi(argv[6]), argv[7], argc >= 9 ? argv[8] : NULL);

@@ -366,3 +366,50 @@ def test_meta_network_subnets_run_concurrently_with_equal_results():
     np.testing.assert_allclose(losses[0], m.loss, rtol=1e-4)
     m, _ = o.epoch(c["X"], c["Y"], train=False, want_preds=False)
     np.testing.assert_allclose(raw[3], m.accuracy, rtol=1e-4)             # cross-validation accuracy = mean test accuracy
+
+
+@needs_bin
+@pytest.mark.gpu
+def test_dropout_through_the_class_api_follows_the_rand_stream():
+    """NNInfo rows with dropout rates -> NNetwork::train: the class draws the flags from libc rand()
+    in the reference's order (input row's rate for the input layer AND the first hidden layer, hidden
+    row k for hidden layer k+1, the last hidden row unused: nninfo.cpp:321-333), one epoch per launch.
+    Checked against the CPU restatement fed from the same srand(seed) stream; a checkpoint taken in the
+    middle continues bit for bit; the test pass draws flags too."""
+    c = load_case("batch1_5_7_6_4", "dropout")
+    seed, e1, e2 = 11, 2, 3
+    rows = [0.2, 0.3, 0.9]                      # input row, hidden row 0, hidden row 1 (never used)
+    resolved = np.array([0.2, 0.2, 0.3], np.float32)   # node layers 0, 1, 2
+    with tempfile.TemporaryDirectory() as td:
+        cin, ck, cout = os.path.join(td, "c.bin"), os.path.join(td, "n.ckpt"), os.path.join(td, "o.bin")
+        write_case(cin, c)
+        subprocess.check_call([BIN, "dropout", cin, str(seed), str(e1), str(e2), ck, cout] + [str(p) for p in rows],
+                              stdout=subprocess.DEVNULL)
+        raw = np.fromfile(cout, np.float32)
+    assert raw[0] == e1 + e2 and raw[1] == e1 + e2
+    assert bits_equal(raw[2:3], raw[3:4])       # restored and straight run end on the same loss
+    body = raw[6:]
+    half = body.size // 2
+    assert bits_equal(body[:half], body[half:])
+    o = po.ExactNet(c["spec"])
+    for l in range(c["nl"]):
+        o.set_weights(l, c["W0"][l])
+        o.set_bias(l, c["bias0"][l])
+    po.libc_srand(seed)
+    dropped = 0
+    for _ in range(e1 + e2):
+        masks = po.dropout_draw(c["spec"], resolved, c["N"])
+        dropped += int(masks.sum())
+        m, _ = o.epoch(c["X"], c["Y"], masks=masks)
+    assert dropped > 0
+    mt, _ = o.epoch(c["X"], c["Y"], train=False, masks=po.dropout_draw(c["spec"], resolved, c["N"]))
+    assert int(raw[5]) == po.libc_rand() % 65536   # both sides consumed the same number of draws
+    np.testing.assert_allclose(raw[3], m.loss, rtol=1e-4)
+    np.testing.assert_allclose(raw[4], mt.accuracy, rtol=1e-4)
+    pos = half
+    for l in range(c["nl"]):
+        n = c["sizes"][l] * c["sizes"][l + 1]
+        W = body[pos:pos + n].reshape(c["sizes"][l + 1], c["sizes"][l])
+        pos += n + 1
+        scale = np.abs(o.get_weights(l)).max()
+        np.testing.assert_allclose(W, o.get_weights(l), rtol=1e-3, atol=1e-4 * scale)
