@@ -57,6 +57,12 @@ def build_all(verbose=False):
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I", os.path.join(HERE, "..", "include"),
               "-pthread", "-o", HOST_LIB] + host_srcs + ["-L", HERE, "-lglades_hip", "-Wl,-rpath,$ORIGIN"])
         # driver of the C++ class API used by tests/test_host_api.py (built here, run on the GPU box)
+        # CPU checker of the restated float routines against this machine's C library (tests/test_libm_exact.py)
+        libm_src = os.path.join(HERE, "..", "tests", "libm_check.cpp")
+        if os.path.exists(libm_src):
+            os.makedirs(os.path.join(HERE, "..", "tests", "bin"), exist_ok=True)
+            _run(["g++", "-O2", "-std=c++17", "-ffp-contract=off", "-fopenmp", "-o",
+                  os.path.join(HERE, "..", "tests", "bin", "libm_check"), libm_src, "-lm"])
         check_src = os.path.join(HERE, "..", "tests", "host_api_check.cpp")
         if os.path.exists(check_src):
             bindir = os.path.join(HERE, "..", "tests", "bin")

@@ -236,6 +236,7 @@ int setup_exact(ghip_net* n)
     e.state_floats = woff;
     e.node_floats = aoff;
     e.mb = s.batch; e.cost = s.cost; e.bias_mode = s.bias_mode;
+    e.metric_cap = s.sizes[s.n_layers] > 128 ? s.sizes[s.n_layers] : 128;  // 1 KB: keeps two cfg2-sized networks per CU
     int T = pow2ceil((max_edges + 7) / 8);
     if (T < pow2ceil(max_nodes)) T = pow2ceil(max_nodes);
     if (T < 64) T = 64;
@@ -591,6 +592,29 @@ int ghip_init(int device_ordinal)
         HIP_TRY(hipStreamDestroy(s));
     }
     g_device = device_ordinal;
+    return 0;
+}
+
+int ghip_gmath_eval(int fn, int kind, float param, const float* host_a, const float* host_b, float* host_out, int64_t n)
+{
+    if (fn < 0 || fn > 3 || !host_a || !host_out || n < 0 || (fn >= 2 && !host_b)) return fail(GHIP_EINVAL, "bad arguments");
+    if (fn <= 1 && (kind < GHIP_TANH || kind > GHIP_STEP)) return fail(GHIP_EINVAL, "unknown activation %d", kind);
+    if (fn >= 2 && (kind < GHIP_REGRESSION || kind > GHIP_KL)) return fail(GHIP_EINVAL, "unknown cost %d", kind);
+    if (n == 0) return 0;
+    if (g_device < 0) TRY(ghip_init(0));
+    HIP_TRY(hipSetDevice(g_device));
+    float *a = nullptr, *b = nullptr, *o = nullptr;
+    int rc = dalloc(&a, (size_t)n);
+    if (rc == 0) rc = dalloc(&o, (size_t)n);
+    if (rc == 0 && fn >= 2) rc = dalloc(&b, (size_t)n);
+    hipError_t e = hipSuccess;
+    if (rc == 0) e = hipMemcpy(a, host_a, (size_t)n * 4, hipMemcpyHostToDevice);
+    if (rc == 0 && e == hipSuccess && b) e = hipMemcpy(b, host_b, (size_t)n * 4, hipMemcpyHostToDevice);
+    if (rc == 0 && e == hipSuccess) e = ghip_launch_gmath_eval(fn, kind, param, a, b, o, n, 0);
+    if (rc == 0 && e == hipSuccess) e = hipMemcpy(host_out, o, (size_t)n * 4, hipMemcpyDeviceToHost);
+    dfree(a); dfree(b); dfree(o);
+    if (rc != 0) return rc;
+    if (e != hipSuccess) return fail(GHIP_EHIP, "gmath_eval: %s", hipGetErrorString(e));
     return 0;
 }
 

@@ -96,7 +96,13 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     int* sflag = (int*)(sbias + GHIP_MAX_LAYERS);
     // dropout only: the row's flags (1 = dropped; output layer always 0) and the nodes' error
     // accumulators (Node::errorDer), which outlive the row
-    int* sm = sflag + 4;
+    // (predicted, expected) pairs of the rows since the last flush; their cost and accuracy terms
+    // are computed a ring-full at a time, one lane each, and summed in visiting order afterwards
+    const int cap = p.metric_cap;
+    float* rp = (float*)(sflag + 4);
+    float* re = rp + cap;
+    int fill = 0;
+    int* sm = (int*)(re + cap);
     float* sE = (float*)(sm + p.node_floats);
     const int mask_len = p.aoff[L];  // flags of one row: the non-output layers side by side
 
@@ -195,28 +201,50 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
                     }
                     if (l != 0) z = __fadd_rn(z, bl);
-                    aout[o] = ghip_squash<true>(z, act, par);
+                    const float a = ghip_squash<true>(z, act, par);
+                    aout[o] = a;
+                    if (l == L - 1) {
+                        rp[fill + o] = a;
+                        re[fill + o] = sy[o];
+                    }
                 }
                 __syncthreads();
             }
+            fill += nout;
             const float* pred = sa + p.aoff[L];
             if (own.preds && last_epoch)
                 for (int o = tid; o < nout; o += T) own.preds[r * nout + o] = pred[o];
 
-            // ---- output metrics in visiting order (network.cpp:519-559)
+            // ---- output metrics (network.cpp:519-559): the class of the row now, ...
             if (tid == serial) {
                 float mp = 0.0f, my = 0.0f;
                 int ip = -1, iy = -1;
                 for (int o = 0; o < nout; ++o) {
                     const float pr = pred[o], ex = sy[o];
-                    tot_err = __fadd_rn(tot_err, ghip_cost<false>(ex, pr, data_size, p.cost));
-                    tot_acc = __fadd_rn(tot_acc, ghip_accuracy_term(pr, ex));
                     if (pr > mp) { mp = pr; ip = o; }
                     if (ex > my) { my = ex; iy = o; }
                 }
                 if (ip == iy) ++correct;
                 // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
                 if (own.cm && ip >= 0 && iy >= 0) atomicAdd(&own.cm[iy * nout + ip], 1);
+            }
+            // ... cost and accuracy once the ring is full: the terms in parallel (the logarithms of
+            // the cost are the expensive part), the two running sums in visiting order by one lane.
+            // The ring is written again only after the barriers that follow, so that lane is done.
+            if (fill + nout > cap || r == p.n_rows - 1) {
+                for (int k = tid; k < fill; k += T) {
+                    const float pr = rp[k], ex = re[k];
+                    rp[k] = ghip_cost<true>(ex, pr, data_size, p.cost);
+                    re[k] = ghip_accuracy_term(pr, ex);
+                }
+                __syncthreads();
+                if (tid == serial) {
+                    for (int k = 0; k < fill; ++k) {
+                        tot_err = __fadd_rn(tot_err, rp[k]);
+                        tot_acc = __fadd_rn(tot_acc, re[k]);
+                    }
+                }
+                fill = 0;
             }
 
             if (p.train) {
@@ -389,11 +417,37 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
         for (int k = tid; k < p.node_floats; k += T) own.errder[k] = sE[k];
 }
 
+// GMath::squash / activationErrDer / outputNodeCost / costErrDer over arrays, with exact mode's arithmetic
+__global__ void gmath_eval_kernel(int fn, int kind, float param, const float* __restrict__ a, const float* __restrict__ b,
+                                  float* __restrict__ out, long long n)
+{
+    for (long long k = (long long)blockIdx.x * blockDim.x + threadIdx.x; k < n; k += (long long)gridDim.x * blockDim.x) {
+        float v = 0.0f;
+        switch (fn) {
+        case 0: v = ghip_squash<true>(a[k], kind, param); break;
+        case 1: v = ghip_act_der_ref(a[k], kind, param); break;
+        case 2: v = ghip_cost<true>(a[k], b[k], param, kind); break;
+        case 3: v = ghip_cost_der(a[k], b[k], kind); break;
+        }
+        out[k] = v;
+    }
+}
+
 }  // namespace
+
+hipError_t ghip_launch_gmath_eval(int fn, int kind, float param, const float* a, const float* b, float* out, long long n,
+                                  hipStream_t s)
+{
+    long long blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(gmath_eval_kernel, dim3((unsigned)blocks), dim3(256), 0, s, fn, kind, param, a, b, out, n);
+    return hipGetLastError();
+}
 
 size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropout)
 {
-    size_t f = (size_t)3 * p.node_floats + p.sizes[p.n_layers] + GHIP_MAX_LAYERS + 4;
+    size_t f = (size_t)3 * p.node_floats + p.sizes[p.n_layers] + GHIP_MAX_LAYERS + 4 + (size_t)2 * p.metric_cap;
     if (dropout) f += (size_t)2 * p.node_floats;
     if (state_in_lds) f += (size_t)3 * p.state_floats;
     return f * sizeof(float);

@@ -5,31 +5,32 @@
 #include <stdint.h>
 
 #include "../../include/glades_hip.h"
+#include "libm_exact.h"
 
 #define GHIP_OUTLIER 0.046f  // knee of RELU / LEAKY in the reference (gmath.h:35, gmath.cpp:62-82)
 
 // ---------------------------------------------------------------- element-wise device functions
 
-// Reference GMath::squash (gmath.cpp:22-101).  kPrecise selects transcendental evaluation in
-// double rounded once to float, which tracks glibc's float routines to the last bit far more
-// often than the fast fp32 device routines do (exact mode is sequential and order-faithful,
-// so the transcendental is the only remaining source of divergence from the CPU path).
+// Reference GMath::squash (gmath.cpp:22-101).  kPrecise selects the routines that return, for every
+// input, the float the reference's C library returns (libm_exact.h): exact mode is sequential and
+// order-faithful, so with them nothing is left that could differ from the CPU path.  The fast fp32
+// device routines serve the batched kernels.
 template <bool kPrecise>
 __device__ __forceinline__ float ghip_tanh(float z)
 {
-    if (kPrecise) return (float)tanh((double)z);
+    if (kPrecise) return glm_tanhf(z);
     return tanhf(z);
 }
 template <bool kPrecise>
 __device__ __forceinline__ float ghip_exp(float z)
 {
-    if (kPrecise) return (float)exp((double)z);
+    if (kPrecise) return glm_expf(z);
     return expf(z);
 }
 template <bool kPrecise>
 __device__ __forceinline__ float ghip_log(float z)
 {
-    if (kPrecise) return (float)log((double)z);
+    if (kPrecise) return glm_logf(z);
     return logf(z);
 }
 
@@ -237,6 +238,7 @@ struct ExactLaunch {
     const float* Y;
     ExactPointers ptr;  // this network's own arrays (a launch over several networks passes a list instead)
     int    state_in_lds;
+    int    metric_cap;  // outputs held back before their cost / accuracy terms are computed (>= sizes[n_layers])
     int    dropout;     // run the instantiation that reads flags and keeps accumulators / window lengths
 };
 
@@ -244,6 +246,10 @@ struct ExactLaunch {
 hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads, size_t lds_bytes,
                              hipStream_t s);
 size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropout);
+// fn 0 squash(a; kind, param), 1 activationErrDer(a; kind, param), 2 outputNodeCost(expected a, predicted b; cost
+// kind, dataSize param), 3 costErrDer(expected a, predicted b; cost kind): device arrays of n floats
+hipError_t ghip_launch_gmath_eval(int fn, int kind, float param, const float* a, const float* b, float* out, long long n,
+                                  hipStream_t s);
 
 // ---------------------------------------------------------------- canonical kernels
 

@@ -19,7 +19,7 @@ F32, BF16, FP8_INFER = 0, 1, 2
 BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
 
 EXPORTS = [
-    "ghip_init", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
+    "ghip_init", "ghip_gmath_eval", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
     "ghip_net_get_state", "ghip_net_set_state",
     "ghip_net_set_dropout_masks", "ghip_net_get_dropout_state", "ghip_net_set_dropout_state",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
@@ -74,6 +74,7 @@ def load():
         vp, i, f, i64 = C.c_void_p, C.c_int, C.c_float, C.c_int64
         sig = {
             "ghip_init": (i, [i]),
+            "ghip_gmath_eval": (i, [i, i, f, vp, vp, vp, i64]),
             "ghip_net_create": (i, [C.POINTER(Spec), C.POINTER(vp)]),
             "ghip_net_destroy": (i, [vp]),
             "ghip_net_set_params": (i, [vp, i, vp, vp, i]),
@@ -141,6 +142,16 @@ def make_spec(sizes, acts, lr=0.01, mom=0.0, wd1=0.0, wd2=0.0, act_params=0.0, b
 
 def _ptr(a):
     return None if a is None else C.c_void_p(a.ctypes.data)
+
+
+def gmath_eval(fn, kind, a, b=None, param=0.0):
+    """fn 0 squash, 1 activationErrDer, 2 outputNodeCost(expected a, predicted b, dataSize param),
+    3 costErrDer(expected a, predicted b), element by element on the device with exact mode's arithmetic."""
+    a = np.ascontiguousarray(a, np.float32)
+    b = None if b is None else np.ascontiguousarray(b, np.float32)
+    out = np.empty_like(a)
+    _check(load().ghip_gmath_eval(int(fn), int(kind), float(param), _ptr(a), _ptr(b), _ptr(out), a.size))
+    return out
 
 
 class Net:

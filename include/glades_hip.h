@@ -96,6 +96,16 @@ typedef struct {
  * dropout (ML/State/layer.cpp:102-134) read stays reproducible. */
 int ghip_init(int device_ordinal);
 
+/* The element-wise functions of the path over arrays, with exact mode's arithmetic (what one row of
+ * the persistent kernel applies to one node), for callers and tests that want them on their own:
+ * fn 0  GMath::squash(a[k], kind, param)                       ML/GMath/gmath.cpp:22-101
+ * fn 1  GMath::activationErrDer(a[k], kind, param)             ML/GMath/gmath.cpp:182-245
+ * fn 2  GMath::outputNodeCost(expected a[k], predicted b[k], dataSize = param, cost kind)  :272-321
+ * fn 3  GMath::costErrDer(expected a[k], predicted b[k], cost kind)                        :323-353
+ * kind is an activation id for fn 0/1 and a cost id for fn 2/3; host_b is unused for fn 0/1.  tanh, exp
+ * and log return the floats of the reference platform's C library (GNU libc 2.35), bit for bit. */
+int ghip_gmath_eval(int fn, int kind, float param, const float* host_a, const float* host_b, float* host_out, int64_t n);
+
 /* Builds the device-side network: replaces LayerBuilder::build (ML/State/LayerBuilder.cpp:54-98)
  * minus the weight sampling, which stays with the caller (ghip_net_set_params). */
 int ghip_net_create(const ghip_net_spec* spec, ghip_net** out);

@@ -245,6 +245,21 @@ void go_ref_xavier_layer(int fan_in, int n_out, int act_type, float* W)
         }
 }
 
+/* the element-wise functions over arrays: fn 0 squash, 1 act_der, 2 cost(expected a, predicted b,
+   data_size param), 3 cost_der(expected a, predicted b) */
+void go_eval(int fn, int kind, float param, const float* a, const float* b, float* out, int64_t n)
+{
+#pragma omp parallel for schedule(static)
+    for (int64_t k = 0; k < n; ++k) {
+        switch (fn) {
+        case 0: out[k] = go_squash(a[k], kind, param); break;
+        case 1: out[k] = go_act_der(a[k], kind, param); break;
+        case 2: out[k] = go_cost(a[k], b[k], param, kind); break;
+        default: out[k] = go_cost_der(a[k], b[k], kind); break;
+        }
+    }
+}
+
 /* ------------------------------------------------------------------ exact mode */
 
 struct go_exact {

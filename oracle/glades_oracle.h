@@ -94,6 +94,9 @@ float go_act_der(float a, int act, float param);
 float go_cost(float expect, float pred, float data_size, int cost);
 float go_cost_der(float expect, float pred, int cost);
 float go_percent_error(float pred, float expect);
+/* the four functions above over arrays: fn 0 squash(a), 1 act_der(a), 2 cost(expect a, pred b, data_size
+   param), 3 cost_der(expect a, pred b); kind = activation or cost id */
+void  go_eval(int fn, int kind, float param, const float* a, const float* b, float* out, int64_t n);
 int   go_argmax_ref(const float* v, int n);  /* -1 when no element is > 0 */
 
 /* confusion matrix, ML/GMath/cmatrix.cpp: M is n x n int32 row-major (row expected, column predicted) */

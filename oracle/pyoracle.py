@@ -65,6 +65,7 @@ def lib():
             "go_cost_der": (C.c_float, [C.c_float, C.c_float, C.c_int]),
             "go_percent_error": (C.c_float, [C.c_float, C.c_float]),
             "go_argmax_ref": (C.c_int, [f32p, C.c_int]),
+            "go_eval": (None, [C.c_int, C.c_int, C.c_float, f32p, vp, f32p, C.c_int64]),
             "go_cmatrix_add": (None, [C.c_int, i32p, f32p, f32p]),
             "go_cmatrix_params": (None, [C.c_int, i32p, i32p, i32p, i32p, i32p]),
             "go_cmatrix_overall": (None, [C.c_int, i32p, i32p, i32p, i32p, f32p]),
@@ -290,6 +291,15 @@ def fp8_forward(spec, Wq, wscale, X):
 
 def have_ref():
     return os.path.exists(REF_HARNESS)
+
+
+def gmath_eval(fn, kind, a, b=None, param=0.0):
+    """fn 0 squash, 1 act_der, 2 cost(expected a, predicted b, data_size param), 3 cost_der, per element."""
+    a = np.ascontiguousarray(a, np.float32)
+    b = None if b is None else np.ascontiguousarray(b, np.float32)
+    out = np.empty_like(a)
+    lib().go_eval(int(fn), int(kind), float(param), a, _vp(b), out, a.size)
+    return out
 
 
 def libc_srand(seed):
