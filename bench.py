@@ -144,7 +144,7 @@ def run_canonical(w, args):
     gemm_names = {
         "bf16": {"gemm_bf16_forward": "fwd_hidden", "gemm_bf16_forward_out": "fwd_out", "gemm_bf16_dgrad": "dgrad", "gemm_bf16_wgrad_sgd": "wgrad"},
         "fp8": {"gemm_fp8_forward": "fwd_hidden", "gemm_fp8_forward_out": "fwd_out"},
-        "f32": {"gemm_f32_forward": "fwd_all", "gemm_f32_dgrad": "dgrad", "gemm_f32_wgrad": "wgrad"},
+        "f32": {"gemm_f32_forward": "fwd_all", "gemm_f32_dgrad": "dgrad", "gemm_f32_wgrad_sgd": "wgrad"},
     }[w["dtype"]]
     wl = [sizes[l] * sizes[l + 1] for l in range(nl)]
     per_step = {"fwd_hidden": 2 * B * sum(wl[:-1]), "fwd_out": 2 * B * wl[-1], "fwd_all": 2 * B * sum(wl),

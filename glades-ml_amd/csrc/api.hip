@@ -84,13 +84,15 @@ struct ghip_net {
     float* b[GHIP_MAX_LAYERS] = {};
     float* vW[GHIP_MAX_LAYERS] = {};
     float* vb[GHIP_MAX_LAYERS] = {};
-    float* gW[GHIP_MAX_LAYERS] = {};
     float* act[GHIP_MAX_LAYERS + 1] = {};
     float* dlt[GHIP_MAX_LAYERS + 1] = {};
     float* stageX = nullptr;
-    float* bpart = nullptr;   // fp32 path: bias-gradient partial sums [16][widest layer]
     int cap_batch = 0;
+    // metrics of a batch: three banks of 4 doubles.  A metrics launch adds into bank accBank^1 and
+    // clears the bank the launch after it will use, so no separate clearing launch is needed; bank 2
+    // takes the sums of launches whose metrics nobody reads.
     double* dAcc = nullptr;
+    int accBank = 0;
     int last_batch = 0;
     // bf16
     uint16_t* Wh[GHIP_MAX_LAYERS] = {};
@@ -291,7 +293,6 @@ int setup_canon(ghip_net* n)
             HIP_TRY(hipMemsetAsync(n->vW[l], 0, cnt * 4, n->stream));
             HIP_TRY(hipMemsetAsync(n->vb[l], 0, (size_t)s.sizes[l + 1] * 4, n->stream));
         }
-        if (s.dtype == GHIP_F32) TRY(dalloc(&n->gW[l], cnt));
         if (s.dtype == GHIP_BF16) {
             TRY(dalloc(&n->Wh[l], cnt));
             TRY(dalloc(&n->WhT[l], cnt));
@@ -301,8 +302,8 @@ int setup_canon(ghip_net* n)
             TRY(dalloc(&n->wscale[l], (size_t)s.sizes[l + 1]));
         }
     }
-    TRY(dalloc(&n->dAcc, 4));
-    HIP_TRY(hipMemsetAsync(n->dAcc, 0, 4 * sizeof(double), n->stream));
+    TRY(dalloc(&n->dAcc, 12));
+    HIP_TRY(hipMemsetAsync(n->dAcc, 0, 12 * sizeof(double), n->stream));
     return 0;
 }
 
@@ -313,7 +314,7 @@ void free_batch_buffers(ghip_net* n)
         if (l > 0) dfree(n->H[l]);
         dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]); dfree(n->csum[l]);
     }
-    dfree(n->stageX); dfree(n->logits); dfree(n->bpart);
+    dfree(n->stageX); dfree(n->logits);
     dfree(n->Aq[0]); dfree(n->Aq[1]); dfree(n->ascale[0]); dfree(n->ascale[1]);
     dfree(n->amax_bits); dfree(n->Hq); dfree(n->out8);
     n->cap_batch = 0;
@@ -330,7 +331,6 @@ int reserve_batch(ghip_net* n, int B)
     for (int l = 0; l <= L; ++l) if (s.sizes[l] > maxw) maxw = s.sizes[l];
     if (s.dtype == GHIP_F32) {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
-        TRY(dalloc(&n->bpart, (size_t)16 * maxw));
         for (int l = 1; l <= L; ++l) {
             TRY(dalloc(&n->act[l], (size_t)B * s.sizes[l]));
             TRY(dalloc(&n->dlt[l], (size_t)B * s.sizes[l]));
@@ -405,14 +405,16 @@ int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
 {
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
-    LAUNCH(n, "fill_metrics", ghip_fill_f64(n->dAcc, 4, 0.0, n->stream));
+    const int bank = n->accBank ^ 1;
     DeltaArgs a;
     memset(&a, 0, sizeof(a));
     a.P = P; a.Y = Y; a.D = D; a.Dbf = Dbf; a.DbfT = nullptr;
     a.B = B; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
-    a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost; a.acc = n->dAcc;
+    a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost;
+    a.acc = n->dAcc + 4 * bank; a.acc_clear = n->dAcc + 4 * (bank ^ 1);
     a.cm = n->cm;
     LAUNCH(n, "output_delta", ghip_output_delta(a, n->stream));
+    n->accBank = bank;
     return 0;
 }
 
@@ -428,13 +430,6 @@ int step_f32(ghip_net* n, int64_t row0, int B)
         const int ni = s.sizes[l], no = s.sizes[l + 1];
         const float* Ain = (l == 0) ? X : n->act[l];
         GemmF32Args g;
-        memset(&g, 0, sizeof(g));
-        // gradient: G[no][ni] = D^T A / B
-        g.A = n->dlt[l + 1]; g.lda = no; g.a_kmajor = 1;
-        g.B = Ain; g.ldb = ni; g.b_kmajor = 1;
-        g.C = n->gW[l]; g.ldc = ni; g.M = no; g.N = ni; g.K = B;
-        g.epilogue = EPI_STORE; g.alpha = 1.0f / (float)B;
-        LAUNCH(n, "gemm_f32_wgrad", ghip_gemm_f32(g, n->stream));
         if (l > 0) {  // back-prop with the pre-update weights: E = D W, times f'(a_l)
             memset(&g, 0, sizeof(g));
             g.A = n->dlt[l + 1]; g.lda = no; g.a_kmajor = 0;
@@ -444,13 +439,16 @@ int step_f32(ghip_net* n, int64_t row0, int B)
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1]; g.alpha = 1.0f;
             LAUNCH(n, "gemm_f32_dgrad", ghip_gemm_f32(g, n->stream));
         }
-        {   // bias gradient = column sums of the delta, over row chunks that are then added in order
-            const int chunks = B >= 1024 ? 16 : (B >= 128 ? 8 : 1);
-            LAUNCH(n, "bias_colsum", ghip_colsum_f32(n->dlt[l + 1], B, no, no, chunks, n->bpart, n->stream));
-            LAUNCH(n, "bias_update", ghip_bias_update_partials(n->bpart, chunks, no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
-        }
-        LAUNCH(n, "sgd_update_f32", ghip_sgd_update_f32(n->W[l], n->vW[l], n->gW[l], (long long)ni * no, s.lr[l], s.mom[l],
-                                                       s.wd1[l], s.wd2[l], 1.0f, n->stream));
+        // gradient D^T A / B and, in the same kernel's epilogue, the update of the weights (momentum,
+        // both decays) and of the bias (batch mean of the delta = the row sums of the A operand)
+        memset(&g, 0, sizeof(g));
+        g.A = n->dlt[l + 1]; g.lda = no; g.a_kmajor = 1;
+        g.B = Ain; g.ldb = ni; g.b_kmajor = 1;
+        g.C = n->W[l]; g.ldc = ni; g.M = no; g.N = ni; g.K = B;
+        g.epilogue = EPI_SGD; g.alpha = 1.0f / (float)B;
+        g.V = n->vW[l]; g.lr = s.lr[l]; g.mom = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l];
+        g.bias_w = n->b[l]; g.bias_v = n->vb[l];
+        LAUNCH(n, "gemm_f32_wgrad_sgd", ghip_gemm_f32(g, n->stream));
     }
     return 0;
 }
@@ -547,7 +545,7 @@ int forward_fp8(ghip_net* n, const uint16_t* Xbf, int B, float* dev_out)
 int fetch_metrics(ghip_net* n, ghip_metrics* m)
 {
     double acc[4];
-    HIP_TRY(hipMemcpyAsync(acc, n->dAcc, sizeof(acc), hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipMemcpyAsync(acc, n->dAcc + 4 * n->accBank, sizeof(acc), hipMemcpyDeviceToHost, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
     const int B = n->last_batch > 0 ? n->last_batch : 1;
     m->loss = (float)(acc[0] / (double)B);
@@ -647,7 +645,7 @@ int ghip_net_destroy(ghip_net* n)
     dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass); dfree(n->exMulti);
     dfree(n->exMasks); dfree(n->exCnt); dfree(n->exErr);
     for (int l = 0; l < GHIP_MAX_LAYERS; ++l) {
-        dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]); dfree(n->gW[l]);
+        dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]);
         dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
     }
     dfree(n->dAcc);
@@ -1060,7 +1058,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
             DeltaArgs a;
             memset(&a, 0, sizeof(a));
             a.P = n->act[L]; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
-            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc; a.store_p = 1;
+            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc + 8; a.store_p = 1;
             LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
         }
         *result = n->act[L];
@@ -1071,7 +1069,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
             DeltaArgs a;
             memset(&a, 0, sizeof(a));
             a.P = n->logits; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
-            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc; a.store_p = 1;
+            a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc + 8; a.store_p = 1;
             LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
         }
         *result = n->logits;

@@ -31,11 +31,12 @@ __device__ __forceinline__ double wave_sum_d(double v)
 // up to 64*kRegs outputs is read from memory once and kept in registers (lane j-th value =
 // column j*64 + lane): one exp per element, and the softmax passes cost no extra HBM traffic.
 constexpr int kRowsPerWave = 2;
-constexpr int kRegs = 16;
 
-template <bool kInRegs>
+template <int kRegs>  // row held in kRegs registers per lane (n <= 64 * kRegs); 0: read from memory on every pass
 __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
 {
+    constexpr bool kInRegs = kRegs > 0;
+    if (blockIdx.x == 0 && threadIdx.x < 4 && a.acc_clear) a.acc_clear[threadIdx.x] = 0.0;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int row0 = (blockIdx.x * 4 + w) * kRowsPerWave;
     double loss = 0.0, accs = 0.0, corr = 0.0;
@@ -46,7 +47,7 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
         if (b >= a.B) break;
         float* p = a.P + (long long)b * a.ldp;
         const float* y = a.Y ? a.Y + (long long)b * a.ldy : nullptr;
-        float reg[kRegs];
+        float reg[kRegs > 0 ? kRegs : 1];
         float inv = 1.0f, mx = 0.0f;
         if (kInRegs) {
 #pragma unroll
@@ -137,6 +138,7 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
 template <int Q>
 __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
 {
+    if (blockIdx.x == 0 && threadIdx.x < 4 && a.acc_clear) a.acc_clear[threadIdx.x] = 0.0;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     double loss = 0.0, accs = 0.0, corr = 0.0;
     const bool softmax = a.act == GHIP_SOFTMAX;
@@ -229,62 +231,6 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
         double v = red[0][threadIdx.x] + red[1][threadIdx.x] + red[2][threadIdx.x] + red[3][threadIdx.x];
         atomicAdd(&a.acc[threadIdx.x], v);
     }
-}
-
-__global__ void __launch_bounds__(256)
-sgd_update_f32_kernel(float* __restrict__ W, float* __restrict__ V, const float* __restrict__ G,
-                      long long n, float lr, float mom, float wd1, float wd2, float gscale)
-{
-    long long i = (long long)blockIdx.x * 256 + threadIdx.x;
-    const long long stride = (long long)gridDim.x * 256;
-    for (; i < n; i += stride) {
-        const float w = W[i];
-        const float sg = (w > 0.0f) ? 1.0f : ((w < 0.0f) ? -1.0f : 0.0f);
-        const float g = G[i] * gscale + wd1 * sg + wd2 * w;
-        const float d = lr * g + mom * V[i];
-        V[i] = d;
-        W[i] = w - d;
-    }
-}
-
-// one workgroup per 64 output channels; lanes walk channels (coalesced), wavefronts split rows
-__global__ void __launch_bounds__(256)
-bias_update_f32_kernel(const float* __restrict__ D, int B, int n, int ldd, float* __restrict__ bias,
-                       float* __restrict__ vb, float lr, float mom)
-{
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int o = blockIdx.x * 64 + lane;
-    float s = 0.0f;
-    if (o < n)
-        for (int b = w; b < B; b += 4) s += D[(long long)b * ldd + o];
-    __shared__ float red[4][64];
-    red[w][lane] = s;
-    __syncthreads();
-    if (w == 0 && o < n) {
-        const float g = (red[0][lane] + red[1][lane] + red[2][lane] + red[3][lane]) / (float)B;
-        const float d = lr * g + mom * vb[o];
-        vb[o] = d;
-        bias[o] = bias[o] - d;
-    }
-}
-
-// column sums of a slice of rows: partial[blockIdx.y][o] = sum over rows [y*rpc, (y+1)*rpc) of D[b][o]
-// (the bias gradient of the fp32 path, split over row chunks so that small batches still fill the
-// device; the chunks are added in order by bias_update_partials_kernel)
-__global__ void __launch_bounds__(256)
-colsum_f32_kernel(const float* __restrict__ D, int B, int n, int ldd, int rows_per_chunk, float* __restrict__ partial)
-{
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-    const int o = blockIdx.x * 64 + lane;
-    const int b0 = blockIdx.y * rows_per_chunk;
-    const int b1 = (b0 + rows_per_chunk) < B ? (b0 + rows_per_chunk) : B;
-    float s = 0.0f;
-    if (o < n)
-        for (int b = b0 + w; b < b1; b += 4) s += D[(long long)b * ldd + o];
-    __shared__ float red[4][64];
-    red[w][lane] = s;
-    __syncthreads();
-    if (w == 0 && o < n) partial[(long long)blockIdx.y * n + o] = (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
 // bf16 delta^T [n][B]: one wavefront per channel, 16-byte loads (B is a multiple of 8)
@@ -542,30 +488,10 @@ hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
     }
     const int rows_per_block = 4 * kRowsPerWave;
     const dim3 grid((a.B + rows_per_block - 1) / rows_per_block);
-    if (a.n <= 64 * kRegs) hipLaunchKernelGGL(output_delta_kernel<true>, grid, dim3(256), 0, s, a);
-    else hipLaunchKernelGGL(output_delta_kernel<false>, grid, dim3(256), 0, s, a);
-    return hipGetLastError();
-}
-
-hipError_t ghip_sgd_update_f32(float* W, float* V, const float* G, long long n, float lr, float mom,
-                               float wd1, float wd2, float gscale, hipStream_t s)
-{
-    hipLaunchKernelGGL(sgd_update_f32_kernel, dim3(grid_for(n, 4096)), dim3(256), 0, s, W, V, G, n, lr, mom,
-                       wd1, wd2, gscale);
-    return hipGetLastError();
-}
-
-hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bias, float* vb, float lr,
-                                float mom, hipStream_t s)
-{
-    hipLaunchKernelGGL(bias_update_f32_kernel, dim3((n + 63) / 64), dim3(256), 0, s, D, B, n, ldd, bias, vb, lr, mom);
-    return hipGetLastError();
-}
-
-hipError_t ghip_colsum_f32(const float* D, int B, int n, int ldd, int chunks, float* partial, hipStream_t s)
-{
-    const int rpc = (B + chunks - 1) / chunks;
-    hipLaunchKernelGGL(colsum_f32_kernel, dim3((n + 63) / 64, chunks), dim3(256), 0, s, D, B, n, ldd, rpc, partial);
+    if (a.n <= 64) hipLaunchKernelGGL(output_delta_kernel<1>, grid, dim3(256), 0, s, a);
+    else if (a.n <= 256) hipLaunchKernelGGL(output_delta_kernel<4>, grid, dim3(256), 0, s, a);
+    else if (a.n <= 1024) hipLaunchKernelGGL(output_delta_kernel<16>, grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(output_delta_kernel<0>, grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -259,6 +259,7 @@ enum GemmEpilogue {
     EPI_STORE = 0,        // C = acc * alpha
     EPI_BIAS_ACT = 1,     // C = squash(acc + bias[n])
     EPI_MUL_DER = 2,      // C = acc * act_der(aux[m][n])
+    EPI_SGD = 3,          // C is the weight matrix: g = acc*alpha + wd1*sign(W) + wd2*W; d = lr*g + mom*V; V = d; W -= d
 };
 struct GemmF32Args {
     const float* A; const float* B; float* C;
@@ -270,6 +271,11 @@ struct GemmF32Args {
     const float* aux;    // EPI_MUL_DER: activations [M][N], ld = ldc
     int act; float act_param;
     float alpha;
+    // EPI_SGD: momentum of C, hyper-parameters; with bias_w the kernel also sums its A operand over K
+    // (A = delta^T: the bias gradient, times alpha) and updates bias_w / bias_v[M] the same way, no decay
+    float* V;
+    float lr, mom, wd1, wd2;
+    float* bias_w; float* bias_v;
 };
 hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s);
 
@@ -282,19 +288,12 @@ struct DeltaArgs {
     int B, n, ldp, ldy;
     int act; float act_param; int cost;
     double* acc;
+    double* acc_clear;  // 4 doubles set to zero by this launch (the next launch's accumulators), or NULL
     int* cm;       // n x n confusion counters (row expected, column predicted) or NULL
     int store_p;   // write the activated outputs (softmax probabilities) back into P
 };
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s);
 
-// Fused SGD + momentum + L1/L2 update:  d = lr*(g*gscale + wd1*sign(w) + wd2*w) + mom*v; v = d; w -= d
-hipError_t ghip_sgd_update_f32(float* W, float* V, const float* G, long long n, float lr, float mom,
-                               float wd1, float wd2, float gscale, hipStream_t s);
-// gb[o] = sum_b D[b][o] (fp32 D [B][n]) fused with the bias update (no decay)
-hipError_t ghip_bias_update_f32(const float* D, int B, int n, int ldd, float* bias, float* vbias,
-                                float lr, float mom, hipStream_t s);
-// partial[c][o] = column sums of D over row chunk c (chunks of ceil(B / chunks) rows)
-hipError_t ghip_colsum_f32(const float* D, int B, int n, int ldd, int chunks, float* partial, hipStream_t s);
 hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s);
 hipError_t ghip_fill_f64(double* p, long long n, double v, hipStream_t s);
 
