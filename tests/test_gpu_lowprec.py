@@ -161,3 +161,35 @@ def test_bf16_step_at_full_tile_size():
         print("layer", l, "update error vs pipeline statement", fro, flush=True)
         assert fro <= 1e-2, (l, fro)
     g.close()
+
+
+@pytest.mark.parametrize("kind", ["bf16", "e4m3"])
+def test_full_size_forward_is_row_wise(kind):
+    """At the benchmark's full shapes (bf16: 4096-4096-4096-4096-4096-1024, batch 8192; e4m3: 8192 wide,
+    batch 4096) no CPU statement finishes in seconds, but the forward pass has properties that hold at
+    any size: every row's outputs depend on that row alone (a row-permuted batch gives the permuted
+    outputs, duplicated rows give duplicated outputs), bit for bit -- whatever tile a row lands in,
+    its dot products run over K in the same order (for e4m3 the scale is per row as well) -- and a
+    batch of zeros gives the activation of the bias, zero here."""
+    import pyglades as pg
+    print("full size", kind, flush=True)
+    rng = np.random.default_rng(5)
+    if kind == "bf16":
+        sizes, B, dt = [4096, 4096, 4096, 4096, 4096, 1024], 8192, pg.BF16
+    else:
+        sizes, B, dt = [8192, 8192, 8192, 8192, 1024], 4096, pg.FP8_INFER
+    nl = len(sizes) - 1
+    g = pg.Net(pg.make_spec(sizes, [po.RELU] * nl, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=dt))
+    for l in range(nl):
+        g.set_params(l, rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l])))
+    if kind == "e4m3":
+        g.quantize_fp8(want=False)
+    X = rng.standard_normal((B, sizes[0]), dtype=np.float32)
+    X[B // 2:B // 2 + 256] = X[:256]          # duplicated rows, a tile apart
+    out = g.forward(X)
+    assert np.isfinite(out).all() and (out > 0).any() and (out == 0).any()   # ReLU outputs of a live network
+    assert np.array_equal(out[B // 2:B // 2 + 256], out[:256])
+    perm = rng.permutation(B)
+    assert np.array_equal(g.forward(X[perm]), out[perm])
+    assert not np.any(g.forward(np.zeros((256, sizes[0]), np.float32)))
+    g.close()
