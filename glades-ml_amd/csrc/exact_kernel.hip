@@ -55,6 +55,17 @@ __device__ __forceinline__ float bias_chain(float b, const float* bs, int no, in
     return b;
 }
 
+// Barrier between the phases of a row.  With the state in LDS the phases only hand LDS data to one
+// another, so the wait covers LDS operations alone: __syncthreads() would also wait for the global
+// loads that prefetch the next row and for the confusion-matrix atomics, a trip to memory per row.
+// With the state in global memory the full barrier stays.
+template <bool kLds>
+__device__ __forceinline__ void row_barrier()
+{
+    if (kLds) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else __syncthreads();
+}
+
 // One workgroup per network: `p` describes the (shared) architecture, hyper-parameters and data
 // table; with `multi` each workgroup b takes its own parameter / result pointers from multi[b]
 // (the subnets of a MetaNetwork train at the same time, one per compute unit), without it the
@@ -99,7 +110,9 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     // (predicted, expected) pairs of the rows since the last flush; their cost and accuracy terms
     // are computed a ring-full at a time, one lane each, and summed in visiting order afterwards
     const int cap = p.metric_cap;
-    float* rp = (float*)(sflag + 4);
+    // the 2^(i/32) table of expf, so that a sigmoid costs an LDS read instead of a trip to memory
+    unsigned long long* sT = (unsigned long long*)(((uintptr_t)(sflag + 4) + 7) & ~(uintptr_t)7);
+    float* rp = (float*)(sT + 32);
     float* re = rp + cap;
     int fill = 0;
     int* sm = (int*)(re + cap);
@@ -121,6 +134,10 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     }
     if (tid < GHIP_MAX_LAYERS) sbias[tid] = own.bias[tid];
     if (tid == 0) sflag[0] = 0;
+    if (tid < 32) {
+        const unsigned long long tab[32] = GLM_EXP2_TAB;
+        sT[tid] = tab[tid];
+    }
 
     const float data_size = (float)((unsigned)p.n_rows * (unsigned)nout);
     const float fmb = (float)p.mb;
@@ -146,6 +163,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
             __threadfence();
             __syncthreads();
         }
+        int rmod = 0;  // r % mb
         for (long long r = 0; r < p.n_rows; ++r) {
             // ---- stage the row (prefetched) and start fetching the next one
             if (small_row) {
@@ -173,7 +191,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 const unsigned char* mr = own.masks + ((long long)ep * p.n_rows + r) * mask_len;
                 for (int k = tid; k < mask_len; k += T) sm[k] = mr[k];
             }
-            __syncthreads();
+            row_barrier<kLds>();
 
             // ---- ForwardPass (network.cpp:457-516)
             for (int l = 0; l < L; ++l) {
@@ -201,14 +219,14 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
                     }
                     if (l != 0) z = __fadd_rn(z, bl);
-                    const float a = ghip_squash<true>(z, act, par);
+                    const float a = ghip_squash<true>(z, act, par, (const uint64_t*)sT);
                     aout[o] = a;
                     if (l == L - 1) {
                         rp[fill + o] = a;
                         re[fill + o] = sy[o];
                     }
                 }
-                __syncthreads();
+                row_barrier<kLds>();
             }
             fill += nout;
             const float* pred = sa + p.aoff[L];
@@ -237,7 +255,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     rp[k] = ghip_cost<true>(ex, pr, data_size, p.cost);
                     re[k] = ghip_accuracy_term(pr, ex);
                 }
-                __syncthreads();
+                row_barrier<kLds>();
                 if (tid == serial) {
                     for (int k = 0; k < fill; ++k) {
                         tot_err = __fadd_rn(tot_err, rp[k]);
@@ -260,8 +278,8 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         if (kDrop) sE[p.aoff[L] + o] = e;
                     }
                 }
-                __syncthreads();
-                const bool apply = (r % p.mb) == 0;
+                row_barrier<kLds>();
+                const bool apply = rmod == 0;
                 for (int Lo = L; Lo > 0; --Lo) {
                     const int l = Lo - 1;
                     const int ni = p.sizes[l], no = p.sizes[Lo], ld = p.ld[l];
@@ -343,7 +361,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         }
                         if (tid == serial) sbias[l] = b;
                     }
-                    __syncthreads();
+                    row_barrier<kLds>();
                     // ---- error partials of the in-layer with the UPDATED weights
                     //      (network.cpp:660-662), then its own d and lr*d for the next round
                     if (l != 0) {
@@ -374,7 +392,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                             dn[i] = d;
                             bn[i] = __fmul_rn(lrn, d);
                         }
-                        __syncthreads();
+                        row_barrier<kLds>();
                     }
                     if (kDrop && Lo < L) {
                         // clearErrDer of the out-layer's nodes: only by a valid pair with the last
@@ -382,10 +400,13 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         if (!mi[ni - 1])
                             for (int o = tid; o < no; o += T)
                                 if (!mo[o]) sE[p.aoff[Lo] + o] = 0.0f;
-                        __syncthreads();
+                        row_barrier<kLds>();
                     }
                 }
+            } else {
+                row_barrier<kLds>();  // the metrics lane reads this row's outputs and targets: the next row waits
             }
+            if (++rmod == p.mb) rmod = 0;
         }
         // ---- end of epoch (network.cpp:193-195, Terminator.cpp:73-74)
         if (tid == serial) {
@@ -447,7 +468,7 @@ hipError_t ghip_launch_gmath_eval(int fn, int kind, float param, const float* a,
 
 size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropout)
 {
-    size_t f = (size_t)3 * p.node_floats + p.sizes[p.n_layers] + GHIP_MAX_LAYERS + 4 + (size_t)2 * p.metric_cap;
+    size_t f = (size_t)3 * p.node_floats + p.sizes[p.n_layers] + GHIP_MAX_LAYERS + 4 + 2 + 64 + (size_t)2 * p.metric_cap;
     if (dropout) f += (size_t)2 * p.node_floats;
     if (state_in_lds) f += (size_t)3 * p.state_floats;
     return f * sizeof(float);

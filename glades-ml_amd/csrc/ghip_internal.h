@@ -21,10 +21,11 @@ __device__ __forceinline__ float ghip_tanh(float z)
     if (kPrecise) return glm_tanhf(z);
     return tanhf(z);
 }
+// exp_tab: the table of glm_expf_tab where the caller keeps a copy close by (LDS), or NULL
 template <bool kPrecise>
-__device__ __forceinline__ float ghip_exp(float z)
+__device__ __forceinline__ float ghip_exp(float z, const uint64_t* exp_tab = nullptr)
 {
-    if (kPrecise) return glm_expf(z);
+    if (kPrecise) return exp_tab ? glm_expf_tab(z, exp_tab) : glm_expf(z);
     return expf(z);
 }
 template <bool kPrecise>
@@ -35,7 +36,7 @@ __device__ __forceinline__ float ghip_log(float z)
 }
 
 template <bool kPrecise>
-__device__ __forceinline__ float ghip_squash(float z, int act, float p)
+__device__ __forceinline__ float ghip_squash(float z, int act, float p, const uint64_t* exp_tab = nullptr)
 {
     switch (act) {
     case GHIP_TANH: return ghip_tanh<kPrecise>(z);
@@ -43,11 +44,11 @@ __device__ __forceinline__ float ghip_squash(float z, int act, float p)
         if (z > 1.0f - p) return 1.0f;
         if (z < p - 1.0f) return -1.0f;
         return ghip_tanh<kPrecise>(z);
-    case GHIP_SIGMOID: return __fdiv_rn(1.0f, __fadd_rn(1.0f, ghip_exp<kPrecise>(-z)));
+    case GHIP_SIGMOID: return __fdiv_rn(1.0f, __fadd_rn(1.0f, ghip_exp<kPrecise>(-z, exp_tab)));
     case GHIP_SIGMOIDP:
         if (z < p) return 0.01f;
         if (z > 1.0f - p) return 0.99f;
-        return __fdiv_rn(1.0f, __fadd_rn(1.0f, ghip_exp<kPrecise>(-z)));
+        return __fdiv_rn(1.0f, __fadd_rn(1.0f, ghip_exp<kPrecise>(-z, exp_tab)));
     case GHIP_RELU: return (z < GHIP_OUTLIER) ? 0.0f : z;
     case GHIP_LEAKY: return (z < GHIP_OUTLIER) ? __fmul_rn(p, z) : z;
     case GHIP_LINEAR: return __fmul_rn(p, z);

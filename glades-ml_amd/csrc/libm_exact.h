@@ -155,9 +155,9 @@ GLM_FN float glm_tanhf(float x)
         0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull                   \
     }
 
-GLM_FN float glm_expf(float x)
+// T: the 32 table entries above, wherever the caller keeps them (a kernel may hold them in LDS)
+GLM_FN float glm_expf_tab(float x, const uint64_t* T)
 {
-    const uint64_t T[32] = GLM_EXP2_TAB;
     const double C0 = 0x1.c6af84b912394p-5 / 32 / 32 / 32, C1 = 0x1.ebfce50fac4f3p-3 / 32 / 32,
                  C2 = 0x1.62e42ff0c52d6p-1 / 32;
     const double InvLn2N = 0x1.71547652b82fep+0 * 32, Shift = 0x1.8p+52;
@@ -180,6 +180,12 @@ GLM_FN float glm_expf(float x)
     y = __builtin_fma(p, r2, y);
     y = y * s;
     return (float)y;
+}
+
+GLM_FN float glm_expf(float x)
+{
+    const uint64_t T[32] = GLM_EXP2_TAB;
+    return glm_expf_tab(x, T);
 }
 
 GLM_FN float glm_logf(float x)
