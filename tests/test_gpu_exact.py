@@ -141,6 +141,44 @@ def test_edge_shapes_against_oracle(sizes, N, mb):
     net.close()
 
 
+def test_network_too_large_for_lds_keeps_its_state_in_global_memory():
+    """1100-40-3: three floats per edge are 529 KB, more than a compute unit's LDS, so weights and
+    delta windows stay in global memory (L2) and every phase ends with a full barrier; alone and as
+    three networks in one launch, bit for bit against the CPU restatement."""
+    import pyglades as pg
+    rng = np.random.default_rng(17)
+    sizes, N, mb, E = [1100, 40, 3], 9, 4, 3
+    acts = [po.TANH, po.SIGMOID]
+    ospec = po.make_spec(sizes, acts, lr=0.001, mom=0.5, wd2=0.001, batch=mb, cost=po.CLASSIFICATION)
+    gspec = pg.make_spec(sizes, acts, lr=0.001, mom=0.5, wd2=0.001, batch=mb, cost=pg.CLASSIFICATION, mode=pg.MODE_EXACT)
+    X = rng.random((N, sizes[0])).astype(np.float32)
+    Y = (np.eye(3, dtype=np.float32)[rng.integers(0, 3, N)] * 0.98 + 0.01).astype(np.float32)
+    nets, want = [], []
+    for k in range(4):
+        Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (0.5 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(2)]
+        o = po.ExactNet(ospec)
+        g = pg.Net(gspec)
+        for l in range(2):
+            o.set_weights(l, Ws[l]); o.set_bias(l, 0.01 * l)
+            g.set_params(l, Ws[l], 0.01 * l)
+        g.set_dataset(X, Y)
+        oms = [o.epoch(X, Y)[0] for _ in range(E)]
+        nets.append(g)
+        want.append((o, oms))
+    got = [nets[0].run_epochs_exact(E)[0]] + pg.run_epochs_exact_multi(nets[1:], E)
+    for g, (o, oms), ms in zip(nets, want, got):
+        assert bits_equal([m[0] for m in ms], [m.loss for m in oms])
+        assert [m[2] for m in ms] == [m.correct for m in oms]
+        for l in range(2):
+            W, b = g.get_params(l)
+            assert bits_equal(W, o.get_weights(l)), l
+            s, t = g.get_state(l)
+            os_, ot = o.get_window(l)
+            assert bits_equal(s, os_) and bits_equal(t, ot), l
+        assert bits_equal(g.get_params(1)[1][0], o.get_bias(1))
+        g.close()
+
+
 def test_error_paths():
     import pyglades as pg
     with pytest.raises(pg.GladesHipError):   # BATCH_FULL = 0 is "row % 0" in the reference
