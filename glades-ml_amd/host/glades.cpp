@@ -123,6 +123,73 @@ void NNInfo::setActivationParam(unsigned int index, float v)
 }
 void NNInfo::addHiddenLayer(HiddenLayerInfo* l) { if (l) layers.push_back(l); }
 
+void LayerInfo::copyParamsFrom(const LayerInfo* src)
+{
+    if (!src) return;
+    setSize(src->size());
+    learningRate = src->getLearningRate(); momentumFactor = src->getMomentumFactor();
+    weightDecay1 = src->getWeightDecay1(); weightDecay2 = src->getWeightDecay2();
+    pDropout = src->getPDropout(); activationType = src->getActivationType();
+}
+
+void NNInfo::setPInput(float v) { if (inputLayer) inputLayer->setPDropout(v); }
+void NNInfo::setWeightDecay1(unsigned int index, float v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setWeightDecay1(v); }
+    else if (layers[index - 1]) layers[index - 1]->setWeightDecay1(v);
+}
+void NNInfo::setWeightDecay2(unsigned int index, float v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setWeightDecay2(v); }
+    else if (index >= 2 && layers[index - 2]) layers[index - 2]->setWeightDecay2(v);
+}
+void NNInfo::setPDropout(unsigned int index, float v)
+{
+    if (index > layers.size()) return;
+    if (index == 0) { if (inputLayer) inputLayer->setPDropout(v); }
+    else if (layers[index - 1]) layers[index - 1]->setPDropout(v);
+}
+void NNInfo::copyHiddenLayer(unsigned int dst, unsigned int src)
+{
+    if (dst >= layers.size() || src >= layers.size() || !layers[dst] || !layers[src]) return;
+    layers[dst]->copyParamsFrom(layers[src]);
+}
+void NNInfo::resizeHiddenLayers(unsigned int newCount)
+{
+    while (layers.size() > newCount) { delete layers.back(); layers.pop_back(); }
+    while (layers.size() < newCount) layers.push_back(new HiddenLayerInfo(2, 0.01f, 0.0f, 0.0f, 0.0f, 0.0f, 0, 0.0f));
+}
+void NNInfo::removeHiddenLayer(unsigned int index)
+{
+    if (index >= layers.size() || !layers[index]) return;
+    layers.erase(layers.begin() + index);
+}
+
+void NNInfo::print() const
+{
+    if (!inputLayer || !outputLayer) return;
+    static const char* headers[10] = {"Layer", "Size", "batchSize", "lrnRate", "mFactor", "wDecay", "pDropout", "actvtn", "actParam", "cost"};
+    printf("[NNINFO] Current NNInfo Values\n[NNINFO] ");
+    for (int i = 0; i < 10; ++i) printf("%s\t", headers[i]);
+    printf("\n");
+    const NNTable t = toTable();
+    for (size_t row = 0; row < t.size(); ++row) {
+        printf("[NNINFO] ");
+        if (row == 0) printf("Input\t");
+        else if (row + 1 < t.size()) printf("H[%d]\t", (int)row);
+        else printf("Output\t");
+        for (size_t col = 0; col < t[row].size(); ++col) {
+            const bool whole = col == COL_SIZE || col == COL_BATCH_SIZE || col == COL_ACTIVATION_TYPE || col == COL_OUTPUT_TYPE;
+            if ((int)t[row][col] == -1) printf("\t");
+            else if (whole) printf("%d\t", (int)t[row][col]);
+            else printf("%f\t", t[row][col]);
+        }
+        printf("\n");
+    }
+}
+
 NNTable NNInfo::toTable() const
 {
     NNTable t;

@@ -66,6 +66,8 @@ public:
     void setPDropout(float v) { pDropout = v; }
     void setActivationType(int v) { activationType = v; }
     void setActivationParam(float v) { activationParam = v; }
+    // layerinfo.cpp:57-66: size, rates, decays, dropout and activation type; the activation parameter stays
+    void copyParamsFrom(const LayerInfo* src);
 };
 
 class InputLayerInfo : public LayerInfo
@@ -131,6 +133,7 @@ public:
     InputLayerInfo* getInputLayer() const { return inputLayer; }
     std::vector<HiddenLayerInfo*> getLayers() const { return layers; }
     int numHiddenLayers() const { return (int)layers.size(); }
+    int getInputLayerSize() const { return inputLayer ? inputLayer->size() : 0; }
     int getHiddenLayerSize(unsigned int) const;
     unsigned int getOutputLayerSize() const;
     // index 0 reads the input row, index k >= 1 the hidden row k-1 (nninfo.cpp:240-373);
@@ -143,15 +146,31 @@ public:
     int getActivationType(unsigned int) const;
     float getActivationParam(unsigned int) const;
 
+    void print() const;  // nninfo.cpp:379-431: "[NNINFO]" lines, one per layer row, -1 cells left blank
+
     void setName(const std::string& v) { name = v; }
+    void setInputType(int v) { inputType = v; }
+    void setPInput(float);
+    void setLayers(const std::vector<HiddenLayerInfo*>& newLayers) { layers = newLayers; }
     void setOutputType(int);
     void setOutputSize(int);
     void setBatchSize(int);
     void setLearningRate(unsigned int, float);
     void setMomentumFactor(unsigned int, float);
+    void setWeightDecay1(unsigned int, float);
+    // the reference addresses hidden row index-2 here (nninfo.cpp:586-603), so index 1 reaches no row
+    // (there it reads layers[-1]); this does nothing for index 1
+    void setWeightDecay2(unsigned int, float);
+    void setPDropout(unsigned int, float);
     void setActivationType(unsigned int, int);
     void setActivationParam(unsigned int, float);
     void addHiddenLayer(HiddenLayerInfo*);
+    void copyHiddenLayer(unsigned int dst, unsigned int src);
+    // new rows are HiddenLayerInfo(2, 0.01, 0, 0, 0, 0, TANH, 0) (nninfo.cpp:683-686), one object per row
+    // here (the reference puts ONE object into every new slot and deletes it once per slot); rows cut
+    // off are deleted
+    void resizeHiddenLayers(unsigned int newCount);
+    void removeHiddenLayer(unsigned int index);  // the row leaves the list; like the reference, it is not deleted
 
     NNTable toTable() const;
     bool fromTable(const std::string& netName, const NNTable& table);

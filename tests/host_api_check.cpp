@@ -48,6 +48,37 @@ static int do_nninfo(const char* path, const char* resave)
     return net.save(resave) ? 0 : 2;
 }
 
+// the editing methods of NNInfo (nninfo.cpp:436-703) on a loaded table; prints the table after every step
+static int do_nnedit(const char* path)
+{
+    NNetwork net;
+    if (!net.load(path)) return 1;
+    NNInfo* s = net.getNNInfo();
+    auto dump = [&](const char* what) {
+        printf("-- %s\n", what);
+        const NNTable t = s->toTable();
+        for (size_t r = 0; r < t.size(); ++r) {
+            for (size_t c = 0; c < t[r].size(); ++c) printf("%s%g", c ? "," : "", t[r][c]);
+            printf("\n");
+        }
+    };
+    dump("loaded");
+    s->setPInput(0.25f); s->setPDropout(1, 0.5f); s->setWeightDecay1(2, 0.125f);
+    s->setWeightDecay2(0, 0.75f); s->setWeightDecay2(1, 0.0625f); s->setWeightDecay2(2, 0.03125f);
+    dump("rates");
+    s->copyHiddenLayer(1, 0);
+    dump("copy 1 <- 0");
+    s->resizeHiddenLayers(4);
+    s->setLearningRate(3, 0.5f);   // hidden row 2 only: the new rows are separate objects
+    dump("resize 4");
+    s->removeHiddenLayer(0);
+    s->resizeHiddenLayers(2);
+    dump("remove 0, resize 2");
+    printf("input size %d hidden %d p %g/%g\n", s->getInputLayerSize(), s->numHiddenLayers(), s->getPInput(), s->getPDropout(0));
+    s->print();
+    return 0;
+}
+
 // pairs.bin: rows of n (expected, predicted) float pairs, interleaved as NNetwork's results list holds them
 static int do_cmatrix(int n, const char* in, const char* out)
 {
@@ -420,6 +451,7 @@ int main(int argc, char** argv)
 {
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
+    if (argc >= 3 && !strcmp(argv[1], "nnedit")) return do_nnedit(argv[2]);
     if (argc >= 7 && !strcmp(argv[1], "meta")) return do_meta(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 8 && !strcmp(argv[1], "checkpoint")) return do_checkpoint(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7]);
     if (argc >= 9 && !strcmp(argv[1], "dropout")) {

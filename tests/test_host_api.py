@@ -50,6 +50,44 @@ def test_nninfo_table_round_trip_and_index_shift():
 
 
 @needs_bin
+def test_nninfo_editing_methods():
+    """setPInput / setPDropout / setWeightDecay1 / setWeightDecay2 (which addresses hidden row index-2,
+    nninfo.cpp:586-603) / copyHiddenLayer (everything but the activation parameter, layerinfo.cpp:57-66) /
+    resizeHiddenLayers (rows of 2 nodes, lr 0.01) / removeHiddenLayer / print."""
+    table = ("Size,batchSize,learningRate,momentumFactor,weightDecay1,weightDecay2,pDropout,activationType,activationParam,outputType\n"
+             "-1,7,0.003000,0.500000,0.010000,0.020000,0.000000,0,0.000000,-1\n"
+             "5,7,0.010000,0.250000,0.030000,0.040000,0.000000,2,0.100000,-1\n"
+             "3,7,0.020000,0.125000,0.050000,0.060000,0.000000,5,0.200000,-1\n"
+             "2,7,-1.000000,-1.000000,-1.000000,-1.000000,-1.000000,-1,-1.000000,1")
+    with tempfile.TemporaryDirectory() as td:
+        src = os.path.join(td, "net")
+        open(src, "w").write(table)
+        out = subprocess.check_output([BIN, "nnedit", src], text=True).splitlines()
+    blocks, cur = {}, None
+    for ln in out:
+        if ln.startswith("-- "):
+            cur = ln[3:]
+            blocks[cur] = []
+        elif cur is not None and not ln.startswith(("[NNINFO]", "input size")):
+            blocks[cur].append(ln)
+    assert blocks["loaded"][1] == "5,7,0.01,0.25,0.03,0.04,0,2,0.1,-1"
+    r = blocks["rates"]
+    assert r[0] == "-1,7,0.003,0.5,0.01,0.75,0.25,0,0,-1"          # input row: pInput, weightDecay2(0)
+    assert r[1] == "5,7,0.01,0.25,0.03,0.03125,0.5,2,0.1,-1"       # hidden row 0: pDropout(1), weightDecay2(2) lands here
+    assert r[2] == "3,7,0.02,0.125,0.125,0.06,0,5,0.2,-1"          # hidden row 1: weightDecay1(2); weightDecay2(1) reached no row
+    c = blocks["copy 1 <- 0"]
+    assert c[2] == "5,7,0.01,0.25,0.03,0.03125,0.5,2,0.2,-1"       # all of row 0 except the activation parameter
+    z = blocks["resize 4"]
+    assert len(z) == 6 and z[3] == "2,7,0.5,0,0,0,0,0,0,-1" and z[4] == "2,7,0.01,0,0,0,0,0,0,-1"
+    e = blocks["remove 0, resize 2"]
+    assert len(e) == 4 and e[1] == c[2] and e[2] == z[3]
+    assert "input size 0 hidden 2 p 0.25/0.25" in out   # InputLayerInfo is a LayerInfo(0) (inputlayerinfo.cpp:29-33)
+    nn = [ln for ln in out if ln.startswith("[NNINFO]")]
+    assert nn[0] == "[NNINFO] Current NNInfo Values" and nn[1].split("\t")[:3] == ["[NNINFO] Layer", "Size", "batchSize"]
+    assert nn[2].startswith("[NNINFO] Input\t\t7\t0.003000") and nn[3].startswith("[NNINFO] H[1]\t5\t7\t") and nn[-1].startswith("[NNINFO] Output\t2\t7\t")
+
+
+@needs_bin
 def test_cmatrix_class_matches_restatement():
     """CMatrix::addResult / updateResultParams / getOverall* fed with (expected, predicted) pairs."""
     rng = np.random.default_rng(9)
