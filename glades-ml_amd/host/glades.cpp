@@ -6,6 +6,8 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <sys/stat.h>
+#include <sys/time.h>
 #include <time.h>
 #include <thread>
 
@@ -419,10 +421,34 @@ void NNetwork::clean()
 
 std::string NNetwork::getName() const { return skeleton ? skeleton->getName() : std::string(); }
 
+int64_t NNetwork::getCurrentTimeMilliseconds() const
+{
+    struct timeval tv;
+    gettimeofday(&tv, NULL);
+    return (int64_t)((unsigned long long)tv.tv_sec * 1000ULL + (unsigned long long)tv.tv_usec / 1000ULL);
+}
+
+void NNetwork::resetGraphs()
+{
+    learningCurve.clear();
+    results.clear();
+}
+
+bool NNetwork::save() const
+{
+    if (!skeleton) return false;
+    if (!doesDatabaseExist()) createDatabase();
+    mkdir("database/neuralnetworks", 0777);
+    return skeleton->saveFile("database/neuralnetworks/" + skeleton->getName());
+}
+
 bool NNetwork::load(const std::string& path)
 {
     NNInfo* info = new NNInfo("");
-    if (!info->loadFile(path)) { delete info; return false; }
+    struct stat st;
+    const bool as_given = stat(path.c_str(), &st) == 0;
+    if (!info->loadFile(as_given ? path : "database/neuralnetworks/" + path)) { delete info; return false; }
+    if (!as_given) info->setName(path);
     skeleton = info;  // like the reference, the loaded skeleton is never freed by the network
     return true;
 }
@@ -1107,6 +1133,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
     const bool want_preds = (size_t)nRows * nOut <= (1u << 20);
     std::vector<float> preds(want_preds ? (size_t)nRows * nOut : 0);
     std::vector<float> Ylast = di->getTrainExpectedRow(nRows - 1);
+    resetGraphs();  // network.cpp:167
     running = true;
     while (running) {
         if (mode == MODE_EXACT) {
@@ -1124,6 +1151,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
                 break;
             }
             if (ran <= 0) break;
+            for (int e = 0; e < ran; ++e) learningCurve.push_back(ms[e].accuracy);
             afterEpochs(&ms[ran - 1], ran, runType);
         } else {
             if (confusionMatrix.size() > 0) ghip_net_confusion_reset(dev);  // network.cpp:183-185
@@ -1142,6 +1170,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             if (failed) break;
             ghip_metrics last;
             last.loss = (float)(loss / nRows); last.accuracy = (float)(acc / nRows); last.correct = correct;
+            learningCurve.push_back(last.accuracy);
             afterEpochs(&last, 1, runType);
         }
         if (terminator.triggered(time(NULL), epochs, overallTotalAccuracy)) break;
@@ -1213,7 +1242,26 @@ bool MetaNetwork::runGroup(DataInput* d, int runType)
 
 // ------------------------------------------------------------------ facade (ML/main.cpp:51-243)
 
+// ML/main.cpp:32-45.  glades::init() of the reference also creates the folder (main.cpp:51-56); here that
+// is left to the first NNetwork::save(), so that initialising the device writes nothing to disk.
+bool doesDatabaseExist()
+{
+    struct stat buffer;
+    return stat("database", &buffer) == 0 && S_ISDIR(buffer.st_mode);
+}
+void createDatabase() { mkdir("database", 0777); }
+
 void init() { ghip_init(0); }
+
+bool saveNeuralNetwork(NNetwork* newNet)  // ML/main.cpp:58-73
+{
+    if (!newNet) return false;
+    if (!newNet->save()) {
+        printf("Unable to save \"%s\"\n", newNet->getName().c_str());
+        return false;
+    }
+    return true;
+}
 
 MetaNetwork* train(NNetwork* net, DataInput* d)
 {

@@ -349,6 +349,7 @@ class NNetwork
     int minibatchSize;
     int64_t id;
     std::vector<float> results;                 // (expected, predicted) pairs of the last row
+    std::vector<float> learningCurve;           // accuracy after every epoch of the current run
     std::vector<std::vector<float> > initW;     // weights injected before the first run
     std::vector<std::vector<float> > initB;
     std::vector<std::vector<float> > initStateA, initStateB;  // optimiser state of a restored checkpoint
@@ -368,7 +369,6 @@ class NNetwork
     bool prepare(DataInput*);                        // checks + build on first use
     void afterEpochs(const void* lastMetrics, int ran, int runType);  // statistics, class figures, progress line
     bool build();
-    void clean();
 
 public:
     bool hasDropout() const;  // some layer's rate int(p*100) lies in 1..99
@@ -382,12 +382,17 @@ public:
     NNetwork();
     explicit NNetwork(NNInfo*);
     virtual ~NNetwork();
+    int64_t getCurrentTimeMilliseconds() const;  // network.cpp:82-87
     bool getRunning() const { return running; }
     int getEpochs() const { return epochs; }
     void stop() { running = false; }
 
-    bool load(const std::string& path);  // reads an NNInfo table file (network.cpp:701-712)
+    // reads an NNInfo table file (network.cpp:701-712).  The reference resolves a network's name inside
+    // its database folder (SaveFolder("neuralnetworks"), nninfo.cpp:787-798): a path that does not exist
+    // is looked up as database/neuralnetworks/<path>
+    bool load(const std::string& path);
     bool save(const std::string& path) const;
+    bool save() const;  // network.cpp:714-722 -> NNInfo::save: database/neuralnetworks/<name>
 
     void train(DataInput*);
     void test(DataInput*);
@@ -397,6 +402,11 @@ public:
     NNInfo* getNNInfo() { return skeleton; }
     float getAccuracy() const { return overallTotalAccuracy; }
     std::vector<float> getResults() const { return results; }
+    // The reference declares the list and never fills it (network.cpp:730-733, 764-775); here it holds
+    // the accuracy after every epoch since the run started.
+    std::vector<float> getLearningCurve() const { return learningCurve; }
+    void clean();        // network.cpp:745-762: lets go of the device network and the data
+    void resetGraphs();  // network.cpp:764-775
 
     // ---- absent from the reference (its loss has no getter and its weights are not reachable)
     float getLoss() const { return overallTotalError; }
@@ -456,6 +466,9 @@ public:
 };
 
 void init();
+bool doesDatabaseExist();                 // ML/main.cpp:32-36: is there a "database" folder in the working directory
+void createDatabase();                    // ML/main.cpp:38-45
+bool saveNeuralNetwork(NNetwork*);        // ML/main.cpp:58-73
 // ML/main.cpp:82-243: wrap in a MetaNetwork the caller owns, run every subnet on the same data
 MetaNetwork* train(NNInfo*, DataInput*);
 MetaNetwork* train(NNetwork*, DataInput*);

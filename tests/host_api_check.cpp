@@ -79,6 +79,27 @@ static int do_nnedit(const char* path)
     return 0;
 }
 
+// NNetwork::save() / load(name) / glades::saveNeuralNetwork through the database folder of the working
+// directory (the caller runs this in a scratch directory), getLearningCurve, getCurrentTimeMilliseconds
+static int do_db(const char* table)
+{
+    if (glades::doesDatabaseExist()) return 1;
+    NNetwork net;
+    if (!net.load(table)) return 2;
+    net.getNNInfo()->setName("saved-net");
+    if (!glades::saveNeuralNetwork(&net) || !glades::doesDatabaseExist()) return 3;
+    NNetwork again;
+    if (!again.load("saved-net")) return 4;           // no such path: looked up in database/neuralnetworks/
+    if (again.getName() != "saved-net") return 5;
+    if (again.getNNInfo()->toTable() != net.getNNInfo()->toTable()) return 6;
+    NNetwork none;
+    if (none.load("no-such-net") || none.save() || glades::saveNeuralNetwork(NULL)) return 7;
+    const int64_t t0 = net.getCurrentTimeMilliseconds();
+    if (t0 < 1600000000000LL) return 8;
+    printf("db ok\n");
+    return 0;
+}
+
 // pairs.bin: rows of n (expected, predicted) float pairs, interleaved as NNetwork's results list holds them
 static int do_cmatrix(int n, const char* in, const char* out)
 {
@@ -191,6 +212,8 @@ static int train_and_dump(NNetwork& net, DataInput* di, int nl, const char* out)
     if (!net.getLastError().empty()) { fprintf(stderr, "error: %s\n", net.getLastError().c_str()); return 5; }
     const int trained = net.getEpochs();
     const float acc = net.getAccuracy(), loss = net.getLoss();
+    const std::vector<float> curve = net.getLearningCurve();
+    if ((int)curve.size() != trained || (trained > 0 && curve.back() != acc)) return 6;  // one accuracy per epoch of the run
     std::vector<float> results = net.getResults();
     // the class figures of the last training epoch (network.cpp:218-224) and the matrix behind them
     const CMatrix& cm = net.getConfusionMatrix();
@@ -452,6 +475,7 @@ int main(int argc, char** argv)
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
     if (argc >= 3 && !strcmp(argv[1], "nnedit")) return do_nnedit(argv[2]);
+    if (argc >= 3 && !strcmp(argv[1], "db")) return do_db(argv[2]);
     if (argc >= 7 && !strcmp(argv[1], "meta")) return do_meta(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 8 && !strcmp(argv[1], "checkpoint")) return do_checkpoint(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7]);
     if (argc >= 9 && !strcmp(argv[1], "dropout")) {

@@ -88,6 +88,16 @@ def test_nninfo_editing_methods():
 
 
 @needs_bin
+def test_database_folder_conventions():
+    """NNetwork::save() writes database/neuralnetworks/<name> under the working directory, load(name)
+    finds it there, glades::saveNeuralNetwork reports failures (ML/main.cpp:32-73, nninfo.cpp:787-798)."""
+    with tempfile.TemporaryDirectory() as td:
+        assert subprocess.check_output([BIN, "db", os.path.join(NETS, "iris")], text=True, cwd=td).strip().splitlines()[-1] == "db ok"
+        saved = os.path.join(td, "database", "neuralnetworks", "saved-net")
+        assert open(saved).read().split() == open(os.path.join(NETS, "iris")).read().split()
+
+
+@needs_bin
 def test_cmatrix_class_matches_restatement():
     """CMatrix::addResult / updateResultParams / getOverall* fed with (expected, predicted) pairs."""
     rng = np.random.default_rng(9)
