@@ -1306,6 +1306,34 @@ MetaNetwork* train(MetaNetwork* m, DataInput* d)
     return m;
 }
 
+MetaNetwork::MetaNetwork(NNInfo* networkInfo, int subnetCount)
+    : name(networkInfo ? networkInfo->getName() : std::string()), collectionType(subnetCount > 1 ? ONE_TO_MANY : ONE_TO_ONE),
+      concurrent(true)
+{
+    for (int i = 0; i < subnetCount; ++i) addSubnet(networkInfo);
+}
+
+MetaNetwork::MetaNetwork(const std::string& metaNetName, const std::string& nname, int k)
+    : name(metaNetName), collectionType(k > 1 ? ONE_TO_MANY : ONE_TO_ONE), concurrent(true)
+{
+    for (int i = 0; i < k; ++i) addSubnet(nname);
+}
+
+void MetaNetwork::addSubnet(const std::string& nNetName)
+{
+    if (nNetName.empty()) return;
+    NNetwork* n = new NNetwork();
+    if (n->load(nNetName)) subnets.push_back(n);
+    else delete n;
+}
+
+NNetwork* MetaNetwork::getSubnetByName(const std::string& n) const
+{
+    for (size_t i = 0; i < subnets.size(); ++i)
+        if (subnets[i] && subnets[i]->getName() == n) return subnets[i];
+    return NULL;
+}
+
 float MetaNetwork::crossValidate(DataInput* newDataInput)
 {
     if (!newDataInput || subnets.empty()) return 0.0f;

@@ -439,11 +439,18 @@ public:
 class MetaNetwork
 {
     std::string name;
+    int collectionType;
     std::vector<NNetwork*> subnets;
     bool concurrent;
 
 public:
-    explicit MetaNetwork(const std::string& newName) : name(newName), concurrent(true) {}
+    static const int ONE_TO_ONE = 0, ONE_TO_MANY = 1;  // metanetwork.h:36-37
+    explicit MetaNetwork(const std::string& newName) : name(newName), collectionType(ONE_TO_ONE), concurrent(true) {}
+    // subnetCount networks over the same skeleton (metanetwork.cpp:36-50), e.g. for cross-validation
+    MetaNetwork(NNInfo* networkInfo, int subnetCount = 1);
+    // k networks loaded from the table `nname` (metanetwork.cpp:52-63)
+    MetaNetwork(const std::string& metaNetName, const std::string& nname, int k = 1);
+    virtual ~MetaNetwork() { name = ""; clearSubnets(); }  // the list is cleared, the networks are not deleted (metanetwork.cpp:65-69, 129-132)
     // Subnets are independent networks (metanetwork.cpp:86-127): with `concurrent` (the default) train /
     // test / crossValidate run them at the same time, one host thread and one HIP stream each, instead
     // of one after the other as the reference's loop does (ML/main.cpp:137-160).  Results are the same.
@@ -460,7 +467,12 @@ public:
     // one kernel launch for all subnets where they allow it (see glades.cpp); false = not applicable
     bool runGroup(DataInput*, int runType);
     std::string getName() const { return name; }
+    void setName(const std::string& v) { name = v; }
+    int getCollectionType() const { return collectionType; }
     void addSubnet(NNetwork* n) { if (n) subnets.push_back(n); }
+    void addSubnet(const std::string& nNetName);  // metanetwork.cpp:104-113: a network loaded from that table; nothing on failure
+    std::string getSubnetName(unsigned int i) const { return (i < subnets.size() && subnets[i]) ? subnets[i]->getName() : std::string(); }
+    NNetwork* getSubnetByName(const std::string& n) const;
     const std::vector<NNetwork*>& getSubnets() const { return subnets; }
     unsigned int size() const { return (unsigned int)subnets.size(); }
 };

@@ -94,6 +94,21 @@ static int do_db(const char* table)
     if (again.getNNInfo()->toTable() != net.getNNInfo()->toTable()) return 6;
     NNetwork none;
     if (none.load("no-such-net") || none.save() || glades::saveNeuralNetwork(NULL)) return 7;
+    // MetaNetwork's constructors and look-ups (metanetwork.cpp:30-214)
+    {
+        MetaNetwork byInfo(net.getNNInfo(), 3);
+        if (byInfo.size() != 3 || byInfo.getName() != "saved-net" || byInfo.getCollectionType() != MetaNetwork::ONE_TO_MANY) return 9;
+        if (byInfo.getSubnet(0) == byInfo.getSubnet(1) || byInfo.getSubnet(2)->getNNInfo() != net.getNNInfo()) return 10;
+        MetaNetwork byName("meta", "saved-net", 2);
+        if (byName.size() != 2 || byName.getSubnetName(1) != "saved-net" || byName.getSubnetByName("saved-net") != byName.getSubnet(0)) return 11;
+        if (byName.getSubnetByName("other") || byName.getSubnetName(5) != "") return 12;
+        byName.addSubnet(std::string("no-such-net"));
+        byName.addSubnet(std::string(""));
+        if (byName.size() != 2 || byName.getCollectionType() != MetaNetwork::ONE_TO_MANY) return 13;
+        MetaNetwork one("solo");
+        one.setName("renamed");
+        if (one.size() != 0 || one.getName() != "renamed" || one.getCollectionType() != MetaNetwork::ONE_TO_ONE) return 14;
+    }
     const int64_t t0 = net.getCurrentTimeMilliseconds();
     if (t0 < 1600000000000LL) return 8;
     printf("db ok\n");
