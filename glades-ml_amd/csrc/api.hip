@@ -862,7 +862,9 @@ int ghip_net_set_dataset(ghip_net* n, const float* host_X, const float* host_Y, 
 {
     if (!n || !host_X || n_rows <= 0) return fail(GHIP_EINVAL, "bad dataset arguments");
     const ghip_net_spec& s = n->spec;
+    HIP_TRY(hipSetDevice(g_device));
     HIP_TRY(hipStreamSynchronize(n->stream));
+    n->exMaskEpochs = 0;  // dropout flags are per row of the table they were set for
     dfree(n->ownX); dfree(n->ownY);
     const size_t nx = (size_t)n_rows * s.sizes[0], ny = (size_t)n_rows * s.sizes[s.n_layers];
     TRY(dalloc(&n->ownX, nx));
@@ -878,7 +880,9 @@ int ghip_net_set_dataset(ghip_net* n, const float* host_X, const float* host_Y, 
 int ghip_net_set_dataset_device(ghip_net* n, const float* dev_X, const float* dev_Y, int64_t n_rows)
 {
     if (!n || !dev_X || n_rows <= 0) return fail(GHIP_EINVAL, "bad dataset arguments");
+    HIP_TRY(hipSetDevice(g_device));
     HIP_TRY(hipStreamSynchronize(n->stream));
+    n->exMaskEpochs = 0;
     dfree(n->ownX); dfree(n->ownY);
     n->dX = dev_X; n->dY = dev_Y; n->n_rows = n_rows;
     return make_bf16_table(n);
@@ -1083,6 +1087,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
 int ghip_net_forward(ghip_net* n, const float* host_X, int batch, float* host_out)
 {
     if (!n || !host_X || !host_out || batch < 1) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
     if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
     const ghip_net_spec& s = n->spec;
     if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
@@ -1105,6 +1110,7 @@ int ghip_net_forward(ghip_net* n, const float* host_X, int batch, float* host_ou
 int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_out)
 {
     if (!n || batch < 1 || row0 < 0) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
     if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
     if (!n->dX) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
@@ -1120,6 +1126,7 @@ int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_o
 int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* host_metrics)
 {
     if (!n || batch < 1 || row0 < 0 || !host_metrics) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
     if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");

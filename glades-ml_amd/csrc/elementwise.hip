@@ -1,5 +1,6 @@
-// HBM-bound kernels of the canonical path: output delta / loss / metrics, fused SGD update,
-// bias update, precision conversion, transposition, per-row e4m3 quantisation.
+// HBM-bound kernels of the canonical path: output delta / loss / metrics, bias updates of the bf16
+// path, precision conversion, transposition, per-row e4m3 quantisation.  (The weight updates live in
+// the weight-gradient GEMMs' epilogues.)
 
 #include "ghip_internal.h"
 

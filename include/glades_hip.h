@@ -128,7 +128,10 @@ int ghip_net_get_params(ghip_net* net, int layer, float* host_W, float* host_bia
  *                 (ML/State/edge.cpp:54-101), which survive from one epoch into the next.
  * canonical mode: a = weight momentum (previous update) sizes[layer+1] x sizes[layer],
  *                 b = bias momentum sizes[layer+1].
- * Either pointer may be NULL.  ghip_net_set_params clears this state: set the parameters first. */
+ * Either pointer may be NULL.  ghip_net_set_params clears this state: set the parameters first.
+ * Exact mode: the windows' lengths are implied for a network that has never run with dropout (every
+ * edge of a layer holds the same number of entries); one that has carries them separately, see
+ * ghip_net_get_dropout_state. */
 int ghip_net_get_state(ghip_net* net, int layer, float* host_a, float* host_b);
 int ghip_net_set_state(ghip_net* net, int layer, const float* host_a, const float* host_b);
 
