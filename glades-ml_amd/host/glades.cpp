@@ -1205,6 +1205,7 @@ bool MetaNetwork::runGroup(DataInput* d, int runType)
     }
     for (size_t i = 0; i < subnets.size(); ++i) {
         if (!subnets[i]->prepare(d)) return false;
+        subnets[i]->resetGraphs();
         subnets[i]->running = true;
         act.push_back(subnets[i]);
     }
@@ -1223,6 +1224,7 @@ bool MetaNetwork::runGroup(DataInput* d, int runType)
         for (size_t i = 0; i < act.size(); ++i) {
             NNetwork* n = act[i];
             if (ran[i] <= 0) { n->running = false; continue; }
+            for (int e = 0; e < ran[i]; ++e) n->learningCurve.push_back(ms[i * chunk + e].accuracy);
             n->afterEpochs(&ms[i * chunk + ran[i] - 1], ran[i], runType);
             const bool done = !n->running || n->terminator.triggered(time(NULL), n->epochs, n->overallTotalAccuracy) || runType == NNetwork::RUN_TEST;
             if (done) n->running = false;

@@ -464,7 +464,9 @@ public:
     // un-vendored GTable::stratify and then passes the WHOLE DataInput to every subnet all the same;
     // this does what that code does, without the unused split.)
     float crossValidate(DataInput* newDataInput);
-    // one kernel launch for all subnets where they allow it (see glades.cpp); false = not applicable
+    // one kernel launch for all subnets where they allow it (see glades.cpp); false = not applicable.
+    // Subnets trained this way keep their metrics, learning curve and weights; getResults() (the last
+    // row's predictions) stays empty, since the grouped launch returns no predictions.
     bool runGroup(DataInput*, int runType);
     std::string getName() const { return name; }
     void setName(const std::string& v) { name = v; }
