@@ -8,6 +8,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -76,6 +77,9 @@ struct ghip_net {
     int ex_drop_in_lds = 0;
     ExactPointers* exMulti = nullptr;  // pointer list of a launch over several networks (held by the first one)
     int exMultiCap = 0;
+    ghip_metrics* exMultiMetrics = nullptr;  // results of such a launch, all networks side by side: one copy back
+    int* exMultiEpochs = nullptr;
+    size_t exMultiMetricsCap = 0;
     int* cm = nullptr;              // confusion counters (both modes), n_out x n_out
     float* exClass = nullptr;       // exact mode: 5 floats per epoch of the last call
     int exClassCap = 0, exClassRan = 0;
@@ -643,7 +647,7 @@ int ghip_net_destroy(ghip_net* n)
     dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf);
     dfree(n->exW); dfree(n->exSum); dfree(n->exLast); dfree(n->exBias); dfree(n->exPreds);
     dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass); dfree(n->exMulti);
-    dfree(n->exMasks); dfree(n->exCnt); dfree(n->exErr);
+    dfree(n->exMasks); dfree(n->exCnt); dfree(n->exErr); dfree(n->exMultiMetrics); dfree(n->exMultiEpochs);
     for (int l = 0; l < GHIP_MAX_LAYERS; ++l) {
         dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]);
         dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
@@ -889,10 +893,10 @@ int ghip_net_set_dataset_device(ghip_net* n, const float* dev_X, const float* de
 }
 
 // buffers of one network for a call of n_epochs epochs; fills ptr
-static int exact_prepare(ghip_net* n, int n_epochs, bool want_preds, ExactPointers* ptr)
+static int exact_prepare(ghip_net* n, int n_epochs, bool want_preds, bool own_metrics, ExactPointers* ptr)
 {
     const int nout = n->spec.sizes[n->L];
-    if (n_epochs > n->exMetricsCap) {
+    if (own_metrics && n_epochs > n->exMetricsCap) {
         HIP_TRY(hipStreamSynchronize(n->stream));
         dfree(n->exMetrics);
         TRY(dalloc(&n->exMetrics, (size_t)n_epochs));
@@ -937,7 +941,7 @@ int ghip_net_run_epochs_exact(ghip_net* n, int n_epochs, int train, float stop_a
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     const int nout = n->spec.sizes[n->L];
     ExactLaunch e = n->ex;
-    TRY(exact_prepare(n, n_epochs, host_preds != nullptr, &e.ptr));
+    TRY(exact_prepare(n, n_epochs, host_preds != nullptr, true, &e.ptr));
     e.X = n->dX; e.Y = n->dY; e.n_rows = n->n_rows;
     e.n_epochs = n_epochs; e.train = train ? 1 : 0; e.stop_accuracy = stop_accuracy;
     size_t lds = n->ex_lds;
@@ -970,11 +974,15 @@ int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epoc
     if (!nets || count < 1 || n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
     HIP_TRY(hipSetDevice(g_device));
     ghip_net* lead = nets[0];
+    {
+        std::vector<const ghip_net*> sorted(nets, nets + count);
+        std::sort(sorted.begin(), sorted.end());
+        for (int k = 1; k < count; ++k)
+            if (sorted[k] && sorted[k] == sorted[k - 1]) return fail(GHIP_EINVAL, "a network appears twice in the list");
+    }
     for (int k = 0; k < count; ++k) {
         ghip_net* n = nets[k];
         if (!n) return fail(GHIP_EINVAL, "network %d is NULL", k);
-        for (int j = 0; j < k; ++j)
-            if (nets[j] == n) return fail(GHIP_EINVAL, "network %d appears twice", k);
         if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "network %d is not in exact mode", k);
         if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "network %d has no dataset", k);
         // one launch = one architecture, one schedule, one table: everything but the parameters is shared
@@ -982,15 +990,26 @@ int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epoc
         if (n->n_rows != lead->n_rows) return fail(GHIP_EINVAL, "network %d has a table of another length", k);
     }
     std::vector<ExactPointers> list(count);
-    for (int k = 0; k < count; ++k) {
-        TRY(exact_prepare(nets[k], n_epochs, false, &list[k]));
-        if (nets[k] != lead) HIP_TRY(hipStreamSynchronize(nets[k]->stream));  // its earlier work is done before lead's stream touches its arrays
-    }
+    for (int k = 0; k < count; ++k) TRY(exact_prepare(nets[k], n_epochs, false, false, &list[k]));
+    // every network's earlier work (on its own stream) is done before lead's stream touches its arrays
+    if (count > 1) HIP_TRY(hipDeviceSynchronize());
     if (count > lead->exMultiCap) {
         HIP_TRY(hipStreamSynchronize(lead->stream));
-        dfree(lead->exMulti);
+        dfree(lead->exMulti); dfree(lead->exMultiEpochs);
         TRY(dalloc(&lead->exMulti, (size_t)count));
+        TRY(dalloc(&lead->exMultiEpochs, (size_t)count));
         lead->exMultiCap = count;
+    }
+    if ((size_t)count * n_epochs > lead->exMultiMetricsCap) {
+        HIP_TRY(hipStreamSynchronize(lead->stream));
+        dfree(lead->exMultiMetrics);
+        TRY(dalloc(&lead->exMultiMetrics, (size_t)count * n_epochs));
+        lead->exMultiMetricsCap = (size_t)count * n_epochs;
+    }
+    // every network writes its results into its slot of one array: two copies back instead of two per network
+    for (int k = 0; k < count; ++k) {
+        list[k].metrics = (float*)(lead->exMultiMetrics + (size_t)k * n_epochs);
+        list[k].epochs_run = lead->exMultiEpochs + k;
     }
     HIP_TRY(hipMemcpyAsync(lead->exMulti, list.data(), sizeof(ExactPointers) * count, hipMemcpyHostToDevice, lead->stream));
     ExactLaunch e = lead->ex;
@@ -1016,14 +1035,17 @@ int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epoc
     }
     LAUNCH(lead, any_drop ? "exact_epochs_multi_dropout" : "exact_epochs_multi",
            ghip_launch_exact(e, lead->exMulti, count, lead->ex_threads, lds, lead->stream));
+    std::vector<int> ran(count);
+    std::vector<ghip_metrics> all(host_metrics ? (size_t)count * n_epochs : 0);
+    HIP_TRY(hipMemcpyAsync(ran.data(), lead->exMultiEpochs, sizeof(int) * count, hipMemcpyDeviceToHost, lead->stream));
+    if (host_metrics)
+        HIP_TRY(hipMemcpyAsync(all.data(), lead->exMultiMetrics, sizeof(ghip_metrics) * all.size(), hipMemcpyDeviceToHost, lead->stream));
     HIP_TRY(hipStreamSynchronize(lead->stream));
     for (int k = 0; k < count; ++k) {
-        int ran = 0;
-        HIP_TRY(hipMemcpy(&ran, nets[k]->exEpochs, sizeof(int), hipMemcpyDeviceToHost));
-        if (epochs_run) epochs_run[k] = ran;
-        nets[k]->exClassRan = list[k].class_metrics ? ran : 0;
-        if (host_metrics && ran > 0)
-            HIP_TRY(hipMemcpy(host_metrics + (size_t)k * n_epochs, nets[k]->exMetrics, sizeof(ghip_metrics) * ran, hipMemcpyDeviceToHost));
+        if (epochs_run) epochs_run[k] = ran[k];
+        nets[k]->exClassRan = list[k].class_metrics ? ran[k] : 0;
+        if (host_metrics && ran[k] > 0)
+            memcpy(host_metrics + (size_t)k * n_epochs, all.data() + (size_t)k * n_epochs, sizeof(ghip_metrics) * ran[k]);
     }
     return 0;
 }

@@ -52,6 +52,10 @@ class Metrics(C.Structure):
     _fields_ = [("loss", C.c_float), ("accuracy", C.c_float), ("correct", C.c_int64)]
 
 
+METRICS_DTYPE = np.dtype([("loss", "<f4"), ("accuracy", "<f4"), ("correct", "<i8")])  # Metrics as a numpy record
+assert METRICS_DTYPE.itemsize == C.sizeof(Metrics)
+
+
 class ClassMetrics(C.Structure):
     _fields_ = [("accuracy", C.c_float), ("precision", C.c_float), ("recall", C.c_float),
                 ("specificity", C.c_float), ("f1", C.c_float)]
@@ -337,9 +341,8 @@ def run_epochs_exact_multi(nets, n_epochs, train=True, stop_accuracy=0.0):
     lib = load()
     k = len(nets)
     handles = (C.c_void_p * k)(*[n.h for n in nets])
-    ms = (Metrics * (k * n_epochs))()
-    ran = (C.c_int * k)()
+    ms = np.zeros((k, n_epochs), dtype=METRICS_DTYPE)
+    ran = np.zeros(k, dtype=np.int32)
     _check(lib.ghip_net_run_epochs_exact_multi(C.cast(handles, C.c_void_p), k, n_epochs, 1 if train else 0, float(stop_accuracy),
-                                               C.cast(ms, C.c_void_p), C.cast(ran, C.c_void_p)))
-    return [[(ms[j * n_epochs + e].loss, ms[j * n_epochs + e].accuracy, ms[j * n_epochs + e].correct) for e in range(ran[j])]
-            for j in range(k)]
+                                               _ptr(ms), _ptr(ran)))
+    return [ms[j, :ran[j]].tolist() for j in range(k)]
