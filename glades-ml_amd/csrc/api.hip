@@ -90,6 +90,8 @@ struct ghip_net {
     float* vb[GHIP_MAX_LAYERS] = {};
     float* act[GHIP_MAX_LAYERS + 1] = {};
     float* dlt[GHIP_MAX_LAYERS + 1] = {};
+    double* narrowMetrics = nullptr;  // and the loss / accuracy / correct sums per chunk
+    float* narrowPart = nullptr;  // fp32 canonical, output layer at most 16 wide: partial gradient sums per chunk of rows
     float* stageX = nullptr;
     int cap_batch = 0;
     // metrics of a batch: three banks of 4 doubles.  A metrics launch adds into bank accBank^1 and
@@ -318,7 +320,7 @@ void free_batch_buffers(ghip_net* n)
         if (l > 0) dfree(n->H[l]);
         dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]); dfree(n->csum[l]);
     }
-    dfree(n->stageX); dfree(n->logits);
+    dfree(n->stageX); dfree(n->logits); dfree(n->narrowPart); dfree(n->narrowMetrics);
     dfree(n->Aq[0]); dfree(n->Aq[1]); dfree(n->ascale[0]); dfree(n->ascale[1]);
     dfree(n->amax_bits); dfree(n->Hq); dfree(n->out8);
     n->cap_batch = 0;
@@ -338,6 +340,12 @@ int reserve_batch(ghip_net* n, int B)
         for (int l = 1; l <= L; ++l) {
             TRY(dalloc(&n->act[l], (size_t)B * s.sizes[l]));
             TRY(dalloc(&n->dlt[l], (size_t)B * s.sizes[l]));
+        }
+        if (ghip_narrow_out_ok(s.sizes[L], s.sizes[L - 1])) {
+            // any batch up to B splits into at most this many chunks of rows (ghip_narrow_out_chunks)
+            const int chunks = (B + 3) / 4 < 128 ? (B + 3) / 4 : 128;
+            TRY(dalloc(&n->narrowPart, (size_t)chunks * s.sizes[L] * s.sizes[L - 1]));
+            TRY(dalloc(&n->narrowMetrics, (size_t)chunks * 4));
         }
     } else if (s.dtype == GHIP_BF16) {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
@@ -386,11 +394,11 @@ int out_act(const ghip_net_spec& s, int l, float* param)
 }
 
 // ---- canonical fp32 ----
-int forward_f32(ghip_net* n, const float* X, int B)
+int forward_f32(ghip_net* n, const float* X, int B, int layers)
 {
     const ghip_net_spec& s = n->spec;
     const float* in = X;
-    for (int l = 0; l < s.n_layers; ++l) {
+    for (int l = 0; l < layers; ++l) {
         GemmF32Args g;
         memset(&g, 0, sizeof(g));
         g.A = in; g.B = n->W[l]; g.C = n->act[l + 1];
@@ -399,13 +407,21 @@ int forward_f32(ghip_net* n, const float* X, int B)
         g.epilogue = EPI_BIAS_ACT; g.bias = n->b[l];
         g.act = out_act(s, l, &g.act_param);
         g.alpha = 1.0f;
-        LAUNCH(n, "gemm_f32_forward", ghip_gemm_f32(g, n->stream));
+        if (l == s.n_layers - 1 && ghip_narrow_out_ok(g.N, g.K) && ((uintptr_t)in % 16) == 0) {
+            NarrowOutArgs a;
+            memset(&a, 0, sizeof(a));
+            a.H = in; a.W = n->W[l]; a.B = B; a.ni = g.K; a.no = g.N;
+            a.bias = n->b[l]; a.P = n->act[l + 1]; a.act = g.act; a.act_param = g.act_param;
+            LAUNCH(n, "narrow_out_forward", ghip_narrow_forward(a, n->stream));
+        } else
+            LAUNCH(n, "gemm_f32_forward", ghip_gemm_f32(g, n->stream));
         in = n->act[l + 1];
     }
     return 0;
 }
 
-int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* Dbf, int B)
+// arguments of the output-delta step of one batch; moves on to the other bank of accumulators
+DeltaArgs delta_args(ghip_net* n, float* P, const float* Y, float* D, uint16_t* Dbf, int B)
 {
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
@@ -417,8 +433,14 @@ int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
     a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost;
     a.acc = n->dAcc + 4 * bank; a.acc_clear = n->dAcc + 4 * (bank ^ 1);
     a.cm = n->cm;
-    LAUNCH(n, "output_delta", ghip_output_delta(a, n->stream));
     n->accBank = bank;
+    return a;
+}
+
+int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* Dbf, int B)
+{
+    const DeltaArgs a = delta_args(n, P, Y, D, Dbf, B);
+    LAUNCH(n, "output_delta", ghip_output_delta(a, n->stream));
     return 0;
 }
 
@@ -428,12 +450,33 @@ int step_f32(ghip_net* n, int64_t row0, int B)
     const int L = s.n_layers;
     const float* X = n->dX + row0 * s.sizes[0];
     const float* Y = n->dY + row0 * s.sizes[L];
-    TRY(forward_f32(n, X, B));
-    TRY(output_delta_f32(n, n->act[L], Y, n->dlt[L], nullptr, B));
+    // an output layer of a few units: its forward, the output delta and its backward are one launch
+    const bool narrow = n->narrowPart && ((uintptr_t)(L == 1 ? X : n->act[L - 1]) % 16) == 0;
+    TRY(forward_f32(n, X, B, narrow ? L - 1 : L));
+    if (!narrow) TRY(output_delta_f32(n, n->act[L], Y, n->dlt[L], nullptr, B));
     for (int l = L - 1; l >= 0; --l) {
         const int ni = s.sizes[l], no = s.sizes[l + 1];
         const float* Ain = (l == 0) ? X : n->act[l];
         GemmF32Args g;
+        if (l == L - 1 && narrow) {
+            // the launch leaves the outputs, the metrics, the deltas of this layer and of the layer below
+            // and the gradient's partial sums; a second small kernel adds those up and updates
+            NarrowOutArgs a;
+            memset(&a, 0, sizeof(a));
+            a.H = Ain; a.W = n->W[l]; a.B = B; a.ni = ni; a.no = no;
+            a.bias = n->b[l]; a.P = n->act[l + 1]; a.act = out_act(s, l, &a.act_param);
+            a.D = n->dlt[l + 1]; a.E = (l > 0) ? n->dlt[l] : nullptr;
+            if (l > 0) { a.act_below = s.act[l - 1]; a.act_below_param = s.act_param[l - 1]; }
+            a.part = n->narrowPart;
+            ghip_narrow_out_chunks(B, &a.chunks, &a.rows_per_chunk);
+            a.Wm = n->W[l]; a.V = n->vW[l]; a.lr = s.lr[l]; a.mom = s.mom[l]; a.wd1 = s.wd1[l]; a.wd2 = s.wd2[l];
+            a.alpha = 1.0f / (float)B; a.bias_w = n->b[l]; a.bias_v = n->vb[l];
+            const DeltaArgs da = delta_args(n, n->act[L], Y, n->dlt[L], nullptr, B);
+            a.metric_part = n->narrowMetrics; a.metric_acc = da.acc;
+            LAUNCH(n, "narrow_out_train", ghip_narrow_train(a, da, n->stream));
+            LAUNCH(n, "narrow_out_update", ghip_narrow_update(a, n->stream));
+            continue;
+        }
         if (l > 0) {  // back-prop with the pre-update weights: E = D W, times f'(a_l)
             memset(&g, 0, sizeof(g));
             g.A = n->dlt[l + 1]; g.lda = no; g.a_kmajor = 0;
@@ -1079,7 +1122,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
     if (s.dtype == GHIP_F32) {
-        TRY(forward_f32(n, dev_X32, batch));
+        TRY(forward_f32(n, dev_X32, batch, n->spec.n_layers));
         if (s.act[L - 1] == GHIP_SOFTMAX) {
             DeltaArgs a;
             memset(&a, 0, sizeof(a));
@@ -1157,7 +1200,7 @@ int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* h
     TRY(reserve_batch(n, batch));
     const int L = s.n_layers;
     float* P = nullptr;
-    if (s.dtype == GHIP_F32) { TRY(forward_f32(n, n->dX + row0 * s.sizes[0], batch)); P = n->act[L]; }
+    if (s.dtype == GHIP_F32) { TRY(forward_f32(n, n->dX + row0 * s.sizes[0], batch, L)); P = n->act[L]; }
     else if (s.dtype == GHIP_BF16) { TRY(refresh_shadows(n)); TRY(forward_bf16(n, n->Xbf + row0 * s.sizes[0], batch)); P = n->logits; }
     else { TRY(forward_fp8(n, n->Xbf + row0 * s.sizes[0], batch, n->out8)); P = n->out8; }
     TRY(output_delta_f32(n, P, n->dY + row0 * s.sizes[L], nullptr, nullptr, batch));

@@ -3,6 +3,7 @@
 // the weight-gradient GEMMs' epilogues.)
 
 #include "ghip_internal.h"
+#include "delta_row.h"
 
 namespace {
 
@@ -46,6 +47,11 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
     for (int rr = 0; rr < kRowsPerWave; ++rr) {
         const int b = row0 + rr;
         if (b >= a.B) break;
+        if constexpr (kRegs == 1) {  // a row of at most 64 outputs, one per lane
+            ghip_delta_row64(a, b, lane, (lane < a.n) ? a.P[(long long)b * a.ldp + lane] : -3.0e38f, ghip_delta_target(a, b, lane),
+                             loss, accs, corr);
+            continue;
+        }
         float* p = a.P + (long long)b * a.ldp;
         const float* y = a.Y ? a.Y + (long long)b * a.ldy : nullptr;
         float reg[kRegs > 0 ? kRegs : 1];

@@ -280,6 +280,27 @@ struct GemmF32Args {
 };
 hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s);
 
+// ---------------------------------------------------------------- narrow fp32 output layer (narrow_out.hip)
+// The products of a layer with at most 16 outputs as streams over its input activations H [B][ni]
+// (ni a multiple of 4, rows 16-byte aligned) instead of padded GEMM tiles.
+struct NarrowOutArgs {
+    const float* H; const float* W; int B, ni, no;
+    // forward: P [B][no] = squash(H W^T + bias)
+    const float* bias; float* P; int act; float act_param;
+    // backward: D [B][no] deltas of this layer; E [B][ni] = (D W) .* f'(H) or NULL (no layer below);
+    // part [chunks][no][ni] receives the gradient summed over each chunk of rows_per_chunk rows
+    const float* D; float* E; int act_below; float act_below_param;
+    float* part; int chunks, rows_per_chunk;
+    // metric_part [chunks][4] doubles: loss / accuracy / correct sums of each chunk, written by ghip_narrow_train;
+    // ghip_narrow_update adds them (in chunk order) to metric_acc[0..2]
+    double* metric_part; double* metric_acc;
+    // update: G = sum of the chunks; the EPI_SGD step on Wm / V [no][ni] and on bias_w / bias_v [no] (may be NULL)
+    float* Wm; float* V; float lr, mom, wd1, wd2, alpha; float* bias_w; float* bias_v;
+};
+bool ghip_narrow_out_ok(int no, int ni);
+void ghip_narrow_out_chunks(int B, int* chunks, int* rows_per_chunk);
+hipError_t ghip_narrow_forward(const NarrowOutArgs& a, hipStream_t s);
+
 // softmax / output delta / metrics for fp32 logits-or-activations P[B][n] against Y[B][n].
 // If act == SOFTMAX, P holds pre-softmax logits and is overwritten with probabilities.
 // D (fp32, may be NULL) receives dL/dz; Dbf/DbfT (bf16 [B][n] and [n][B], may be NULL) too.
@@ -294,6 +315,10 @@ struct DeltaArgs {
     int store_p;   // write the activated outputs (softmax probabilities) back into P
 };
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s);
+// forward of the narrow output layer, output delta / loss / metrics (as ghip_output_delta; da.P = a.P,
+// da.D = the deltas a.D reads) and backward in one launch; ghip_narrow_update finishes the step
+hipError_t ghip_narrow_train(const NarrowOutArgs& a, const DeltaArgs& da, hipStream_t s);
+hipError_t ghip_narrow_update(const NarrowOutArgs& a, hipStream_t s);
 
 hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s);
 hipError_t ghip_fill_f64(double* p, long long n, double v, hipStream_t s);

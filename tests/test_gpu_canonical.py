@@ -35,6 +35,13 @@ CASES = [
     ("cfg2_shape_tanh_mse", [32, 64, 64, 1], [po.TANH, po.TANH, po.LINEAR], [0, 0, 1.0], po.REGRESSION, 256),
     ("one_row", [5, 4, 3], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 1),
     ("leaky_sigmoidp_kl", [9, 11, 7, 3], [po.LEAKY, po.TANHP, po.SIGMOID], [0.05, 0.1, 0], po.KL, 12),
+    # output layers of at most 16 units on rows of a multiple of 4 floats take the streaming kernels
+    # instead of GEMM tiles (the cases above with 33, 9 and 7 inputs to the last layer do not)
+    ("narrow_16_out_chunks_of_8_rows", [40, 256, 16], [po.RELU, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 1000),
+    ("narrow_single_layer", [64, 5], [po.SIGMOID], [0], po.CLASSIFICATION, 37),
+    ("narrow_8_out_leaky_below", [12, 36, 8], [po.LEAKY, po.LINEAR], [0.05, 1.0], po.REGRESSION, 130),
+    ("narrow_2_out_wide_rows", [20, 1100, 2], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 64),
+    ("wide_output_gemm", [24, 32, 20], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 64),
 ]
 
 
