@@ -91,6 +91,7 @@ struct ghip_net {
     float* act[GHIP_MAX_LAYERS + 1] = {};
     float* dlt[GHIP_MAX_LAYERS + 1] = {};
     double* narrowMetrics = nullptr;  // and the loss / accuracy / correct sums per chunk
+    bool amax_clean = false;        // e4m3 inference: every entry of amax_bits is zero
     float* narrowPart = nullptr;  // fp32 canonical, output layer at most 16 wide: partial gradient sums per chunk of rows
     float* stageX = nullptr;
     int cap_batch = 0;
@@ -367,6 +368,7 @@ int reserve_batch(ghip_net* n, int B)
         TRY(dalloc(&n->ascale[0], (size_t)B));
         TRY(dalloc(&n->ascale[1], (size_t)B));
         TRY(dalloc(&n->amax_bits, (size_t)B));
+        n->amax_clean = false;
         TRY(dalloc(&n->Hq, (size_t)B * maxw));
         TRY(dalloc(&n->out8, (size_t)B * s.sizes[L]));
     }
@@ -567,7 +569,13 @@ int forward_fp8(ghip_net* n, const uint16_t* Xbf, int B, float* dev_out)
     const int L = s.n_layers;
     if (!n->quantized) return fail(GHIP_ESTATE, "call ghip_net_quantize_fp8 first");
     int cur = 0;
-    LAUNCH(n, "quant_rows_e4m3", ghip_quant_rows_e4m3(Xbf, 1, B, s.sizes[0], n->Aq[0], n->ascale[0], nullptr, n->stream));
+    LAUNCH(n, "quant_rows_e4m3", ghip_quant_rows_e4m3(Xbf, 1, B, s.sizes[0], n->Aq[0], n->ascale[0], nullptr, 0, n->stream));
+    // the row maxima start at zero and every re-quantisation puts the entries it has read back to
+    // zero; they are only cleared here after a forward pass that stopped between the two
+    if (!n->amax_clean) {
+        LAUNCH(n, "fill_amax", ghip_fill_u32(n->amax_bits, n->cap_batch, 0u, n->stream));
+        n->amax_clean = true;
+    }
     for (int l = 0; l < L; ++l) {
         GemmLpArgs g;
         memset(&g, 0, sizeof(g));
@@ -575,11 +583,12 @@ int forward_fp8(ghip_net* n, const uint16_t* Xbf, int B, float* dev_out)
         g.fp8 = 1; g.row_scale = n->ascale[cur]; g.col_scale = n->wscale[l];
         g.act = out_act(s, l, &g.act_param);
         if (l < L - 1) {
-            LAUNCH(n, "fill_amax", ghip_fill_u32(n->amax_bits, B, 0u, n->stream));
             g.epilogue = LP_FP8_ACT; g.out = n->Hq; g.row_amax_bits = n->amax_bits;
+            n->amax_clean = false;
             LAUNCH(n, "gemm_fp8_forward", ghip_gemm_lp(g, n->stream));
             LAUNCH(n, "requant_rows_e4m3", ghip_quant_rows_e4m3(n->Hq, 1, B, s.sizes[l + 1], n->Aq[cur ^ 1], n->ascale[cur ^ 1],
-                                                                n->amax_bits, n->stream));
+                                                                n->amax_bits, 1, n->stream));
+            n->amax_clean = true;
             cur ^= 1;
         } else {
             g.epilogue = LP_FP8_F32; g.out = dev_out;
@@ -1258,7 +1267,7 @@ int ghip_net_quantize_fp8(ghip_net* n, float* const* host_scales, uint8_t* const
     const ghip_net_spec& s = n->spec;
     if (!is_canon(n) || s.dtype != GHIP_FP8_INFER) return fail(GHIP_ESTATE, "network was not created with GHIP_FP8_INFER");
     for (int l = 0; l < s.n_layers; ++l)
-        LAUNCH(n, "quant_weights_e4m3", ghip_quant_rows_e4m3(n->W[l], 0, s.sizes[l + 1], s.sizes[l], n->Wq[l], n->wscale[l], nullptr, n->stream));
+        LAUNCH(n, "quant_weights_e4m3", ghip_quant_rows_e4m3(n->W[l], 0, s.sizes[l + 1], s.sizes[l], n->Wq[l], n->wscale[l], nullptr, 0, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
     n->quantized = true;
     for (int l = 0; l < s.n_layers; ++l) {

@@ -364,7 +364,7 @@ bf16_transpose64_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__
 template <typename SrcT>
 __global__ void __launch_bounds__(256)
 quant_rows_kernel(const SrcT* __restrict__ src, int rows, int cols, uint8_t* __restrict__ q,
-                  float* __restrict__ scale, const unsigned int* __restrict__ amax_bits)
+                  float* __restrict__ scale, unsigned int* __restrict__ amax_bits, int consume)
 {
     const int r = blockIdx.x;
     const SrcT* x = src + (long long)r * cols;
@@ -372,6 +372,10 @@ quant_rows_kernel(const SrcT* __restrict__ src, int rows, int cols, uint8_t* __r
     float amax;
     if (amax_bits) {
         amax = __uint_as_float(amax_bits[r]);
+        if (consume) {  // every lane has its copy: the entry goes back to zero for the next producer
+            __syncthreads();
+            if (threadIdx.x == 0) amax_bits[r] = 0u;
+        }
     } else {
         float m = 0.0f;
         for (int c = threadIdx.x; c < cols; c += 256) {
@@ -407,7 +411,7 @@ __device__ __forceinline__ uint32_t e4m3x4(float a, float b, float c, float d)
 }
 __global__ void __launch_bounds__(256)
 quant_rows_bf16x8_kernel(const uint16_t* __restrict__ src, int cols, uint8_t* __restrict__ q,
-                         float* __restrict__ scale, const unsigned int* __restrict__ amax_bits)
+                         float* __restrict__ scale, unsigned int* __restrict__ amax_bits, int consume)
 {
     const int r = blockIdx.x;
     const uint4* x = reinterpret_cast<const uint4*>(src + (long long)r * cols);
@@ -423,6 +427,10 @@ quant_rows_bf16x8_kernel(const uint16_t* __restrict__ src, int cols, uint8_t* __
     float amax;
     if (amax_bits) {
         amax = __uint_as_float(amax_bits[r]);
+        if (consume) {  // every lane has its copy: the entry goes back to zero for the next producer
+            __syncthreads();
+            if (threadIdx.x == 0) amax_bits[r] = 0u;
+        }
     } else {
         // bf16 magnitudes order like their bit patterns
         unsigned int m = 0;
@@ -449,13 +457,25 @@ quant_rows_bf16x8_kernel(const uint16_t* __restrict__ src, int cols, uint8_t* __
     }
     const float sc = (amax > 0.0f) ? __fdiv_rn(amax, 448.0f) : 1.0f;
     if (threadIdx.x == 0) scale[r] = sc;
+    // x / sc for the whole row with the reciprocal taken once: the hardware's approximation refined by
+    // one Newton step, then per element the product, its exact remainder and one correction.  That is
+    // the correctly rounded quotient unless the true one lies within ~2^-20 of a unit in the last
+    // place of a rounding boundary; quotients are at most 448 in magnitude here, so the scaling an IEEE
+    // division needs for its exceptional ranges (8 divisions of a dozen instructions each per 16 bytes
+    // made this kernel bound by arithmetic, not by memory) has nothing to do.
+    float rcp = __frcp_rn(sc);
+    rcp = __fmaf_rn(__fmaf_rn(-sc, rcp, 1.0f), rcp, rcp);
+    auto quot = [&](float xv) {
+        const float q0 = __fmul_rn(xv, rcp);
+        return __fmaf_rn(__fmaf_rn(-q0, sc, xv), rcp, q0);
+    };
     auto conv = [&](const uint4& v) -> uint2 {
         const unsigned int wds[4] = {v.x, v.y, v.z, v.w};
         float f[8];
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            f[2 * j] = __fdiv_rn(__uint_as_float(wds[j] << 16), sc);
-            f[2 * j + 1] = __fdiv_rn(__uint_as_float(wds[j] & 0xffff0000u), sc);
+            f[2 * j] = quot(__uint_as_float(wds[j] << 16));
+            f[2 * j + 1] = quot(__uint_as_float(wds[j] & 0xffff0000u));
         }
         uint2 o;
         o.x = e4m3x4(f[0], f[1], f[2], f[3]);
@@ -551,13 +571,13 @@ hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, in
 }
 
 hipError_t ghip_quant_rows_e4m3(const void* src, int src_is_bf16, int rows, int cols, uint8_t* q,
-                                float* scale, const unsigned int* amax_bits, hipStream_t s)
+                                float* scale, unsigned int* amax_bits, int consume_amax, hipStream_t s)
 {
     if (src_is_bf16 && (cols % 8) == 0 && ((uintptr_t)src % 16) == 0 && ((uintptr_t)q % 8) == 0)
-        hipLaunchKernelGGL(quant_rows_bf16x8_kernel, dim3(rows), dim3(256), 0, s, (const uint16_t*)src, cols, q, scale, amax_bits);
+        hipLaunchKernelGGL(quant_rows_bf16x8_kernel, dim3(rows), dim3(256), 0, s, (const uint16_t*)src, cols, q, scale, amax_bits, consume_amax);
     else if (src_is_bf16)
-        hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, dim3(rows), dim3(256), 0, s, (const uint16_t*)src, rows, cols, q, scale, amax_bits);
+        hipLaunchKernelGGL(quant_rows_kernel<uint16_t>, dim3(rows), dim3(256), 0, s, (const uint16_t*)src, rows, cols, q, scale, amax_bits, consume_amax);
     else
-        hipLaunchKernelGGL(quant_rows_kernel<float>, dim3(rows), dim3(256), 0, s, (const float*)src, rows, cols, q, scale, amax_bits);
+        hipLaunchKernelGGL(quant_rows_kernel<float>, dim3(rows), dim3(256), 0, s, (const float*)src, rows, cols, q, scale, amax_bits, consume_amax);
     return hipGetLastError();
 }

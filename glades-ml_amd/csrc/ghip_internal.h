@@ -373,7 +373,8 @@ hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B,
                                      float mom, hipStream_t s);
 // per-row e4m3 quantisation: src fp32/bf16 [rows][cols]; scale = amax/448 (1 if row is zero).
 // amax_bits: if non-NULL the row amax is taken from there (uint bits of a non-negative float)
-// instead of being reduced from the row.
+// instead of being reduced from the row; with consume_amax the entry is set back to zero once read
+// (ready for the next GEMM epilogue's atomic maxima).
 hipError_t ghip_quant_rows_e4m3(const void* src, int src_is_bf16, int rows, int cols, uint8_t* q,
-                                float* scale, const unsigned int* amax_bits, hipStream_t s);
+                                float* scale, unsigned int* amax_bits, int consume_amax, hipStream_t s);
 hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream_t s);
