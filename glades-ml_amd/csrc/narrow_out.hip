@@ -315,7 +315,9 @@ __global__ void __launch_bounds__(64 * UPD_GROUPS) narrow_update_kernel(NarrowOu
 
 bool ghip_narrow_out_ok(int no, int ni)
 {
-    return no >= 1 && no <= kMaxOut && ni >= 4 && (ni % 4) == 0;
+    // rows longer than 8192 stay with the GEMM path: a chunk of rows is walked by 4 wavefronts only, and
+    // the partial sums (up to 128 chunks x no x ni floats) would grow past 64 MB
+    return no >= 1 && no <= kMaxOut && ni >= 4 && ni <= 8192 && (ni % 4) == 0;
 }
 
 static_assert(8 * UPD_GROUPS == 128, "narrow_update_kernel reads at most 8 chunks per lane");

@@ -42,6 +42,7 @@ CASES = [
     ("narrow_8_out_leaky_below", [12, 36, 8], [po.LEAKY, po.LINEAR], [0.05, 1.0], po.REGRESSION, 130),
     ("narrow_2_out_wide_rows", [20, 1100, 2], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 64),
     ("wide_output_gemm", [24, 32, 20], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 64),
+    ("cfg3_full_shape", [784, 1024, 1024, 10], [po.RELU, po.RELU, po.SOFTMAX], [0, 0, 0], po.CLASSIFICATION, 512),
 ]
 
 
@@ -65,10 +66,14 @@ def test_training_steps_match_cpu(name, sizes, acts, params, cost, B):
         assert abs(mg.loss - mo.loss) <= 1e-4 * abs(mo.loss) + 1e-6, (s, mg.loss, mo.loss)
         assert abs(mg.accuracy - mo.accuracy) <= 1e-4 * abs(mo.accuracy) + 1e-4
         assert mg.correct == mo.correct, s
+    # The L1 decay term wd1 * sign(W) jumps by 2 * lr * wd1 = 1e-5 when a weight that sits within
+    # rounding distance of zero lands on the other side; among a million weights a few dozen do, and
+    # the momentum carries the jump on.  The full-shape case allows for that, the small ones do not need it.
+    atol = 3e-5 if name == "cfg3_full_shape" else 2e-6
     for l in range(len(sizes) - 1):
         Wo, bo = o.get_params(l)
         Wg, bg = g.get_params(l)
-        np.testing.assert_allclose(Wg, Wo, rtol=1e-4, atol=2e-6)
+        np.testing.assert_allclose(Wg, Wo, rtol=1e-4, atol=atol)
         np.testing.assert_allclose(bg, bo, rtol=1e-4, atol=2e-6)
     Xt = rng.standard_normal((23, sizes[0])).astype(np.float32)
     po_out, pg_out = o.forward(Xt), g.forward(Xt)
