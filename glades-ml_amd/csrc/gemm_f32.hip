@@ -168,7 +168,8 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
         // slab kt+2 (requested during iteration kt-1) into the buffer slab kt-1 has left
         stage(As + nxt * SLAB, sa_, AKM, t);
         stage(Bs + nxt * SLAB, sb_, BKM, t);
-        __syncthreads();
+        // the wavefronts meet over LDS only (__syncthreads() would also drain the global loads just requested)
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
     for (int kt = 0; kt < nk; kt += 2) {
         iteration(kt, fa0, fb0, fa1, fb1);
