@@ -651,20 +651,23 @@ int ghip_init(int device_ordinal)
 
 int ghip_gmath_eval(int fn, int kind, float param, const float* host_a, const float* host_b, float* host_out, int64_t n)
 {
-    if (fn < 0 || fn > 3 || !host_a || !host_out || n < 0 || (fn >= 2 && !host_b)) return fail(GHIP_EINVAL, "bad arguments");
+    if (fn < 0 || fn > 4 || !host_a || !host_out || n < 0 || (fn >= 2 && !host_b)) return fail(GHIP_EINVAL, "bad arguments");
     if (fn <= 1 && (kind < GHIP_TANH || kind > GHIP_STEP)) return fail(GHIP_EINVAL, "unknown activation %d", kind);
-    if (fn >= 2 && (kind < GHIP_REGRESSION || kind > GHIP_KL)) return fail(GHIP_EINVAL, "unknown cost %d", kind);
+    if ((fn == 2 || fn == 3) && (kind < GHIP_REGRESSION || kind > GHIP_KL)) return fail(GHIP_EINVAL, "unknown cost %d", kind);
+    if (fn == 4 && (kind < 0 || kind > 2 || !(param >= 0.0f && param <= 1.0e6f))) return fail(GHIP_EINVAL, "bias chain: kind 0..2, rounds 0..1e6");
+    const size_t bn = (fn == 4) ? (size_t)n * 64 : (size_t)n;  // floats of host_b
     if (n == 0) return 0;
     if (g_device < 0) TRY(ghip_init(0));
     HIP_TRY(hipSetDevice(g_device));
     float *a = nullptr, *b = nullptr, *o = nullptr;
     int rc = dalloc(&a, (size_t)n);
     if (rc == 0) rc = dalloc(&o, (size_t)n);
-    if (rc == 0 && fn >= 2) rc = dalloc(&b, (size_t)n);
+    if (rc == 0 && fn >= 2) rc = dalloc(&b, bn);
     hipError_t e = hipSuccess;
     if (rc == 0) e = hipMemcpy(a, host_a, (size_t)n * 4, hipMemcpyHostToDevice);
-    if (rc == 0 && e == hipSuccess && b) e = hipMemcpy(b, host_b, (size_t)n * 4, hipMemcpyHostToDevice);
-    if (rc == 0 && e == hipSuccess) e = ghip_launch_gmath_eval(fn, kind, param, a, b, o, n, 0);
+    if (rc == 0 && e == hipSuccess && b) e = hipMemcpy(b, host_b, bn * 4, hipMemcpyHostToDevice);
+    if (rc == 0 && e == hipSuccess)
+        e = (fn == 4) ? ghip_launch_bias_chain_eval(kind, (int)param, a, b, o, n, 0) : ghip_launch_gmath_eval(fn, kind, param, a, b, o, n, 0);
     if (rc == 0 && e == hipSuccess) e = hipMemcpy(host_out, o, (size_t)n * 4, hipMemcpyDeviceToHost);
     dfree(a); dfree(b); dfree(o);
     if (rc != 0) return rc;

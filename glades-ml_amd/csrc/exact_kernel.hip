@@ -55,6 +55,61 @@ __device__ __forceinline__ float bias_chain(float b, const float* bs, int no, in
     return b;
 }
 
+// The same chain without walking it, where that is provably the same.  While the bias stays in one
+// binade [2^e, 2^(e+1)) its values are integers M in units of u = 2^(e-23), and b - x rounds to
+// M - rn(x / u): the rounding does not depend on M unless x / u lies exactly half-way between two
+// integers (a tie goes to the even M).  So with q_k = rn(x_k / u) the chain is integer arithmetic,
+// which is associative: after n_in rounds M has moved by n_in * sum(q_k), and every intermediate
+// value is i * sum(q) + (a prefix sum of q).  One wavefront, lane k holding x_k, checks with a
+// prefix scan that no intermediate value leaves the binade (a value below 2^23 + 1 units could have
+// been rounded on the finer grid underneath) and that there is no tie; if so it returns the result
+// of the n_in * n_out subtractions exactly, otherwise it says no and the caller walks the chain.
+// All 64 lanes call with the same b and n_in; xk is this lane's lr*d (0 past the last output).
+__device__ __forceinline__ bool bias_chain_grid(float b, float xk, int ni, int lane, float* result)
+{
+    const unsigned int bits = __float_as_uint(b);
+    const int ex = (int)((bits >> 23) & 0xffu);
+    if (ex == 0 || ex == 255) return false;                 // zero, subnormal, infinite, not a number
+    const long long m0 = (long long)((bits & 0x7fffffu) | 0x800000u);
+    const bool neg = (bits >> 31) != 0;
+    const long long M0 = neg ? -m0 : m0;
+    // 1 / u = 2^(150 - ex) and u, as doubles: scaling a float by them is exact
+    const double inv_u = __longlong_as_double((long long)(1023 + 150 - ex) << 52);
+    const double u = __longlong_as_double((long long)(1023 - 150 + ex) << 52);
+    const double t = (double)xk * inv_u;
+    const bool in_range = fabs(t) <= 16777216.0;            // false for NaN too; 64 of them stay below 2^31
+    const double q = __builtin_rint(t);                     // to nearest, ties to even
+    const bool tie = fabs(t - q) == 0.5;
+    if (__ballot(!in_range || tie) != 0ull) return false;
+    const int qi = (int)q;
+    // inclusive prefix sums over the lanes, their extremes, and the total
+    int pre = qi;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const int up = __shfl_up(pre, o, 64);
+        if (lane >= o) pre += up;
+    }
+    int pmin = pre, pmax = pre;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const int a = __shfl_xor(pmin, o, 64), c = __shfl_xor(pmax, o, 64);
+        pmin = a < pmin ? a : pmin;
+        pmax = c > pmax ? c : pmax;
+    }
+    const long long Q = (long long)__shfl(pre, 63, 64);
+    const long long span = (long long)(ni - 1) * Q;
+    const long long lo = (span < 0 ? span : 0) + pmin;      // smallest and largest amount subtracted so far,
+    const long long hi = (span > 0 ? span : 0) + pmax;      // over every step of every round
+    const long long Mlo = M0 - hi, Mhi = M0 - lo;
+    const long long kMin = (1ll << 23) + 1, kMax = (1ll << 24) - 1;
+    const bool inside = neg ? (Mhi <= -kMin && Mlo >= -kMax) : (Mlo >= kMin && Mhi <= kMax);
+    if (!inside) return false;
+    *result = (float)((double)(M0 - (long long)ni * Q) * u);
+    return true;
+}
+// chains shorter than this are walked: the check costs about as much as a few hundred subtractions
+constexpr int kGridChainMin = 512;
+
 // Barrier between the phases of a row.  With the state in LDS the phases only hand LDS data to one
 // another, so the wait covers LDS operations alone: __syncthreads() would also wait for the global
 // loads that prefetch the next row and for the confusion-matrix atomics, a trip to memory per row.
@@ -342,7 +397,14 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                             for (int i = 0; i < ni; ++i) nv += mi[i] ? 0 : 1;
                             mk = mo;
                         }
-                        if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
+                        bool walked = false;
+                        if (p.bias_mode == GHIP_BIAS_SEQUENTIAL && no <= 64 && nv > 0 && (long long)nv * no >= kGridChainMin) {
+                            const int k = tid & 63;
+                            const float xk = (k < no && !(mk && mk[k])) ? bs[k] : 0.0f;
+                            walked = bias_chain_grid(b, xk, nv, k, &b);
+                        }
+                        if (walked) {
+                        } else if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
                             if (no <= 4) b = bias_chain<4>(b, bs, no, nv, mk);
                             else if (no <= 8) b = bias_chain<8>(b, bs, no, nv, mk);
                             else if (no <= 16) b = bias_chain<16>(b, bs, no, nv, mk);
@@ -454,7 +516,33 @@ __global__ void gmath_eval_kernel(int fn, int kind, float param, const float* __
     }
 }
 
+// The bias chain of one row for n independent cases, a wavefront each: a[k] the bias before,
+// b[64*k .. 64*k+63] the lr*d of the outputs (zeros past the last), n_in rounds.
+// kind 0: one subtraction after the other; 1: the integer-grid shortcut where it applies, else the walk;
+// 2: 1.0 where the shortcut applies, else 0.0.
+__global__ void __launch_bounds__(256) bias_chain_eval_kernel(int kind, int ni, const float* __restrict__ a,
+                                                              const float* __restrict__ b, float* __restrict__ out, long long n)
+{
+    const int lane = threadIdx.x & 63;
+    const long long k = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (k >= n) return;
+    float v = a[k];
+    const float xk = b[k * 64 + lane];
+    float fast = 0.0f;
+    const bool ok = kind != 0 && ni > 0 && bias_chain_grid(v, xk, ni, lane, &fast);
+    if (kind == 2) v = ok ? 1.0f : 0.0f;
+    else if (ok) v = fast;
+    else v = bias_chain<64>(v, b + k * 64, 64, ni);
+    if (lane == 0) out[k] = v;
+}
+
 }  // namespace
+
+hipError_t ghip_launch_bias_chain_eval(int kind, int ni, const float* a, const float* b, float* out, long long n, hipStream_t s)
+{
+    hipLaunchKernelGGL(bias_chain_eval_kernel, dim3((unsigned)((n + 3) / 4)), dim3(256), 0, s, kind, ni, a, b, out, n);
+    return hipGetLastError();
+}
 
 hipError_t ghip_launch_gmath_eval(int fn, int kind, float param, const float* a, const float* b, float* out, long long n,
                                   hipStream_t s)

@@ -249,6 +249,7 @@ hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_mult
 size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropout);
 // fn 0 squash(a; kind, param), 1 activationErrDer(a; kind, param), 2 outputNodeCost(expected a, predicted b; cost
 // kind, dataSize param), 3 costErrDer(expected a, predicted b; cost kind): device arrays of n floats
+hipError_t ghip_launch_bias_chain_eval(int kind, int ni, const float* a, const float* b, float* out, long long n, hipStream_t s);
 hipError_t ghip_launch_gmath_eval(int fn, int kind, float param, const float* a, const float* b, float* out, long long n,
                                   hipStream_t s);
 

@@ -150,9 +150,13 @@ def _ptr(a):
 
 def gmath_eval(fn, kind, a, b=None, param=0.0):
     """fn 0 squash, 1 activationErrDer, 2 outputNodeCost(expected a, predicted b, dataSize param),
-    3 costErrDer(expected a, predicted b), element by element on the device with exact mode's arithmetic."""
+    3 costErrDer(expected a, predicted b), element by element on the device with exact mode's arithmetic;
+    4 the layer bias after one row's chain of subtractions (a: bias before, b: [cases][64] lr*d, param:
+    rounds; kind 0 walked, 1 as the kernel does it, 2 whether the integer shortcut applies)."""
     a = np.ascontiguousarray(a, np.float32)
     b = None if b is None else np.ascontiguousarray(b, np.float32)
+    if b is not None and b.size != a.size * (64 if fn == 4 else 1):
+        raise ValueError("b has %d elements for %d cases" % (b.size, a.size))
     out = np.empty_like(a)
     _check(load().ghip_gmath_eval(int(fn), int(kind), float(param), _ptr(a), _ptr(b), _ptr(out), a.size))
     return out

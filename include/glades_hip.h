@@ -102,6 +102,12 @@ int ghip_init(int device_ordinal);
  * fn 1  GMath::activationErrDer(a[k], kind, param)             ML/GMath/gmath.cpp:182-245
  * fn 2  GMath::outputNodeCost(expected a[k], predicted b[k], dataSize = param, cost kind)  :272-321
  * fn 3  GMath::costErrDer(expected a[k], predicted b[k], cost kind)                        :323-353
+ * fn 4  the scalar layer bias after one row's back-propagation (ML/Networks/network.cpp:654-656: bias -= lr*d[o]
+ *       once per (input, output) pair, outputs innermost): a[k] the bias before, host_b[64*k .. 64*k+63] the
+ *       lr*d of up to 64 outputs (zeros past the last), param = number of input nodes (rounds).
+ *       kind 0 walks the n_in * 64 subtractions; kind 1 is what the persistent kernel does: an
+ *       integer-arithmetic shortcut where it is provably the same float, else the walk; kind 2 returns
+ *       1.0 where that shortcut applies, else 0.0
  * kind is an activation id for fn 0/1 and a cost id for fn 2/3; host_b is unused for fn 0/1.  tanh, exp
  * and log return the floats of the reference platform's C library (GNU libc 2.35), bit for bit. */
 int ghip_gmath_eval(int fn, int kind, float param, const float* host_a, const float* host_b, float* host_out, int64_t n);
