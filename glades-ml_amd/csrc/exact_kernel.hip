@@ -55,6 +55,47 @@ __device__ __forceinline__ float bias_chain(float b, const float* bs, int no, in
     return b;
 }
 
+// A sequential fold z = step(z, x[i*xs], y[i*ys]) for i = 0..n-1 in that order, with the operands
+// fetched from LDS eight steps at a time and one block ahead of the arithmetic (two register sets,
+// alternating: a copy from one to the other would wait for the block just asked for).  Left to
+// itself the compiler asks for two operands, waits for them, uses them, and asks for the next two: an
+// LDS round trip per pair of steps, which is what a row's dot products then consist of.
+template <typename Step>
+__device__ __forceinline__ float fold8(float z, const float* x, int xs, const float* y, int ys, int n, Step step)
+{
+    constexpr int B = 8;
+    const int nb = n / B;
+    float xa[B], ya[B], xb[B], yb[B];
+    auto fetch = [&](float (&xv)[B], float (&yv)[B], int blk) {
+        const float* px = x + blk * B * xs;
+        const float* py = y + blk * B * ys;
+#pragma unroll
+        for (int j = 0; j < B; ++j) { xv[j] = px[j * xs]; yv[j] = py[j * ys]; }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto run = [&](const float (&xv)[B], const float (&yv)[B]) {
+#pragma unroll
+        for (int j = 0; j < B; ++j) z = step(z, xv[j], yv[j]);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    if (nb > 0) {
+        int b = 0;
+        fetch(xa, ya, 0);
+        // nothing else is outstanding when the loop is entered: with a scalar load possibly in flight
+        // (they return out of order) the first wait inside the loop would be for everything
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+        while (b + 2 < nb) {
+            fetch(xb, yb, b + 1); run(xa, ya);
+            fetch(xa, ya, b + 2); run(xb, yb);
+            b += 2;
+        }
+        if (nb - b == 2) { fetch(xb, yb, b + 1); run(xa, ya); run(xb, yb); }
+        else run(xa, ya);
+    }
+    for (int i = nb * B; i < n; ++i) z = step(z, x[i * xs], y[i * ys]);
+    return z;
+}
+
 // The same chain without walking it, where that is provably the same.  While the bias stays in one
 // binade [2^e, 2^(e+1)) its values are integers M in units of u = 2^(e-23), and b - x rounds to
 // M - rn(x / u): the rounding does not depend on M unless x / u lies exactly half-way between two
@@ -270,8 +311,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         for (int i = 0; i < ni; ++i)
                             z = __fadd_rn(z, (vo && !mi[i]) ? __fmul_rn(w[i], ain[i]) : 0.0f);
                     } else {
-#pragma unroll 16
-                        for (int i = 0; i < ni; ++i) z = __fadd_rn(z, __fmul_rn(w[i], ain[i]));
+                        z = fold8(z, w, 1, ain, 1, ni, [](float acc, float wv, float av) { return __fadd_rn(acc, __fmul_rn(wv, av)); });
                     }
                     if (l != 0) z = __fadd_rn(z, bl);
                     const float a = ghip_squash<true>(z, act, par, (const uint64_t*)sT);
@@ -357,6 +397,43 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         // an edge that sat out an applying row can hold more than mb pending deltas;
                         // applyDeltas reads the first mb only (node.cpp:299-301), so their number is kept
                         int* Cl = (kDrop && p.mb > 1) ? own.wcnt + p.woff[l] : nullptr;
+                        if (!kDrop) {
+                            // four edges of a lane at a time: their operands are asked for together
+                            for (int i = i0; i < ni; i += tw) {
+                                const float a = ain[i];
+                                const float t1 = __fmul_rn(w1, fabsf(a));
+                                const float t2 = __fmul_rn(w2, a);
+                                for (int o = o0; o < no; o += 4 * rpp) {
+                                    float bv[4], lv[4], sv[4], wv[4];
+                                    int kk[4];
+#pragma unroll
+                                    for (int j = 0; j < 4; ++j) {
+                                        const int oj = o + j * rpp;
+                                        const int oc = oj < no ? oj : no - 1;  // past the end: a repeat that is not stored
+                                        kk[j] = oc * ld + i;
+                                        bv[j] = bs[oc]; lv[j] = Ll[kk[j]]; sv[j] = Sl[kk[j]]; wv[j] = Wl[kk[j]];
+                                    }
+                                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                                    for (int j = 0; j < 4; ++j) {
+                                        if (o + j * rpp < no) {
+                                            float dW = __fadd_rn(__fmul_rn(bv[j], a), __fmul_rn(mom, lv[j]));
+                                            dW = __fadd_rn(dW, t1);
+                                            dW = __fadd_rn(dW, t2);
+                                            const float sn = __fadd_rn(sv[j], dW);
+                                            if (apply) {
+                                                Wl[kk[j]] = __fsub_rn(wv[j], __fdiv_rn(sn, fmb));
+                                                Sl[kk[j]] = 0.0f;
+                                                Ll[kk[j]] = 0.0f;
+                                            } else {
+                                                Sl[kk[j]] = sn;
+                                                Ll[kk[j]] = dW;
+                                            }
+                                        }
+                                    }
+                                }
+                            }
+                        } else
                         for (int i = i0; i < ni; i += tw) {
                             if (kDrop && mi[i]) continue;
                             const float a = ain[i];
@@ -445,9 +522,8 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                                 }
                                 sE[p.aoff[l] + i] = e;
                             } else {
-#pragma unroll 16
-                                for (int o = 0; o < no; ++o)
-                                    e = __fadd_rn(e, __fadd_rn(e, __fmul_rn(dl[o], Wl[o * ld + i])));
+                                e = fold8(e, dl, 1, Wl + i, ld, no,
+                                          [](float acc, float dv, float wv) { return __fadd_rn(acc, __fadd_rn(acc, __fmul_rn(dv, wv))); });
                             }
                             // the reference always passes 0.01 here (network.cpp:617-618)
                             float d = __fmul_rn(e, ghip_act_der_ref(ain[i], actp, 0.01f));
