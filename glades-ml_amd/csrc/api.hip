@@ -91,6 +91,7 @@ struct ghip_net {
     float* act[GHIP_MAX_LAYERS + 1] = {};
     float* dlt[GHIP_MAX_LAYERS + 1] = {};
     double* narrowMetrics = nullptr;  // and the loss / accuracy / correct sums per chunk
+    bool passAcc = false;           // canonical mode: a pass over the table is running (ghip_net_run_epoch_canonical)
     bool amax_clean = false;        // e4m3 inference: every entry of amax_bits is zero
     float* narrowPart = nullptr;  // fp32 canonical, output layer at most 16 wide: partial gradient sums per chunk of rows
     float* stageX = nullptr;
@@ -309,8 +310,8 @@ int setup_canon(ghip_net* n)
             TRY(dalloc(&n->wscale[l], (size_t)s.sizes[l + 1]));
         }
     }
-    TRY(dalloc(&n->dAcc, 12));
-    HIP_TRY(hipMemsetAsync(n->dAcc, 0, 12 * sizeof(double), n->stream));
+    TRY(dalloc(&n->dAcc, 16));  // two alternating banks per step, one for softmax-only launches, one per pass over the table
+    HIP_TRY(hipMemsetAsync(n->dAcc, 0, 16 * sizeof(double), n->stream));
     return 0;
 }
 
@@ -435,6 +436,10 @@ DeltaArgs delta_args(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
     a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost;
     a.acc = n->dAcc + 4 * bank; a.acc_clear = n->dAcc + 4 * (bank ^ 1);
     a.cm = n->cm;
+    if (n->passAcc) {  // a whole pass adds up in its own bank, which nothing clears on the way
+        a.acc = n->dAcc + 12; a.acc_clear = nullptr;
+        return a;
+    }
     n->accBank = bank;
     return a;
 }
@@ -1119,6 +1124,48 @@ int ghip_net_train_step(ghip_net* n, int64_t row0, int batch, ghip_metrics* host
     if (n->spec.dtype == GHIP_F32) TRY(step_f32(n, row0, batch));
     else TRY(step_bf16(n, row0, batch));
     if (host_metrics) return fetch_metrics(n, host_metrics);
+    return 0;
+}
+
+int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics* host_metrics)
+{
+    if (!n || batch < 1 || !host_metrics) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    if (train && s.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "fp8 networks are inference only");
+    const int64_t N = n->n_rows;
+    if (batch > N) batch = (int)N;
+    if (s.dtype != GHIP_F32 && ((batch % 256) || (N % batch) % 256))
+        return fail(GHIP_EINVAL, "bf16/fp8 paths need batches that are multiples of 256 (the last one, %lld rows, too)", (long long)(N % batch));
+    TRY(reserve_batch(n, batch));
+    if (s.dtype == GHIP_BF16) TRY(refresh_shadows(n));
+    LAUNCH(n, "fill_pass_metrics", ghip_fill_f64(n->dAcc + 12, 4, 0.0, n->stream));
+    n->passAcc = true;
+    int rc = 0;
+    for (int64_t r0 = 0; r0 < N && rc == 0; r0 += batch) {
+        const int b = (int)(N - r0 < batch ? N - r0 : batch);
+        if (train) {
+            rc = (s.dtype == GHIP_F32) ? step_f32(n, r0, b) : step_bf16(n, r0, b);
+        } else {
+            float* P = nullptr;
+            if (s.dtype == GHIP_F32) { rc = forward_f32(n, n->dX + r0 * s.sizes[0], b, L); P = n->act[L]; }
+            else if (s.dtype == GHIP_BF16) { rc = forward_bf16(n, n->Xbf + r0 * s.sizes[0], b); P = n->logits; }
+            else { rc = forward_fp8(n, n->Xbf + r0 * s.sizes[0], b, n->out8); P = n->out8; }
+            if (rc == 0) rc = output_delta_f32(n, P, n->dY + r0 * s.sizes[L], nullptr, nullptr, b);
+        }
+        n->last_batch = b;
+    }
+    n->passAcc = false;
+    if (rc != 0) return rc;
+    double acc[4];
+    HIP_TRY(hipMemcpyAsync(acc, n->dAcc + 12, sizeof(acc), hipMemcpyDeviceToHost, n->stream));
+    HIP_TRY(hipStreamSynchronize(n->stream));
+    host_metrics->loss = (float)(acc[0] / (double)N);
+    host_metrics->accuracy = (float)(acc[1] / ((double)N * s.sizes[L]));
+    host_metrics->correct = (int64_t)(acc[2] + 0.5);
     return 0;
 }
 

@@ -1157,19 +1157,12 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             if (confusionMatrix.size() > 0) ghip_net_confusion_reset(dev);  // network.cpp:183-185
             // canonical mode: batches [k*mb, (k+1)*mb), the last one averaged over its true size
             const int mb = minibatchSize > 0 ? minibatchSize : (int)nRows;
-            double loss = 0.0, acc = 0.0;
-            int64_t correct = 0;
-            bool failed = false;
-            for (unsigned int r0 = 0; r0 < nRows && !failed; r0 += mb) {
-                const int b = (int)((nRows - r0) < (unsigned int)mb ? (nRows - r0) : (unsigned int)mb);
-                ghip_metrics m;
-                int rc = (runType == RUN_TRAIN) ? ghip_net_train_step(dev, r0, b, &m) : ghip_net_eval_resident(dev, r0, b, &m);
-                if (rc != 0) { lastError = ghip_last_error(); failed = true; break; }
-                loss += (double)m.loss * b; acc += (double)m.accuracy * b; correct += m.correct;
-            }
-            if (failed) break;
+            // every step of the pass is enqueued back to back; the device adds up the metrics
             ghip_metrics last;
-            last.loss = (float)(loss / nRows); last.accuracy = (float)(acc / nRows); last.correct = correct;
+            if (ghip_net_run_epoch_canonical(dev, mb, runType == RUN_TRAIN ? 1 : 0, &last) != 0) {
+                lastError = ghip_last_error();
+                break;
+            }
             learningCurve.push_back(last.accuracy);
             afterEpochs(&last, 1, runType);
         }

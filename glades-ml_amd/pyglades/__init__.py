@@ -23,7 +23,7 @@ EXPORTS = [
     "ghip_net_get_state", "ghip_net_set_state",
     "ghip_net_set_dropout_masks", "ghip_net_get_dropout_state", "ghip_net_set_dropout_state",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
-    "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
+    "ghip_net_run_epoch_canonical", "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
     "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
     "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
@@ -92,6 +92,7 @@ def load():
             "ghip_net_set_dataset_device": (i, [vp, vp, vp, i64]),
             "ghip_net_run_epochs_exact": (i, [vp, i, i, f, vp, C.POINTER(i), vp]),
             "ghip_net_run_epochs_exact_multi": (i, [vp, i, i, i, f, vp, vp]),
+            "ghip_net_run_epoch_canonical": (i, [vp, i, i, C.POINTER(Metrics)]),
             "ghip_net_train_step": (i, [vp, i64, i, vp]),
             "ghip_net_last_metrics": (i, [vp, C.POINTER(Metrics)]),
             "ghip_net_forward": (i, [vp, vp, i, vp]),
@@ -286,6 +287,12 @@ class Net:
             return m
         _check(self.lib.ghip_net_train_step(self.h, row0, batch, None))
         return None
+
+    def run_epoch_canonical(self, batch, train=True):
+        """One pass over the resident table in batches of `batch`; one synchronisation at the end."""
+        m = Metrics()
+        _check(self.lib.ghip_net_run_epoch_canonical(self.h, int(batch), 1 if train else 0, C.byref(m)))
+        return m
 
     def last_metrics(self):
         m = Metrics()

@@ -189,6 +189,16 @@ int ghip_net_run_epochs_exact(ghip_net* net, int n_epochs, int train, float stop
 int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epochs, int train, float stop_accuracy,
                                     ghip_metrics* host_metrics, int* epochs_run);
 
+/* Canonical mode: one pass over the whole resident table in batches [k*batch, (k+1)*batch) (the last
+ * one shorter and averaged over its true size), every step enqueued back to back and one
+ * synchronisation at the end: the body of NNetwork::run's epoch loop (ML/Networks/network.cpp:171-191:
+ * SGDHelper for every row, then the epoch's error and accuracy) for batched training.  train != 0:
+ * forward, backward and update per batch; 0: forward and metrics only.  host_metrics: the pass's mean
+ * per-sample loss, its accuracy and its count of rows whose predicted class is the expected one
+ * (accumulated on the device over all batches).  ghip_net_last_metrics afterwards still refers to the
+ * last ghip_net_train_step. */
+int ghip_net_run_epoch_canonical(ghip_net* net, int batch, int train, ghip_metrics* host_metrics);
+
 /* Canonical mode: one training step (forward, backward, update) on rows [row0, row0+batch) of
  * the resident table.  host_metrics may be NULL (then the call does not synchronise). */
 int ghip_net_train_step(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);

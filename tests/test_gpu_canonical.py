@@ -116,3 +116,43 @@ def test_last_partial_batch_and_bounds():
     with pytest.raises(pg.GladesHipError):
         g.train_step(20, 6)
     g.close()
+
+
+@pytest.mark.parametrize("sizes,acts,B,N", [
+    ([20, 64, 10], [po.RELU, po.SOFTMAX], 32, 200),      # narrow output layer, last batch of 8 rows
+    ([12, 40, 24], [po.TANH, po.SOFTMAX], 50, 150),      # output layer on the GEMM path, whole batches
+])
+def test_one_pass_call_equals_the_steps_one_by_one(sizes, acts, B, N):
+    """ghip_net_run_epoch_canonical enqueues the same launches as a loop of ghip_net_train_step: the
+    parameters end bit-identical, and the pass's metrics are the row-weighted means of the steps'."""
+    o, a, rng = build_pair(sizes, acts, [0, 0], po.CLASSIFICATION, 0.05, 0.9, 1e-4, 1e-3, 21)
+    _, b, _ = build_pair(sizes, acts, [0, 0], po.CLASSIFICATION, 0.05, 0.9, 1e-4, 1e-3, 21)
+    X = rng.standard_normal((N, sizes[0])).astype(np.float32)
+    Y = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], N)]
+    a.set_dataset(X, Y); b.set_dataset(X, Y)
+    for epoch in range(3):
+        loss = acc = 0.0
+        correct = 0
+        for r0 in range(0, N, B):
+            n = min(B, N - r0)
+            m = a.train_step(r0, n)
+            mo = o.step(X[r0:r0 + n], Y[r0:r0 + n])
+            loss += m.loss * n; acc += m.accuracy * n; correct += m.correct
+            assert abs(m.loss - mo.loss) <= 1e-4 * abs(mo.loss) + 1e-6
+        mp = b.run_epoch_canonical(B)
+        assert abs(mp.loss - loss / N) <= 1e-5 * abs(loss / N)
+        assert abs(mp.accuracy - acc / N) <= 1e-5 * abs(acc / N)
+        assert mp.correct == correct
+    for l in range(len(sizes) - 1):
+        Wa, ba = a.get_params(l)
+        Wb, bb = b.get_params(l)
+        assert np.array_equal(Wa, Wb) and np.array_equal(ba, bb), l
+    # a pass without training: the metrics of the current parameters, which it leaves alone
+    ev = b.run_epoch_canonical(B, train=False)
+    again = b.run_epoch_canonical(B, train=False)
+    assert (ev.loss, ev.accuracy, ev.correct) == (again.loss, again.accuracy, again.correct)
+    assert np.array_equal(b.get_params(0)[0], a.get_params(0)[0])
+    want = o.forward(X)
+    got_correct = int((want.argmax(1) == Y.argmax(1)).sum())
+    assert ev.correct == got_correct
+    a.close(); b.close()
