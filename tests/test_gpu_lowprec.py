@@ -193,3 +193,48 @@ def test_full_size_forward_is_row_wise(kind):
     assert np.array_equal(g.forward(X[perm]), out[perm])
     assert not np.any(g.forward(np.zeros((256, sizes[0]), np.float32)))
     g.close()
+
+
+def test_bf16_and_e4m3_passes_over_the_table():
+    """ghip_net_run_epoch_canonical on the low-precision paths: a bf16 training pass leaves the
+    parameters of the same steps taken one by one, an e4m3 pass only evaluates, and batches that are
+    not multiples of 256 (the last one included) are refused."""
+    import pyglades as pg
+    rng = np.random.default_rng(8)
+    sizes, acts = [256, 512, 256], [po.RELU, po.SOFTMAX]
+    B, N = 256, 768
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * np.sqrt(2.0 / sizes[l])).astype(np.float32) for l in range(2)]
+    X = rng.standard_normal((N, 256)).astype(np.float32)
+    Y = teacher_labels(rng, X, 256)
+    kw = dict(lr=0.02, mom=0.9, wd2=1e-4, cost=po.CLASSIFICATION, mode=pg.MODE_CANONICAL)
+    a = pg.Net(pg.make_spec(sizes, acts, dtype=pg.BF16, **kw))
+    b = pg.Net(pg.make_spec(sizes, acts, dtype=pg.BF16, **kw))
+    for n in (a, b):
+        for l in range(2):
+            n.set_params(l, Ws[l])
+        n.set_dataset(X, Y)
+    loss = correct = 0
+    for r0 in range(0, N, B):
+        m = a.train_step(r0, B)
+        loss += m.loss * B; correct += m.correct
+    mp = b.run_epoch_canonical(B)
+    assert abs(mp.loss - loss / N) <= 1e-5 * abs(loss / N) and mp.correct == correct
+    for l in range(2):
+        assert np.array_equal(a.get_params(l)[0], b.get_params(l)[0]), l
+    q = pg.Net(pg.make_spec(sizes, acts, dtype=pg.FP8_INFER, **kw))
+    for l in range(2):
+        q.set_params(l, Ws[l])
+    q.set_dataset(X, Y)
+    q.quantize_fp8(want=False)
+    ev = q.run_epoch_canonical(B, train=False)
+    assert 0 <= ev.correct <= N and np.isfinite(ev.loss)
+    with pytest.raises(pg.GladesHipError):
+        q.run_epoch_canonical(B, train=True)        # inference only
+    short = pg.Net(pg.make_spec(sizes, acts, dtype=pg.BF16, **kw))
+    short.set_dataset(X[:700], Y[:700])
+    with pytest.raises(pg.GladesHipError):
+        short.run_epoch_canonical(B)                # the last batch would have 188 rows
+    with pytest.raises(pg.GladesHipError):
+        a.run_epoch_canonical(0)
+    for n in (a, b, q, short):
+        n.close()
