@@ -458,6 +458,10 @@ bool NNetwork::save(const std::string& path) const { return skeleton ? skeleton-
 // file: "GLCK" u32 version, i32 mode, i32 dtype, i32 epochs, i32 nLayers, i32 sizes[nLayers+1],
 //       u32 tableBytes, table text (the NNInfo CSV), then per layer: W, u32 biasLen, bias, u32 aLen, a, u32 bLen, b,
 //       and from version 2 on u32 cLen, window lengths (i32), u32 eLen, node error accumulators (exact mode; else 0, 0)
+// fwrite / fread of n elements that leave an empty array's (possibly null) pointer alone
+static size_t put(const void* p, size_t size, size_t n, FILE* f) { return n ? fwrite(p, size, n, f) : 0; }
+static size_t get(void* p, size_t size, size_t n, FILE* f) { return n ? fread(p, size, n, f) : 0; }
+
 bool NNetwork::saveCheckpoint(const std::string& path)
 {
     if (!skeleton || !dev) { lastError = "nothing to checkpoint: the network has not run"; return false; }
@@ -481,8 +485,8 @@ bool NNetwork::saveCheckpoint(const std::string& path)
     if (!f) { lastError = "cannot write " + path; return false; }
     const uint32_t version = 2, tb = (uint32_t)table.size();
     const int32_t head[4] = {mode, dtype, epochs, L};
-    fwrite("GLCK", 1, 4, f); fwrite(&version, 4, 1, f); fwrite(head, 4, 4, f); fwrite(sizes.data(), 4, sizes.size(), f);
-    fwrite(&tb, 4, 1, f); fwrite(table.data(), 1, table.size(), f);
+    fwrite("GLCK", 1, 4, f); fwrite(&version, 4, 1, f); fwrite(head, 4, 4, f); put(sizes.data(), 4, sizes.size(), f);
+    fwrite(&tb, 4, 1, f); put(table.data(), 1, table.size(), f);
     bool ok = true;
     for (int l = 0; l < L && ok; ++l) {
         const size_t cnt = (size_t)sizes[l] * sizes[l + 1];
@@ -491,16 +495,16 @@ bool NNetwork::saveCheckpoint(const std::string& path)
         std::vector<float> W(cnt), b(bl), sa(al), sb(sl);
         ok = ghip_net_get_params(dev, l, W.data(), b.data(), (int)bl) == 0 && ghip_net_get_state(dev, l, sa.data(), sb.data()) == 0;
         if (!ok) { lastError = ghip_last_error(); break; }
-        fwrite(W.data(), 4, cnt, f);
-        fwrite(&bl, 4, 1, f); fwrite(b.data(), 4, bl, f);
-        fwrite(&al, 4, 1, f); fwrite(sa.data(), 4, al, f);
-        fwrite(&sl, 4, 1, f); fwrite(sb.data(), 4, sl, f);
+        put(W.data(), 4, cnt, f);
+        fwrite(&bl, 4, 1, f); put(b.data(), 4, bl, f);
+        fwrite(&al, 4, 1, f); put(sa.data(), 4, al, f);
+        fwrite(&sl, 4, 1, f); put(sb.data(), 4, sl, f);
         const uint32_t cl = mode == MODE_EXACT ? (uint32_t)cnt : 0u, el = mode == MODE_EXACT ? (uint32_t)sizes[l + 1] : 0u;
         std::vector<int32_t> wc(cl);
         std::vector<float> ed(el);
         if (cl && ghip_net_get_dropout_state(dev, l, wc.data(), ed.data()) != 0) { ok = false; lastError = ghip_last_error(); break; }
-        fwrite(&cl, 4, 1, f); fwrite(wc.data(), 4, cl, f);
-        fwrite(&el, 4, 1, f); fwrite(ed.data(), 4, el, f);
+        fwrite(&cl, 4, 1, f); put(wc.data(), 4, cl, f);
+        fwrite(&el, 4, 1, f); put(ed.data(), 4, el, f);
     }
     fclose(f);
     return ok;
@@ -519,24 +523,24 @@ bool NNetwork::loadCheckpoint(const std::string& path)
     std::string table;
     if (ok) {
         sizes.resize(head[3] + 1);
-        ok = fread(sizes.data(), 4, sizes.size(), f) == sizes.size() && fread(&tb, 4, 1, f) == 1 && tb < (1u << 20);
+        ok = get(sizes.data(), 4, sizes.size(), f) == sizes.size() && fread(&tb, 4, 1, f) == 1 && tb < (1u << 20);
     }
-    if (ok) { table.resize(tb); ok = fread(&table[0], 1, tb, f) == tb; }
+    if (ok) { table.resize(tb); ok = get(tb ? &table[0] : nullptr, 1, tb, f) == tb; }
     std::vector<std::vector<float> > W, B, SA, SB, ED;
     std::vector<std::vector<int32_t> > WC;
     for (int l = 0; ok && l < head[3]; ++l) {
         const size_t cnt = (size_t)sizes[l] * sizes[l + 1];
         std::vector<float> w(cnt), b, sa, sb;
         uint32_t n1 = 0;
-        ok = fread(w.data(), 4, cnt, f) == cnt;
-        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { b.resize(n1); ok = fread(b.data(), 4, n1, f) == n1; }
-        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sa.resize(n1); ok = fread(sa.data(), 4, n1, f) == n1; }
-        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sb.resize(n1); ok = fread(sb.data(), 4, n1, f) == n1; }
+        ok = get(w.data(), 4, cnt, f) == cnt;
+        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { b.resize(n1); ok = get(b.data(), 4, n1, f) == n1; }
+        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sa.resize(n1); ok = get(sa.data(), 4, n1, f) == n1; }
+        ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { sb.resize(n1); ok = get(sb.data(), 4, n1, f) == n1; }
         std::vector<int32_t> wc;
         std::vector<float> ed;
         if (version >= 2) {
-            ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { wc.resize(n1); ok = fread(wc.data(), 4, n1, f) == n1; }
-            ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { ed.resize(n1); ok = fread(ed.data(), 4, n1, f) == n1; }
+            ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { wc.resize(n1); ok = get(wc.data(), 4, n1, f) == n1; }
+            ok = ok && fread(&n1, 4, 1, f) == 1 && n1 <= cnt; if (ok) { ed.resize(n1); ok = get(ed.data(), 4, n1, f) == n1; }
         }
         W.push_back(w); B.push_back(b); SA.push_back(sa); SB.push_back(sb); WC.push_back(wc); ED.push_back(ed);
     }
@@ -546,7 +550,7 @@ bool NNetwork::loadCheckpoint(const std::string& path)
     {
         FILE* t = fopen(tmp.c_str(), "wb");
         if (!t) return false;
-        fwrite(table.data(), 1, table.size(), t);
+        put(table.data(), 1, table.size(), t);
         fclose(t);
     }
     const bool loaded = load(tmp);

@@ -21,6 +21,9 @@
 
 #include "glades.h"
 
+// writes a float array; an empty one (whose data() may be null) writes nothing
+static void put(const std::vector<float>& v, FILE* f) { if (!v.empty()) fwrite(v.data(), 4, v.size(), f); }
+
 using namespace glades;
 
 static int do_xavier(int seed, int fi, int no, int act, const char* out)
@@ -30,7 +33,7 @@ static int do_xavier(int seed, int fi, int no, int act, const char* out)
     xavierLayer(fi, no, act, W.data());
     FILE* f = fopen(out, "wb");
     if (!f) return 1;
-    fwrite(W.data(), 4, W.size(), f);
+    put(W, f);
     fclose(f);
     return 0;
 }
@@ -165,8 +168,8 @@ static int do_numberinput(const char* csv, const char* flag, const char* out)
     if (!fo) return 1;
     float head[3] = {(float)di.getTrainSize(), (float)di.getFeatureCount(), (float)di.getOutputCount()};
     fwrite(head, 4, 3, fo);
-    for (unsigned int r = 0; r < di.getTrainSize(); ++r) { std::vector<float> v = di.getTrainRow(r); fwrite(v.data(), 4, v.size(), fo); }
-    for (unsigned int r = 0; r < di.getTrainSize(); ++r) { std::vector<float> v = di.getTrainExpectedRow(r); fwrite(v.data(), 4, v.size(), fo); }
+    for (unsigned int r = 0; r < di.getTrainSize(); ++r) { std::vector<float> v = di.getTrainRow(r); put(v, fo); }
+    for (unsigned int r = 0; r < di.getTrainSize(); ++r) { std::vector<float> v = di.getTrainExpectedRow(r); put(v, fo); }
     fclose(fo);
     for (size_t c = 0; c < di.getOHEMaps().size(); ++c) {
         printf("col %d categorical %d classes", (int)c, (int)di.featureIsCategorical[c]);
@@ -244,16 +247,16 @@ static int train_and_dump(NNetwork& net, DataInput* di, int nl, const char* out)
     if (!fo) return 1;
     float head[6] = {(float)trained, acc, loss, (float)net.getEpochs(), net.getAccuracy(), (float)results.size()};
     fwrite(head, 4, 6, fo);
-    fwrite(results.data(), 4, results.size(), fo);
+    put(results, fo);
     for (int l = 0; l < nl; ++l) {
         std::vector<float> w = net.getWeights(l);
-        fwrite(w.data(), 4, w.size(), fo);
+        put(w, fo);
     }
     for (int l = 0; l < nl; ++l) {
         std::vector<float> b = net.getBias(l);
-        fwrite(b.data(), 4, b.size(), fo);
+        put(b, fo);
     }
-    fwrite(tail.data(), 4, tail.size(), fo);
+    put(tail, fo);
     fclose(fo);
     delete meta;
     return 0;
@@ -384,7 +387,7 @@ static int do_dropout(const char* in, int seed, int e1, int e2, const char* ckpt
     if (!fo) return 1;
     float head[6] = {(float)b.getEpochs(), (float)trained_c, b.getLoss(), train_loss, cn.getAccuracy(), (float)(rand() % 65536)};
     fwrite(head, 4, 6, fo);
-    for (size_t k = 0; k < w.size(); ++k) { fwrite(w[k].data(), 4, w[k].size(), fo); fwrite(bb[k].data(), 4, bb[k].size(), fo); }
+    for (size_t k = 0; k < w.size(); ++k) { put(w[k], fo); put(bb[k], fo); }
     fclose(fo);
     return 0;
 }
@@ -424,8 +427,8 @@ static int do_checkpoint(const char* in, int mode, int e1, int e2, const char* c
     for (int k = 0; k < 2; ++k)
         for (int l = 0; l < c.nl; ++l) {
             std::vector<float> w = nets[k]->getWeights(l), bb = nets[k]->getBias(l);
-            fwrite(w.data(), 4, w.size(), fo);
-            fwrite(bb.data(), 4, bb.size(), fo);
+            put(w, fo);
+            put(bb, fo);
         }
     fclose(fo);
     return 0;
@@ -479,8 +482,8 @@ static int do_meta(const char* in, int mode, int k, int epochs, const char* out)
     if (!fo) return 1;
     float head[4] = {(float)k, (float)secs[0], (float)secs[1], cv};
     fwrite(head, 4, 4, fo);
-    fwrite(losses.data(), 4, losses.size(), fo);
-    for (size_t i = 0; i < keep.size(); ++i) fwrite(keep[i].data(), 4, keep[i].size(), fo);
+    put(losses, fo);
+    for (size_t i = 0; i < keep.size(); ++i) put(keep[i], fo);
     fclose(fo);
     return 0;
 }
