@@ -33,9 +33,9 @@ HBM_PEAK = 8000.0  # GB/s
 # counters sit between L2 and the fabric, so lines re-fetched from the memory-side cache count again.
 # A workload / kernel pair that was not measured reports null.
 MEASURED_TRAFFIC_BYTES = {
-    # mean over the step's 5 launches: 4 x (329294.5 x 2 + 196608) KiB and 1 x (126595.3 x 2 + 49152) KiB
-    ("cfg4", "gemm_bf16_wgrad_sgd"): int((4 * (329294.5 * 2.000 + 196608.0) + (126595.26 * 2.000 + 49152.0)) / 5 * 1024),
-    ("cfg5", "gemm_fp8_forward"): int((789038.85 * 2.000 + 270336.0 * 1.000) * 1024),
+    # mean over the step's 5 launches: 4 x (329199.4 x 2 + 196608) KiB and 1 x (126547.3 x 2 + 49152) KiB
+    ("cfg4", "gemm_bf16_wgrad_sgd"): int((4 * (329199.35 * 2.000 + 196608.0) + (126547.28 * 2.000 + 49152.0)) / 5 * 1024),
+    ("cfg5", "gemm_fp8_forward"): int((789138.46 * 2.000 + 270336.0 * 1.000) * 1024),
 }
 
 WORKLOADS = {
