@@ -42,6 +42,7 @@ CASES = [
     ("narrow_8_out_leaky_below", [12, 36, 8], [po.LEAKY, po.LINEAR], [0.05, 1.0], po.REGRESSION, 130),
     ("narrow_2_out_wide_rows", [20, 1100, 2], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 64),
     ("wide_output_gemm", [24, 32, 20], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 64),
+    ("few_outputs_on_rows_too_long_for_the_streaming_kernels", [16, 8200, 3], [po.TANH, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 32),
     ("cfg3_full_shape", [784, 1024, 1024, 10], [po.RELU, po.RELU, po.SOFTMAX], [0, 0, 0], po.CLASSIFICATION, 512),
 ]
 
