@@ -562,7 +562,9 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
         g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l];
         g.master = n->W[l]; g.mom = n->vW[l];
         g.lr = s.lr[l]; g.momf = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l]; g.gscale = 1.0f / (float)B;
-        LAUNCH(n, "gemm_bf16_wgrad_sgd", ghip_gemm_lp(g, n->stream));
+        // the profile keeps the two tile sizes apart: they are different kernels with different rooflines
+        if (ghip_gemm_lp_tile_m(g.M, g.N) == 128) LAUNCH(n, "gemm_bf16_wgrad_sgd_t128", ghip_gemm_lp(g, n->stream));
+        else LAUNCH(n, "gemm_bf16_wgrad_sgd", ghip_gemm_lp(g, n->stream));
     }
     return 0;
 }
