@@ -108,8 +108,10 @@ template <int V> struct IC { static constexpr int value = V; };
 // `before` MFMAs of the fill's span have been issued before this group; after MFMA number m of
 // the span, loads number ceil(m * NDMA / SPAN) .. ceil((m + 1) * NDMA / SPAN) - 1 go out.  A
 // wavefront that issues its loads back to back stalls on the address unit (16 clocks per load,
-// shared by the 8 wavefronts), and the matrix pipe of its SIMD idles with it.
-template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, typename Dma>
+// shared by the 8 wavefronts), and the matrix pipe of its SIMD idles with it.  With BFIRST the
+// first NDMA / 2 loads (the B half-stage) are the caller's to issue ahead of the span, and only
+// the rest is spread here.
+template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, bool BFIRST, typename Dma>
 __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma)
 {
 #pragma unroll
@@ -128,7 +130,13 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, 
             }
             if constexpr (NDMA > 0) {
                 const int m = BEFORE + mi * NI + ni;
-                const int lo = (m * NDMA + SPAN - 1) / SPAN, hi = ((m + 1) * NDMA + SPAN - 1) / SPAN;
+                // evenly over the span; with BFIRST the caller has issued the B half-stage (the first NDMA / 2
+                // loads) before the stage's first MFMA, and the span carries the A loads only
+                constexpr int NB = NDMA / 2, NA = NDMA - NB, STEP = SPAN / (NA + 1) > 0 ? SPAN / (NA + 1) : 1;
+                static_assert(!BFIRST || SPAN / (NA + 1) > 0, "the span has room for every load");
+                auto before = [](int mm) { return NB + (mm / STEP < NA ? mm / STEP : NA); };
+                const int lo = BFIRST ? before(m) : (m * NDMA + SPAN - 1) / SPAN;
+                const int hi = BFIRST ? ((m + 1 >= SPAN) ? NDMA : before(m + 1)) : ((m + 1) * NDMA + SPAN - 1) / SPAN;
                 if (m < SPAN && hi > lo) {
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -269,6 +277,13 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         if (lane < 8) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
     };
     constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0);  // loads a stage's closing wait leaves in flight
+    // The products of the backward pass find their operands in HBM more often than in the memory-side
+    // cache (the weight gradient's are a forward pass old), and the B half-stage, asked for during the
+    // stage that ends with the wait for it, is the load that arrives late: there it goes out as soon as
+    // the stage begins, ahead of the first MFMA (the earlier the better: after the first four MFMAs
+    // -2.4 % of a training step, ahead of the first another -1 %).  The forward products, whose
+    // operands were written one kernel earlier, run better with every load spread between the MFMAs.
+    constexpr bool kBFirst = !FP8 && (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
     auto stage = [&](auto Pc, int j) {
         constexpr int P = decltype(Pc)::value;
         const unsigned char* const RA = smem + ((2 * P) % NSLOT) * SLOT;
@@ -283,14 +298,20 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         auto none = [](int) {};
         if constexpr (!kDouble) {
             constexpr int SPAN = 2 * G;
-            mma_group<FP8, MI, NI, SPAN, NDMA, 0>(acc, f0, dma);
+            mma_group<FP8, MI, NI, SPAN, NDMA, 0, kBFirst>(acc, f0, dma);
             load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
-            mma_group<FP8, MI, NI, SPAN, NDMA, G>(acc, f0, dma);
+            mma_group<FP8, MI, NI, SPAN, NDMA, G, kBFirst>(acc, f0, dma);
             __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
             load_frags<FP8, MI, NI>(f0, NA, NB, 0, wm, wn, l31, lh);
         } else {
             constexpr int SPAN = (KS - 1) * G;
+            if constexpr (kBFirst) {
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int d = 0; d < PWB; ++d) dma(d);
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 F& cur = (ks & 1) ? f1 : f0;
@@ -304,10 +325,10 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                     load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (ks == 0) mma_group<FP8, MI, NI, SPAN, NDMA, 0>(acc, cur, dma);
-                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, NDMA, G>(acc, cur, dma);
-                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, NDMA, 2 * G>(acc, cur, dma);
-                else mma_group<FP8, MI, NI, 1, 0, 0>(acc, cur, none);
+                if (ks == 0) mma_group<FP8, MI, NI, SPAN, NDMA, 0, kBFirst>(acc, cur, dma);
+                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, NDMA, G, kBFirst>(acc, cur, dma);
+                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, NDMA, 2 * G, kBFirst>(acc, cur, dma);
+                else mma_group<FP8, MI, NI, 1, 0, 0, false>(acc, cur, none);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
