@@ -226,18 +226,26 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;
         lds_direct_16s(gBw + (long long)(jj * 8) * ldb + kb, voffB[jj & 1], smem_u + slot * SLOT + (ws * PWB + jj) * 1024);
     };
+    // X is the operand with two stages of lead, Y the one with one: A and B, except in the 128 x 128-tile
+    // weight gradient, which runs 10 % faster with its B operand (the activations, a forward pass old)
+    // in the place with more lead; the 256 x 256-tile kernels measure the same either way
+    constexpr bool kSwap = !FP8 && EPI == LP_WGRAD_SGD && TM == 128;
+    static_assert(PWA == PWB, "either operand can take either place in the ring");
+    auto dmaX = [&](int slot, int st, int jj) { if constexpr (kSwap) dmaB(slot, st, jj); else dmaA(slot, st, jj); };
+    auto dmaY = [&](int slot, int st, int jj) { if constexpr (kSwap) dmaA(slot, st, jj); else dmaB(slot, st, jj); };
+    constexpr int OA = kSwap ? 1 : 0, OB = kSwap ? 0 : 1;  // places of A and B within a stage's pair of slots
 #pragma unroll
-    for (int jj = 0; jj < PWA; ++jj) dmaA(0, 0, jj);
+    for (int jj = 0; jj < PWA; ++jj) dmaX(0, 0, jj);
 #pragma unroll
-    for (int jj = 0; jj < PWB; ++jj) dmaB(1, 0, jj);
+    for (int jj = 0; jj < PWB; ++jj) dmaY(1, 0, jj);
 #pragma unroll
-    for (int jj = 0; jj < PWA; ++jj) dmaA(2, 1, jj);
+    for (int jj = 0; jj < PWA; ++jj) dmaX(2, 1, jj);
     __builtin_amdgcn_s_waitcnt(0x0F70 | PWA);  // vmcnt(PWA): A0 and B0 have landed
     __builtin_amdgcn_s_barrier();
 
     typedef Frags<FP8, MI, NI> F;
     F f0, f1;
-    load_frags<FP8, MI, NI>(f0, smem, smem + SLOT, 0, wm, wn, l31, lh);
+    load_frags<FP8, MI, NI>(f0, smem + OA * SLOT, smem + OB * SLOT, 0, wm, wn, l31, lh);
 
     // One stage (P = j mod 5 fixes the slots at compile time).  Sub-steps are software pipelined:
     // each one first states that its own fragments (requested one MFMA group earlier) have landed,
@@ -262,19 +270,23 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     constexpr int PF_ARRAYS = (EPI == LP_WGRAD_SGD) ? 2 : 1;
     constexpr int PF_LPR = TN * PF_ES / 128;                     // lines per tile row
     constexpr int PF_PER = TM * PF_LPR;                          // lines per array
-    constexpr int PF_N = PF_ARRAYS * PF_PER / 64;                // stages needed: 64 lines per stage and workgroup
+    // lines a wavefront touches per stage: every line is a request of its own to the address unit that
+    // the operand loads also go through, so wider touches over fewer stages cost more than they save
+    // (16 lanes: the training step 1.6 % slower, 32: 4 %, 64: 26 %)
+    constexpr int PF_LANES = 8;
+    constexpr int PF_N = cmax(PF_ARRAYS * PF_PER / (8 * PF_LANES), 1);    // stages needed: 8 * PF_LANES lines per stage and workgroup
     constexpr int PF_LEAD = 2;
     int pfreg = 0;
     const int pf_j0 = nk - PF_N - PF_LEAD > 0 ? nk - PF_N - PF_LEAD : 0;
     auto touch = [&](int j) {
         int i = j - pf_j0;
         i = i < 0 ? 0 : (i >= PF_N ? PF_N - 1 : i);  // outside the window: repeat a touched line
-        const int line = (i * 8 + ws) * 8 + (lane & 7);
+        const int line = (i * 8 + ws) * PF_LANES + (lane & (PF_LANES - 1));
         const int within = line % PF_PER;
         const unsigned char* base = (EPI == LP_DGRAD) ? (const unsigned char*)g.aux
                                   : (line < PF_PER) ? (const unsigned char*)g.master : (const unsigned char*)g.mom;
         const unsigned char* src = base + ((long long)(bm + within / PF_LPR) * g.N + bn) * PF_ES + (within % PF_LPR) * 128;
-        if (lane < 8) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
+        if (lane < PF_LANES) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
     };
     constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0);  // loads a stage's closing wait leaves in flight
     // The products of the backward pass find their operands in HBM more often than in the memory-side
@@ -286,14 +298,14 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     constexpr bool kBFirst = !FP8 && (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
     auto stage = [&](auto Pc, int j) {
         constexpr int P = decltype(Pc)::value;
-        const unsigned char* const RA = smem + ((2 * P) % NSLOT) * SLOT;
-        const unsigned char* const RB = smem + ((2 * P + 1) % NSLOT) * SLOT;
-        const unsigned char* const NA = smem + ((2 * P + 2) % NSLOT) * SLOT;
-        const unsigned char* const NB = smem + ((2 * P + 3) % NSLOT) * SLOT;
+        const unsigned char* const RA = smem + ((2 * P + OA) % NSLOT) * SLOT;
+        const unsigned char* const RB = smem + ((2 * P + OB) % NSLOT) * SLOT;
+        const unsigned char* const NA = smem + ((2 * P + 2 + OA) % NSLOT) * SLOT;
+        const unsigned char* const NB = smem + ((2 * P + 2 + OB) % NSLOT) * SLOT;
         auto dma = [&](int d) {
-            if (d < PWB) { dmaB((2 * P + 3) % NSLOT, j + 1, d); return; }
+            if (d < PWB) { dmaY((2 * P + 3) % NSLOT, j + 1, d); return; }
             if (kTouch && d == PWB) touch(j);
-            dmaA((2 * P + 4) % NSLOT, j + 2, d - PWB);
+            dmaX((2 * P + 4) % NSLOT, j + 2, d - PWB);
         };
         auto none = [](int) {};
         if constexpr (!kDouble) {
