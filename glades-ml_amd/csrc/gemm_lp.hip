@@ -133,7 +133,7 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, 
                 // evenly over the span; with BFIRST the caller has issued the B half-stage (the first NDMA / 2
                 // loads) before the stage's first MFMA, and the span carries the A loads only
                 constexpr int NB = NDMA / 2, NA = NDMA - NB, STEP = SPAN / (NA + 1) > 0 ? SPAN / (NA + 1) : 1;
-                static_assert(!BFIRST || SPAN / (NA + 1) > 0, "the span has room for every load");
+                static_assert(!BFIRST || SPAN >= NA, "the span has room for every load");
                 auto before = [](int mm) { return NB + (mm / STEP < NA ? mm / STEP : NA); };
                 const int lo = BFIRST ? before(m) : (m * NDMA + SPAN - 1) / SPAN;
                 const int hi = BFIRST ? ((m + 1 >= SPAN) ? NDMA : before(m + 1)) : ((m + 1) * NDMA + SPAN - 1) / SPAN;
@@ -291,11 +291,13 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0);  // loads a stage's closing wait leaves in flight
     // The products of the backward pass find their operands in HBM more often than in the memory-side
     // cache (the weight gradient's are a forward pass old), and the B half-stage, asked for during the
-    // stage that ends with the wait for it, is the load that arrives late: there it goes out as soon as
-    // the stage begins, ahead of the first MFMA (the earlier the better: after the first four MFMAs
-    // -2.4 % of a training step, ahead of the first another -1 %).  The forward products, whose
-    // operands were written one kernel earlier, run better with every load spread between the MFMAs.
-    constexpr bool kBFirst = !FP8 && (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
+    // stage that ends with the wait for it, is the load that arrives late: there it goes out as early
+    // as its slot allows (the earlier the better: after a stage's first four MFMAs -2.4 % of a training
+    // step, ahead of its first another -1 %, right behind the barrier that closes the stage before,
+    // ahead of that stage's last MFMA group, another -0.4 %).  The e4m3 products wait for their operands
+    // more than they compute and gain 7 % from the same order.  The bf16 forward products, whose operands
+    // were written one kernel earlier, run better with every load spread between the MFMAs.
+    constexpr bool kBFirst = FP8 || (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
     auto stage = [&](auto Pc, int j) {
         constexpr int P = decltype(Pc)::value;
         const unsigned char* const RA = smem + ((2 * P + OA) % NSLOT) * SLOT;
@@ -308,6 +310,12 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             dmaX((2 * P + 4) % NSLOT, j + 2, d - PWB);
         };
         auto none = [](int) {};
+        auto next_y = [&]() {  // the next stage's Y loads: their slot is free once this stage's closing barrier is passed
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int d = 0; d < PWB; ++d) dmaY((2 * P + 5) % NSLOT, j + 2, d);
+            __builtin_amdgcn_sched_barrier(0);
+        };
         if constexpr (!kDouble) {
             constexpr int SPAN = 2 * G;
             mma_group<FP8, MI, NI, SPAN, NDMA, 0, kBFirst>(acc, f0, dma);
@@ -315,15 +323,10 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             mma_group<FP8, MI, NI, SPAN, NDMA, G, kBFirst>(acc, f0, dma);
             __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
+            if constexpr (kBFirst) next_y();
             load_frags<FP8, MI, NI>(f0, NA, NB, 0, wm, wn, l31, lh);
         } else {
             constexpr int SPAN = (KS - 1) * G;
-            if constexpr (kBFirst) {
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int d = 0; d < PWB; ++d) dma(d);
-                __builtin_amdgcn_sched_barrier(0);
-            }
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
                 F& cur = (ks & 1) ? f1 : f0;
@@ -334,6 +337,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                 } else {
                     __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
                     __builtin_amdgcn_s_barrier();
+                    if constexpr (kBFirst) next_y();
                     load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -345,6 +349,10 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             }
         }
     };
+    if constexpr (kBFirst) {  // what the first stage's closing wait is for (A1 went out with the ring's first fill)
+#pragma unroll
+        for (int d = 0; d < PWB; ++d) dmaY(3, 1, d);
+    }
     for (int j = 0;;) {
         stage(IC<0>{}, j); if (++j == nk) break;
         stage(IC<1>{}, j); if (++j == nk) break;
