@@ -104,14 +104,12 @@ __device__ __forceinline__ void lds_direct_16s(const unsigned char* sbase, unsig
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 template <int V> struct IC { static constexpr int value = V; };
 
-// MFMAs of one K sub-step with the LDS-direct loads of the running fill spread between them:
-// `before` MFMAs of the fill's span have been issued before this group; after MFMA number m of
-// the span, loads number ceil(m * NDMA / SPAN) .. ceil((m + 1) * NDMA / SPAN) - 1 go out.  A
-// wavefront that issues its loads back to back stalls on the address unit (16 clocks per load,
-// shared by the 8 wavefronts), and the matrix pipe of its SIMD idles with it.  With BFIRST the
-// first NDMA / 2 loads (the B half-stage) are the caller's to issue ahead of the span, and only
-// the rest is spread here.
-template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, bool BFIRST, typename Dma>
+// MFMAs of one K sub-step with NDMA LDS-direct loads of the running fill spread between them:
+// BEFORE MFMAs of the fill's span have been issued before this group; load number i goes out once
+// (i + 1) * STEP MFMAs of the span have, STEP = SPAN / (NDMA + 1).  A wavefront that issues all its
+// loads back to back stalls on the address unit (16 clocks per load, shared by the 8 wavefronts),
+// and the matrix pipe of its SIMD idles with it.
+template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, typename Dma>
 __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma)
 {
 #pragma unroll
@@ -130,13 +128,11 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, 
             }
             if constexpr (NDMA > 0) {
                 const int m = BEFORE + mi * NI + ni;
-                // evenly over the span; with BFIRST the caller has issued the B half-stage (the first NDMA / 2
-                // loads) before the stage's first MFMA, and the span carries the A loads only
-                constexpr int NB = NDMA / 2, NA = NDMA - NB, STEP = SPAN / (NA + 1) > 0 ? SPAN / (NA + 1) : 1;
-                static_assert(!BFIRST || SPAN >= NA, "the span has room for every load");
-                auto before = [](int mm) { return NB + (mm / STEP < NA ? mm / STEP : NA); };
-                const int lo = BFIRST ? before(m) : (m * NDMA + SPAN - 1) / SPAN;
-                const int hi = BFIRST ? ((m + 1 >= SPAN) ? NDMA : before(m + 1)) : ((m + 1) * NDMA + SPAN - 1) / SPAN;
+                constexpr int STEP = SPAN / (NDMA + 1) > 0 ? SPAN / (NDMA + 1) : 1;
+                static_assert(SPAN >= NDMA, "the span has room for every load");
+                auto before = [](int mm) { return mm / STEP < NDMA ? mm / STEP : NDMA; };  // loads out before MFMA mm
+                const int lo = before(m);
+                const int hi = (m + 1 >= SPAN) ? NDMA : before(m + 1);
                 if (m < SPAN && hi > lo) {
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -202,10 +198,10 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     // sequences of 1 KiB slabs of 8 rows, one LDS-direct load each: lane i lands at row i/8,
     // physical chunk i%8 of its slab, so it fetches the logical chunk that the swizzle maps there
     // (every load covers whole 128-byte lines).  A wavefront moves PWA + PWB slabs per stage.
-    // The ring holds the half-stages A0 B0 A1 B1 ... in slots 0 1 2 3 4 0 1 ...: while stage j is
-    // consumed, B(j+1) and then A(j+2) are requested into the two slots stage j-1 has left, so A
-    // has two stages of lead and B one, and the wait that ends stage j leaves the A loads in flight.
-    constexpr int PWA = TM / 64, PWB = TN / 64, NDMA = PWA + PWB;
+    // The ring holds the half-stages A0 B0 A1 B1 ... in slots 0 1 2 3 4 0 1 ...: B(j+1) is requested
+    // as soon as the barrier that ends stage j-1 has freed its slot, A(j+2) while stage j is consumed,
+    // so A has two stages of lead and B one, and the wait that ends stage j leaves the A loads in flight.
+    constexpr int PWA = TM / 64, PWB = TN / 64;
     static_assert(PWA % 2 == 0 && PWB % 2 == 0 && PWA < 8, "slab parity and the vmcnt immediate assume this");
     const int ws = __builtin_amdgcn_readfirstlane(w);
     const unsigned int smem_u = (unsigned int)(uintptr_t)((lptr_t)smem);
@@ -289,15 +285,12 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         if (lane < PF_LANES) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
     };
     constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0);  // loads a stage's closing wait leaves in flight
-    // The products of the backward pass find their operands in HBM more often than in the memory-side
-    // cache (the weight gradient's are a forward pass old), and the B half-stage, asked for during the
-    // stage that ends with the wait for it, is the load that arrives late: there it goes out as early
-    // as its slot allows (the earlier the better: after a stage's first four MFMAs -2.4 % of a training
-    // step, ahead of its first another -1 %, right behind the barrier that closes the stage before,
-    // ahead of that stage's last MFMA group, another -0.4 %).  The e4m3 products wait for their operands
-    // more than they compute and gain 7 % from the same order.  The bf16 forward products, whose operands
-    // were written one kernel earlier, run better with every load spread between the MFMAs.
-    constexpr bool kBFirst = FP8 || (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
+    // The Y half-stage, asked for one stage before the wait for it, is the load that arrives late, and
+    // most of all where the operands come from HBM rather than the memory-side cache (the weight
+    // gradient's are a forward pass old).  So its loads go out as early as their slot allows, back to
+    // back right behind the barrier that closes the stage before (spread over the stage with X's, they
+    // cost the bf16 training step 5 % and the e4m3 products 7 %), and only X's, which have a stage more,
+    // are spread between the MFMAs.
     auto stage = [&](auto Pc, int j) {
         constexpr int P = decltype(Pc)::value;
         const unsigned char* const RA = smem + ((2 * P + OA) % NSLOT) * SLOT;
@@ -305,9 +298,8 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         const unsigned char* const NA = smem + ((2 * P + 2 + OA) % NSLOT) * SLOT;
         const unsigned char* const NB = smem + ((2 * P + 2 + OB) % NSLOT) * SLOT;
         auto dma = [&](int d) {
-            if (d < PWB) { dmaY((2 * P + 3) % NSLOT, j + 1, d); return; }
-            if (kTouch && d == PWB) touch(j);
-            dmaX((2 * P + 4) % NSLOT, j + 2, d - PWB);
+            if (kTouch && d == 0) touch(j);
+            dmaX((2 * P + 4) % NSLOT, j + 2, d);
         };
         auto none = [](int) {};
         auto next_y = [&]() {  // the next stage's Y loads: their slot is free once this stage's closing barrier is passed
@@ -318,12 +310,12 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         };
         if constexpr (!kDouble) {
             constexpr int SPAN = 2 * G;
-            mma_group<FP8, MI, NI, SPAN, NDMA, 0, kBFirst>(acc, f0, dma);
+            mma_group<FP8, MI, NI, SPAN, PWA, 0>(acc, f0, dma);
             load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
-            mma_group<FP8, MI, NI, SPAN, NDMA, G, kBFirst>(acc, f0, dma);
+            mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, f0, dma);
             __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
-            if constexpr (kBFirst) next_y();
+            next_y();
             load_frags<FP8, MI, NI>(f0, NA, NB, 0, wm, wn, l31, lh);
         } else {
             constexpr int SPAN = (KS - 1) * G;
@@ -337,22 +329,21 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                 } else {
                     __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
                     __builtin_amdgcn_s_barrier();
-                    if constexpr (kBFirst) next_y();
+                    next_y();
                     load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (ks == 0) mma_group<FP8, MI, NI, SPAN, NDMA, 0, kBFirst>(acc, cur, dma);
-                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, NDMA, G, kBFirst>(acc, cur, dma);
-                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, NDMA, 2 * G, kBFirst>(acc, cur, dma);
-                else mma_group<FP8, MI, NI, 1, 0, 0, false>(acc, cur, none);
+                if (ks == 0) mma_group<FP8, MI, NI, SPAN, PWA, 0>(acc, cur, dma);
+                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, cur, dma);
+                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, PWA, 2 * G>(acc, cur, dma);
+                else mma_group<FP8, MI, NI, 1, 0, 0>(acc, cur, none);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
-    if constexpr (kBFirst) {  // what the first stage's closing wait is for (A1 went out with the ring's first fill)
+    // what the first stage's closing wait is for (X1 went out with the ring's first fill)
 #pragma unroll
-        for (int d = 0; d < PWB; ++d) dmaY(3, 1, d);
-    }
+    for (int d = 0; d < PWB; ++d) dmaY(3, 1, d);
     for (int j = 0;;) {
         stage(IC<0>{}, j); if (++j == nk) break;
         stage(IC<1>{}, j); if (++j == nk) break;
