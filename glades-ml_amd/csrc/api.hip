@@ -53,6 +53,8 @@ struct ghip_net {
     float* ownY = nullptr;
     int64_t n_rows = 0;
     uint16_t* Xbf = nullptr;  // bf16 copy of the table (BF16 / FP8_INFER)
+    uint16_t* XbfT = nullptr; // BF16 training: the same table transposed, [inputs][XbfT_ld]; a batch's columns are the
+    long long XbfT_ld = 0;    // B operand of the first layer's weight gradient as they lie (nullptr: transposed per step)
     // exact
     ExactLaunch ex;
     int ex_threads = 64;
@@ -538,7 +540,10 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
     TRY(refresh_shadows(n));
     const uint16_t* X = n->Xbf + row0 * s.sizes[0];
     const float* Y = n->dY + row0 * s.sizes[L];
-    LAUNCH(n, "bf16_transpose_input", ghip_bf16_transpose(X, n->HT[0], B, s.sizes[0], n->stream));
+    // the batch transposed: its columns of the transposed table where that is kept and the batch starts on a
+    // cache line of it, a copy made now otherwise
+    const bool inT = n->XbfT && (row0 % 64) == 0;
+    if (!inT) LAUNCH(n, "bf16_transpose_input", ghip_bf16_transpose(X, n->HT[0], B, s.sizes[0], n->stream));
     TRY(forward_bf16(n, X, B));
     TRY(output_delta_f32(n, n->logits, Y, nullptr, n->D[L], B));
     LAUNCH(n, "bf16_transpose_delta", ghip_bf16_transpose(n->D[L], n->DT[L], B, s.sizes[L], n->stream));
@@ -559,6 +564,7 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
             LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
         memset(&g, 0, sizeof(g));
         g.A = n->DT[l + 1]; g.B = n->HT[l]; g.M = no; g.N = ni; g.K = B;
+        if (l == 0 && inT) { g.B = n->XbfT + row0; g.ldb = (int)n->XbfT_ld; }
         g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l];
         g.master = n->W[l]; g.mom = n->vW[l];
         g.lr = s.lr[l]; g.momf = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l]; g.gscale = 1.0f / (float)B;
@@ -706,7 +712,7 @@ int ghip_net_destroy(ghip_net* n)
     if (n->stream) (void)hipStreamSynchronize(n->stream);
     prof_collect(n);
     free_batch_buffers(n);
-    dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf);
+    dfree(n->ownX); dfree(n->ownY); dfree(n->Xbf); dfree(n->XbfT);
     dfree(n->exW); dfree(n->exSum); dfree(n->exLast); dfree(n->exBias); dfree(n->exPreds);
     dfree(n->exMetrics); dfree(n->exEpochs); dfree(n->cm); dfree(n->exClass); dfree(n->exMulti);
     dfree(n->exMasks); dfree(n->exCnt); dfree(n->exErr); dfree(n->exMultiMetrics); dfree(n->exMultiEpochs);
@@ -913,13 +919,24 @@ static int make_bf16_table(ghip_net* n)
     const ghip_net_spec& s = n->spec;
     if (s.mode != GHIP_MODE_CANONICAL || s.dtype == GHIP_F32) return 0;
     dfree(n->Xbf);
+    dfree(n->XbfT);
+    n->XbfT_ld = 0;
     TRY(dalloc(&n->Xbf, (size_t)n->n_rows * s.sizes[0]));
+    // Training reads each batch transposed as well (the weight gradient of the first layer runs over the
+    // batch): the whole table is kept that way, rows padded by one cache line so that the rows of a tile do
+    // not all start in the same memory channel.  A table too large for that is transposed batch by batch.
+    const long long ldT = ((n->n_rows + 63) / 64) * 64 + 64;
+    const size_t bytesT = (size_t)s.sizes[0] * (size_t)ldT * 2;
+    if (s.dtype == GHIP_BF16 && n->n_rows >= 64 && bytesT <= ((size_t)16 << 30)) {
+        if (hipMalloc((void**)&n->XbfT, bytesT) == hipSuccess) n->XbfT_ld = ldT;
+        else { n->XbfT = nullptr; (void)hipGetLastError(); }
+    }
     // convert in slabs of rows to keep the grid small
     const int64_t slab = 65536;
     for (int64_t r = 0; r < n->n_rows; r += slab) {
         const int rows = (int)((n->n_rows - r) < slab ? (n->n_rows - r) : slab);
-        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d(n->dX + r * s.sizes[0], n->Xbf + r * s.sizes[0], nullptr, rows,
-                                                          s.sizes[0], n->stream));
+        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d_ld(n->dX + r * s.sizes[0], n->Xbf + r * s.sizes[0],
+                                                             n->XbfT ? n->XbfT + r : nullptr, ldT, rows, s.sizes[0], n->stream));
     }
     return 0;
 }

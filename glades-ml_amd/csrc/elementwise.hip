@@ -304,11 +304,12 @@ __global__ void __launch_bounds__(256) fill_kernel(T* p, long long n, T v)
     for (; i < n; i += stride) p[i] = v;
 }
 
-// 64x64 tile through LDS: dst[r][c] = bf16(src[r][c]) and dstT[c][r]; src fp32 or bf16
+// 64x64 tile through LDS: dst[r][c] = bf16(src[r][c]) and dstT[c][r] (rows of dstT are ldT elements apart);
+// src fp32 or bf16
 template <typename SrcT>
 __global__ void __launch_bounds__(256)
 convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ dst,
-                         uint16_t* __restrict__ dstT, int rows, int cols)
+                         uint16_t* __restrict__ dstT, int rows, int cols, long long ldT)
 {
     __shared__ uint16_t tile[64][64 + 2];
     const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
@@ -327,7 +328,7 @@ convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ ds
     if (dstT) {
         for (int j = ty; j < 64; j += 4) {
             const int c = c0 + j, r = r0 + tx;
-            if (r < rows && c < cols) dstT[(long long)c * rows + r] = tile[tx][j];
+            if (r < rows && c < cols) dstT[(long long)c * ldT + r] = tile[tx][j];
         }
     }
 }
@@ -554,8 +555,13 @@ hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream
 
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s)
 {
+    return ghip_f32_to_bf16_2d_ld(src, dst, dstT, rows, rows, cols, s);
+}
+
+hipError_t ghip_f32_to_bf16_2d_ld(const float* src, uint16_t* dst, uint16_t* dstT, long long ldT, int rows, int cols, hipStream_t s)
+{
     dim3 grid((cols + 63) / 64, (rows + 63) / 64);
-    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, dst, dstT, rows, cols);
+    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, dst, dstT, rows, cols, ldT);
     return hipGetLastError();
 }
 
@@ -566,7 +572,7 @@ hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, in
         hipLaunchKernelGGL(bf16_transpose64_kernel, grid, dim3(256), 0, s, src, dstT, rows, cols);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols);
+    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols, (long long)rows);
     return hipGetLastError();
 }
 

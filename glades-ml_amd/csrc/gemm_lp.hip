@@ -623,6 +623,11 @@ bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8)
 hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
 {
     if (!ghip_gemm_lp_shape_ok(a_.M, a_.N, a_.K, a_.fp8)) return hipErrorInvalidValue;
+    // the LDS-direct loads move 16 bytes per lane: operand rows start on 16-byte boundaries, pitches cover K
+    const int es = a_.fp8 ? 1 : 2;
+    if ((a_.lda && (a_.lda < a_.K || ((long long)a_.lda * es) % 16)) || (a_.ldb && (a_.ldb < a_.K || ((long long)a_.ldb * es) % 16)) ||
+        (((uintptr_t)a_.A | (uintptr_t)a_.B) % 16))
+        return hipErrorInvalidValue;
     GemmLpArgs a = a_;
     resolve_act(a);
     if (!a.fp8) {

@@ -365,6 +365,8 @@ bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8);
 int ghip_gemm_lp_tile_m(int M, int N);  // rows per tile the launcher picks for this product
 
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
+// the same with the rows of dstT ldT elements apart (a slab of rows of a table whose transposed copy is kept whole)
+hipError_t ghip_f32_to_bf16_2d_ld(const float* src, uint16_t* dst, uint16_t* dstT, long long ldT, int rows, int cols, hipStream_t s);
 hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s);
 // bias update from bf16 delta^T [n][B] rows (contiguous): gb[o] = sum_b
 hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vbias, float lr,

@@ -238,3 +238,40 @@ def test_bf16_and_e4m3_passes_over_the_table():
         a.run_epoch_canonical(0)
     for n in (a, b, q, short):
         n.close()
+
+
+def test_bf16_step_reads_the_batch_from_the_transposed_table_or_transposes_it():
+    """The first layer's weight gradient takes the batch transposed: as columns of the table's
+    transposed copy when the batch starts on a multiple of 64 rows, from a copy made for the step
+    otherwise.  The same rows at offset 0 of one table, at offset 192 and at offset 40 of another
+    (488 rows, so the transposed copy's pitch is not a multiple of the batch) give bit-identical
+    parameters: the products are the same, only the operand's place and pitch differ."""
+    import pyglades as pg
+    print("bf16 step: batch at row 0 / 192 / 40 of the table", flush=True)
+    rng = np.random.default_rng(33)
+    sizes, acts = [256, 256, 256], [po.RELU, po.SOFTMAX]
+    B = 256
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * np.sqrt(2.0 / sizes[l])).astype(np.float32) for l in range(2)]
+    Xb = rng.standard_normal((B, 256)).astype(np.float32)
+    Yb = teacher_labels(rng, Xb, 256)
+    other = rng.standard_normal((488, 256)).astype(np.float32)
+    results = []
+    for off in (0, 192, 40):
+        if off == 0:
+            X, Y = Xb, Yb
+        else:
+            X = other.copy(); Y = teacher_labels(rng, X, 256)
+            X[off:off + B] = Xb; Y[off:off + B] = Yb
+        g = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_CANONICAL, dtype=pg.BF16, lr=0.05, mom=0.9, cost=po.CLASSIFICATION))
+        for l in range(2):
+            g.set_params(l, Ws[l])
+        g.set_dataset(X, Y)
+        losses = [g.train_step(off, B).loss for _ in range(3)]
+        results.append((losses, [g.get_params(l) for l in range(2)]))
+        g.close()
+    for losses, params in results[1:]:
+        assert losses == results[0][0]
+        for l in range(2):
+            assert np.array_equal(params[l][0], results[0][1][l][0]), l
+            assert np.array_equal(params[l][1], results[0][1][l][1]), l
+    assert any(np.any(results[0][1][0][0] != Ws[0]) for _ in [0])  # the first layer did move
