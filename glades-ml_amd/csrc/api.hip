@@ -37,8 +37,39 @@ int fail(int code, const char* fmt, ...)
 int g_device = -1;
 int g_max_lds = 65536;
 
+// Device memory of ghip_forward_noalloc, the one entry point that must not allocate: a header of
+// accumulators (the softmax pass adds its row sums somewhere) and two halves that the hidden layers'
+// activations alternate between.  Every GPU holds its own copy of the array until the process ends.
+// In host code the array's name is only a handle for hipGetSymbolAddress: the address kernels and
+// copies get is the one that call returned for the current device, kept in g_scratch_ptr.
+constexpr size_t kScratchHeader = 256;
+constexpr size_t kScratchHalf = (size_t)GHIP_NOALLOC_MAX_ACTIVATIONS * sizeof(float);
+constexpr size_t kScratchBytes = kScratchHeader + 2 * kScratchHalf;
+constexpr int kMaxDevices = 16;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
 struct ProfRec { std::string name; hipEvent_t a, b; };
 struct ProfAgg { std::string name; double ms; int64_t n; };
+
+}  // namespace
+
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace {
+
+// Address of this device's copy of `scratch` (resolved once per device, with that device current).
+int scratch_for_device(int device, unsigned char** out)
+{
+    if (device < 0 || device >= kMaxDevices) return fail(GHIP_EINVAL, "device %d: at most %d devices are supported", device, kMaxDevices);
+    if (!g_scratch_ptr[device]) {
+        void* p = nullptr;
+        HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(GHIP_EHIP, "hipGetSymbolAddress returned no address for the scratch array");
+        g_scratch_ptr[device] = (unsigned char*)p;
+    }
+    *out = g_scratch_ptr[device];
+    return 0;
+}
 
 }  // namespace
 
@@ -659,6 +690,8 @@ int ghip_init(int device_ordinal)
         HIP_TRY(hipStreamDestroy(s));
     }
     g_device = device_ordinal;
+    unsigned char* sp = nullptr;
+    TRY(scratch_for_device(device_ordinal, &sp));
     return 0;
 }
 
@@ -1263,6 +1296,43 @@ int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_o
     float* res = nullptr;
     TRY(forward_any(n, n->dX + row0 * s.sizes[0], n->Xbf ? n->Xbf + row0 * s.sizes[0] : nullptr, batch, &res));
     if (dev_out) HIP_TRY(hipMemcpyAsync(dev_out, res, (size_t)batch * s.sizes[s.n_layers] * 4, hipMemcpyDeviceToDevice, n->stream));
+    return 0;
+}
+
+int ghip_forward_noalloc(const ghip_net_spec* spec, const float* const* dev_W, const float* const* dev_bias,
+                         const float* dev_X, int batch, float* dev_out, void* hip_stream)
+{
+    if (check_spec(spec)) return GHIP_EINVAL;
+    if (!dev_W || !dev_bias || !dev_X || !dev_out || batch < 1) return fail(GHIP_EINVAL, "bad arguments");
+    if (spec->mode != GHIP_MODE_CANONICAL || spec->dtype != GHIP_F32)
+        return fail(GHIP_EINVAL, "ghip_forward_noalloc is the canonical fp32 forward only");
+    const int L = spec->n_layers;
+    for (int l = 0; l < L; ++l)
+        if (!dev_W[l] || !dev_bias[l]) return fail(GHIP_EINVAL, "layer %d: weights or biases are NULL", l);
+    for (int l = 1; l < L; ++l)
+        if ((int64_t)batch * spec->sizes[l] > (int64_t)GHIP_NOALLOC_MAX_ACTIVATIONS)
+            return fail(GHIP_EINVAL, "batch %d x hidden layer %d of %d units = %lld activations: the fixed scratch of this entry point "
+                        "holds %lld per layer; use ghip_net_forward_resident or a smaller batch",
+                        batch, l, spec->sizes[l], (long long)batch * spec->sizes[l], (long long)GHIP_NOALLOC_MAX_ACTIVATIONS);
+    int device = -1;
+    HIP_TRY(hipGetDevice(&device));
+    unsigned char* sp = nullptr;
+    TRY(scratch_for_device(device, &sp));
+    // A network object on the stack that owns nothing: the caller's parameters, the caller's stream,
+    // hidden activations in the two halves of the scratch array, the last layer straight into dev_out.
+    ghip_net n;
+    n.spec = *spec;
+    n.L = L;
+    n.stream = (hipStream_t)hip_stream;
+    for (int l = 0; l < L; ++l) {
+        n.W[l] = const_cast<float*>(dev_W[l]);
+        n.b[l] = const_cast<float*>(dev_bias[l]);
+        n.act[l + 1] = (l == L - 1) ? dev_out : (float*)(sp + kScratchHeader + (size_t)(l & 1) * kScratchHalf);
+    }
+    // the softmax pass adds its row sums into accumulators nobody reads: they need no clearing
+    n.dAcc = (double*)sp;
+    float* res = nullptr;
+    TRY(forward_any(&n, dev_X, nullptr, batch, &res));
     return 0;
 }
 

@@ -23,7 +23,7 @@ EXPORTS = [
     "ghip_net_get_state", "ghip_net_set_state",
     "ghip_net_set_dropout_masks", "ghip_net_get_dropout_state", "ghip_net_set_dropout_state",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
-    "ghip_net_run_epoch_canonical", "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_net_eval_resident",
+    "ghip_net_run_epoch_canonical", "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_forward_noalloc", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
     "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
     "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
@@ -97,6 +97,7 @@ def load():
             "ghip_net_last_metrics": (i, [vp, C.POINTER(Metrics)]),
             "ghip_net_forward": (i, [vp, vp, i, vp]),
             "ghip_net_forward_resident": (i, [vp, i64, i, vp]),
+            "ghip_forward_noalloc": (i, [C.POINTER(Spec), C.POINTER(vp), C.POINTER(vp), vp, i, vp, vp]),
             "ghip_net_eval_resident": (i, [vp, i64, i, C.POINTER(Metrics)]),
             "ghip_net_confusion_enable": (i, [vp, i]),
             "ghip_net_confusion_reset": (i, [vp]),

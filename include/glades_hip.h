@@ -212,6 +212,22 @@ int ghip_net_forward(ghip_net* net, const float* host_X, int batch, float* host_
  * dev_out (fp32, batch x sizes[n_layers], may be NULL) receives a device-to-device copy. */
 int ghip_net_forward_resident(ghip_net* net, int64_t row0, int batch, float* dev_out);
 
+/* No counterpart in the reference.  The canonical fp32 forward (as ghip_net_forward_resident: same
+ * kernels, same results bit for bit) for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It takes no handle and calls
+ * no allocating routine: parameters, inputs and outputs are the caller's device memory (dev_W[l]:
+ * sizes[l+1] x sizes[l] row-major, dev_bias[l]: sizes[l+1], dev_X: batch x sizes[0], dev_out: batch x
+ * sizes[n_layers], all fp32, 16-byte aligned), and the hidden layers' activations live in a fixed
+ * array in the library's device image (2 x GHIP_NOALLOC_MAX_ACTIVATIONS floats + 256 bytes = 32 MiB
+ * per GPU, held until the process ends).  batch x sizes[l] of every hidden layer l must not exceed
+ * GHIP_NOALLOC_MAX_ACTIVATIONS; larger requests are refused with GHIP_EINVAL.  spec: mode
+ * GHIP_MODE_CANONICAL, dtype GHIP_F32.  The work is queued on hip_stream (a hipStream_t; NULL = the
+ * null stream) of the calling thread's current device and the call does not wait for it.  All
+ * calls on one GPU share that GPU's array: calls that overlap in time on one GPU race. */
+#define GHIP_NOALLOC_MAX_ACTIVATIONS (4 * 1024 * 1024)
+int ghip_forward_noalloc(const ghip_net_spec* spec, const float* const* dev_W, const float* const* dev_bias,
+                         const float* dev_X, int batch, float* dev_out, void* hip_stream);
+
 /* Canonical mode RUN_TEST pass (network.cpp:109-112,372-373) on rows [row0,row0+batch) of the
  * resident table: forward and metrics, no parameter changes. */
 int ghip_net_eval_resident(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);
