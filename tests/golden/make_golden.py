@@ -7,7 +7,8 @@ the reference's unit-test data (xor gate table, iris measurements) and its NNInf
 hyper-parameters (xornet: 2-2-1 TANH lr .003 mb 1 REGRESSION; iris: 4-5-3 SIGMOID lr .01
 mb 1 CLASSIFICATION).
 
-    python tests/golden/make_golden.py
+    python tests/golden/make_golden.py            # everything
+    python tests/golden/make_golden.py full       # only the full-schedule runs (about 5 minutes)
 """
 import os
 import subprocess
@@ -54,7 +55,94 @@ DROPOUT_CASES = [
      [0.5, 0.25]),
 ]
 
+# The two CPU-sized benchmark configurations on their own data and over their whole schedule:
+# (name, sizes, acts, cost, mb, epochs, lr, mom, act_params, seed, data)
+FULL_CASES = [
+    # 150 rows from 3 Gaussian clusters, 4-16-3 sigmoid, BCE, full batch (mb = N), 500 epochs.  lr 0.01
+    # trains; lr 0.1 (the configuration as written) turns to NaN in the reference within the first
+    # epochs, and the NaNs have to sit in the same places
+    ("cfg1_full_lr001", [4, 16, 3], [po.SIGMOID] * 2, po.CLASSIFICATION, 150, 500, 0.01, 0.9, 0, 101, "clusters"),
+    ("cfg1_full_lr01", [4, 16, 3], [po.SIGMOID] * 2, po.CLASSIFICATION, 150, 500, 0.1, 0.9, 0, 101, "clusters"),
+    # 10 000 windows of 32 lagged values of a sum of three sines plus noise, 32-64-64-1 tanh / tanh /
+    # linear, MSE, mb 256, 50 epochs = 500 000 rows through the reference's objects
+    ("cfg2_full", [32, 64, 64, 1], [po.TANH, po.TANH, po.LINEAR], po.REGRESSION, 256, 50, 0.01, 0.9, [0, 0, 1.0], 102, "sines"),
+]
+
 IRIS = os.path.join(HERE, "iris_measurements.csv")
+
+
+def scale_classification_columns(feats):
+    """NumberInput.cpp:68-212 on a classification table: min/max start from 0 for every column but
+    the first; x -> (x-min)/range*0.98+0.01."""
+    X = np.empty_like(feats)
+    for c in range(feats.shape[1]):
+        col = feats[:, c]
+        fmin = np.float32(min(col.min(), col[0] if c == 0 else np.float32(0)))
+        fmax = np.float32(max(col.max(), col[0] if c == 0 else np.float32(0)))
+        X[:, c] = ((col - fmin) / np.float32(fmax - fmin)) * np.float32(0.98) + np.float32(0.01)
+    return X
+
+
+def cluster_table(seed, n_rows=150, n_feat=4, n_cls=3, sigma=0.5):
+    """Rows from n_cls isotropic Gaussian clusters (centres uniform in [0,8]^n_feat), classes
+    interleaved, scaled and labelled (0.99 / 0.01) the way the reference's CSV path would."""
+    rng = np.random.default_rng(seed)
+    centres = rng.uniform(0.0, 8.0, (n_cls, n_feat))
+    cls = np.arange(n_rows) % n_cls
+    feats = (centres[cls] + sigma * rng.standard_normal((n_rows, n_feat))).astype(np.float32)
+    Y = np.where(np.eye(n_cls)[cls] > 0, np.float32(0.99), np.float32(0.01)).astype(np.float32)
+    return scale_classification_columns(feats), Y
+
+
+def sine_series(seed, n_rows=10000, lags=32):
+    """n_rows + lags values of a sum of three sines (random frequency and phase) plus N(0, 0.05)
+    noise, scaled to [0, 1]: row i of the table is series[i : i+lags], its target series[i+lags]."""
+    rng = np.random.default_rng(seed)
+    t = np.arange(n_rows + lags, dtype=np.float64)
+    f = rng.uniform(0.005, 0.05, 3)
+    ph = rng.uniform(0.0, 2 * np.pi, 3)
+    v = sum(np.sin(2 * np.pi * f[k] * t + ph[k]) for k in range(3)) + 0.05 * rng.standard_normal(t.size)
+    v = (v - v.min()) / (v.max() - v.min())
+    return v.astype(np.float32)
+
+
+def windows(series, lags=32):
+    n = series.size - lags
+    X = np.lib.stride_tricks.sliding_window_view(series, lags)[:n].copy()
+    return X, series[lags:].reshape(n, 1).copy()
+
+
+def full_schedule_runs(td):
+    for (name, sizes, acts, cost, mb, epochs, lr, mom, params, seed, data) in FULL_CASES:
+        nl = len(sizes) - 1
+        spec = po.make_spec(sizes, acts, lr=lr, mom=mom, act_params=params, batch=mb, cost=cost)
+        # the reference's own sampler (Layer::initWeights, layer.cpp:196-217) under srand(seed + layer)
+        Ws = [ref_xavier(seed + l, sizes[l], sizes[l + 1], acts[max(l - 1, 0)] if l == nl - 1 else acts[l], td)
+              for l in range(nl)]
+        bs = [0.0] * nl
+        extra = {}
+        if data == "clusters":
+            X, Y = cluster_table(seed)
+            extra = dict(X=X, Y=Y)
+        else:
+            series = sine_series(seed)
+            X, Y = windows(series)
+            extra = dict(series=series)        # the table is rebuilt from it (40 KB instead of 1.3 MB)
+        ref = po.ref_train(spec, Ws, bs, X, Y, epochs, td)
+        d = dict(sizes=np.array(sizes, np.int32), acts=np.array(acts, np.int32),
+                 hyper=np.array([lr, mom, 0, 0], np.float32),
+                 act_params=np.array(params if isinstance(params, list) else [params] * nl, np.float32),
+                 ints=np.array([cost, X.shape[0], mb, epochs], np.int32),
+                 bias0=np.array(bs, np.float32), epochs=ref["epochs"], bias=ref["bias"], preds=ref["preds"], **extra)
+        for l in range(nl):
+            d[f"W0_{l}"] = Ws[l]
+            d[f"W_{l}"] = ref["W"][l]
+            d[f"wsum_{l}"] = ref["wsum"][l]
+            d[f"wlast_{l}"] = ref["wlast"][l]
+        np.savez_compressed(os.path.join(HERE, f"train_{name}.npz"), **d)
+        ep = ref["epochs"]
+        print(name, "epochs", epochs, "first", ep[0], "last", ep[-1], "non-finite epochs", int((~np.isfinite(ep[:, 0])).sum()),
+              "max|W0|", float(np.nanmax(np.abs(ref["W"][0]))), flush=True)
 
 
 def ref_xavier(seed, fan_in, n_out, act, td):
@@ -90,6 +178,9 @@ def main():
     if not po.have_ref():
         raise SystemExit("oracle/_ref/ref_harness missing: run `make -C oracle ref` where /root/reference exists")
     with tempfile.TemporaryDirectory() as td:
+        full_schedule_runs(td)
+        if sys.argv[1:] == ["full"]:
+            return
         # element-wise grid
         g = os.path.join(td, "g.bin")
         subprocess.check_call([po.REF_HARNESS, "gmath", g])

@@ -10,6 +10,11 @@ TRAIN_CASES = ["one_sample_2_3_2", "window_4_5_3_1", "decay_3_4_2", "cfg1_shape_
                "cfg2_shape_32_64_64_1", "mixed_5_7_6_4", "kl_3_5_4_2", "xornet", "iris"]
 
 
+# the two CPU-sized benchmark configurations on their own data over their whole schedule: 500 epochs of
+# 150 rows from 3 Gaussian clusters at lr 0.01 and at lr 0.1 (where the reference turns to NaN), and
+# 50 epochs of 10 000 sine windows (500 000 rows), all through the reference's compiled objects
+FULL_CASES = ["cfg1_full_lr001", "cfg1_full_lr01", "cfg2_full"]
+
 DROPOUT_CASES = ["window_4_5_3_1", "decay_3_4_2", "out_of_range_6_8_2", "heavy_6_8_2", "batch1_5_7_6_4",
                  "deep_64_48_6_2", "wide_1100_12_2"]
 
@@ -24,8 +29,14 @@ def load_case(name, kind="train"):
     lr, mom, wd1, wd2 = [float(v) for v in d["hyper"]]
     spec = po.make_spec(sizes, [int(a) for a in d["acts"]], lr=lr, mom=mom, wd1=wd1, wd2=wd2,
                         act_params=[float(v) for v in d["act_params"]], batch=mb, cost=cost)
+    if "series" in d.files:   # lagged windows of one series: row i = series[i : i+lags], target series[i+lags]
+        series = d["series"]
+        X = np.lib.stride_tricks.sliding_window_view(series, sizes[0])[:N].copy()
+        Y = series[sizes[0]:].reshape(N, 1).copy()
+    else:
+        X, Y = d["X"], d["Y"]
     return dict(d=d, sizes=sizes, nl=nl, cost=cost, N=N, mb=mb, epochs=epochs, spec=spec,
-                W0=[d[f"W0_{l}"] for l in range(nl)], bias0=d["bias0"], X=d["X"], Y=d["Y"])
+                W0=[d[f"W0_{l}"] for l in range(nl)], bias0=d["bias0"], X=X, Y=Y)
 
 
 def bits_equal(a, b):

@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 import pyoracle as po
-from helpers import TRAIN_CASES, bits_equal, load_case
+from helpers import FULL_CASES, TRAIN_CASES, bits_equal, load_case
 
 pytestmark = pytest.mark.gpu
 
@@ -41,7 +41,7 @@ def gpu_net(c, bias_mode=0):
     return net
 
 
-@pytest.mark.parametrize("name", TRAIN_CASES)
+@pytest.mark.parametrize("name", TRAIN_CASES + FULL_CASES)
 def test_fixture_schedule(name):
     print("case", name, flush=True)
     c = load_case(name)

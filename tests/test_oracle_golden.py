@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import pyoracle as po
-from helpers import DROPOUT_CASES, GOLDEN, TRAIN_CASES, bits_equal, load_case
+from helpers import DROPOUT_CASES, FULL_CASES, GOLDEN, TRAIN_CASES, bits_equal, load_case
 
 
 def test_elementwise_grid_bit_exact():
@@ -44,7 +44,7 @@ def test_xavier_sampler_bit_exact():
         assert (W >= 0).all()  # the sampler only ever returns the positive half
 
 
-@pytest.mark.parametrize("name", TRAIN_CASES)
+@pytest.mark.parametrize("name", TRAIN_CASES + FULL_CASES)
 def test_exact_training_bit_exact(name):
     c = load_case(name)
     net = po.ExactNet(c["spec"])
