@@ -57,6 +57,32 @@ def rel_err(a, b):
     return float(np.max(np.abs(a - b) / (np.abs(b) + 1e-6))) if a.size else 0.0
 
 
+def cluster_centres(rng, n_cls, dim):
+    return rng.standard_normal((n_cls, dim), dtype=np.float32)
+
+
+def cluster_rows(rng, centres, n_rows, sigma=1.0, n_out=None):
+    """Rows from isotropic Gaussian clusters around `centres` (class = cluster), scaled so that every
+    feature is N(0,1) overall, with one-hot labels n_out wide: classes that a trained network separates
+    with a margin, so that "which class wins" is a question with an answer for every row."""
+    n_cls, dim = centres.shape
+    cls = rng.integers(0, n_cls, n_rows)
+    X = centres[cls] + np.float32(sigma) * rng.standard_normal((n_rows, dim), dtype=np.float32)
+    X *= np.float32(1.0 / np.sqrt(1.0 + sigma * sigma))
+    Y = np.zeros((n_rows, n_out or n_cls), np.float32)
+    Y[np.arange(n_rows), cls] = 1.0
+    return X, Y, cls
+
+
+def he_init(rng, sizes):
+    return [rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l]))
+            for l in range(len(sizes) - 1)]
+
+
+def rel_rms(a, b):
+    return float(np.sqrt(np.mean((np.asarray(a, np.float64) - b) ** 2)) / np.sqrt(np.mean(np.asarray(b, np.float64) ** 2)))
+
+
 def bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, steps, lr, mom, wd2, wide=True):
     """numpy statement of the bf16 training pipeline: bf16 weights (rounded from the fp32 master),
     bf16 activations and deltas, products exact and summed in float64, fp32 logits/softmax,
