@@ -390,6 +390,45 @@ void xavierLayer(int fanIn, int nOut, int activationType, float* W)
         }
 }
 
+bool sampleInitialWeights(const NNInfo* s, int nFeat, int nOut, std::vector<std::vector<float> >& W, std::string* err)
+{
+    const int H = s->numHiddenLayers();
+    const int outputType = s->getOutputType();
+    W.assign(H + 1, std::vector<float>());
+    bool isPositive = false;
+    int prev = nFeat;
+    for (int i = 0; i < H; ++i) {
+        const int at = s->getActivationType(i);
+        const int cur = s->getHiddenLayerSize(i);
+        if (!isPositive && (at == GMath::SIGMOID || at == GMath::RELU || at == GMath::LEAKY || outputType == GMath::CLASSIFICATION)) {
+            isPositive = true;   // LayerBuilder.cpp:213-222: start over; prev keeps the size of hidden layer i-1
+            for (int k = 0; k < H; ++k) W[k].clear();
+            i = -1;
+            continue;
+        }
+        const int want = i == 0 ? nFeat : s->getHiddenLayerSize(i - 1);
+        if (prev < want) {
+            if (err) {
+                char buf[256];
+                snprintf(buf, sizeof(buf), "the reference would sample the first hidden layer with %d of %d input edges (its hidden-layer "
+                         "restart keeps a stale layer size, LayerBuilder.cpp:196-233): that network is not modelled; inject the weights", prev, want);
+                *err = buf;
+            }
+            return false;
+        }
+        std::vector<float> full((size_t)prev * cur);
+        xavierLayer(prev, cur, at, full.data());
+        W[i].resize((size_t)want * cur);
+        for (int o = 0; o < cur; ++o) memcpy(&W[i][(size_t)o * want], &full[(size_t)o * prev], sizeof(float) * want);
+        prev = cur;
+    }
+    // LayerBuilder.cpp:236-265: fan-in = the last hidden layer, scaled by the last hidden row's activation type
+    const int lastSize = H > 0 ? s->getHiddenLayerSize(H - 1) : nFeat;
+    W[H].resize((size_t)lastSize * nOut);
+    xavierLayer(lastSize, nOut, s->getActivationType(H > 0 ? H - 1 : 0), W[H].data());
+    return true;
+}
+
 // ------------------------------------------------------------------ NNetwork
 
 static int64_t g_next_id = 1;
@@ -398,7 +437,7 @@ NNetwork::NNetwork()
     : di(NULL), skeleton(NULL), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
       dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
-      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false)
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false), prepaidDrawEpochs(0)
 {
 }
 
@@ -406,7 +445,7 @@ NNetwork::NNetwork(NNInfo* newNNInfo)
     : di(NULL), skeleton(newNNInfo), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
       dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
-      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false)
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false), prepaidDrawEpochs(0)
 {
 }
 
@@ -456,7 +495,7 @@ bool NNetwork::load(const std::string& path)
 bool NNetwork::save(const std::string& path) const { return skeleton ? skeleton->saveFile(path) : false; }
 
 // file: "GLCK" u32 version, i32 mode, i32 dtype, i32 epochs, i32 nLayers, i32 sizes[nLayers+1],
-//       u32 tableBytes, table text (the NNInfo CSV), then per layer: W, u32 biasLen, bias, u32 aLen, a, u32 bLen, b,
+//       u32 tableBytes, table text (the NNInfo CSV), from version 3 on u32 nameBytes, the network's name, then per layer: W, u32 biasLen, bias, u32 aLen, a, u32 bLen, b,
 //       and from version 2 on u32 cLen, window lengths (i32), u32 eLen, node error accumulators (exact mode; else 0, 0)
 // fwrite / fread of n elements that leave an empty array's (possibly null) pointer alone
 static size_t put(const void* p, size_t size, size_t n, FILE* f) { return n ? fwrite(p, size, n, f) : 0; }
@@ -483,10 +522,12 @@ bool NNetwork::saveCheckpoint(const std::string& path)
     }
     FILE* f = fopen(path.c_str(), "wb");
     if (!f) { lastError = "cannot write " + path; return false; }
-    const uint32_t version = 2, tb = (uint32_t)table.size();
+    const std::string netName = skeleton->getName();
+    const uint32_t version = 3, tb = (uint32_t)table.size(), nb = (uint32_t)netName.size();
     const int32_t head[4] = {mode, dtype, epochs, L};
     fwrite("GLCK", 1, 4, f); fwrite(&version, 4, 1, f); fwrite(head, 4, 4, f); put(sizes.data(), 4, sizes.size(), f);
     fwrite(&tb, 4, 1, f); put(table.data(), 1, table.size(), f);
+    fwrite(&nb, 4, 1, f); put(netName.data(), 1, netName.size(), f);
     bool ok = true;
     for (int l = 0; l < L && ok; ++l) {
         const size_t cnt = (size_t)sizes[l] * sizes[l + 1];
@@ -517,15 +558,25 @@ bool NNetwork::loadCheckpoint(const std::string& path)
     char magic[4];
     uint32_t version = 0, tb = 0;
     int32_t head[4];
-    bool ok = fread(magic, 1, 4, f) == 4 && memcmp(magic, "GLCK", 4) == 0 && fread(&version, 4, 1, f) == 1 && (version == 1 || version == 2) &&
-              fread(head, 4, 4, f) == 4 && head[3] >= 1 && head[3] <= 16;
+    bool ok = fread(magic, 1, 4, f) == 4 && memcmp(magic, "GLCK", 4) == 0 && fread(&version, 4, 1, f) == 1 && version >= 1 && version <= 3 &&
+              fread(head, 4, 4, f) == 4 && head[3] >= 1 && head[3] <= 16 &&
+              (head[0] == MODE_EXACT || head[0] == MODE_CANONICAL) && (head[1] == DTYPE_F32 || head[1] == DTYPE_BF16) && head[2] >= 0;
     std::vector<int32_t> sizes;
-    std::string table;
+    std::string table, netName;
+    bool named = false;
     if (ok) {
         sizes.resize(head[3] + 1);
         ok = get(sizes.data(), 4, sizes.size(), f) == sizes.size() && fread(&tb, 4, 1, f) == 1 && tb < (1u << 20);
+        // nothing is allocated from sizes the file does not back up: a layer has 1 .. 2^24 nodes and at most 2^31 edges
+        for (size_t l = 0; ok && l < sizes.size(); ++l) ok = sizes[l] >= 1 && sizes[l] <= (1 << 24);
+        for (size_t l = 0; ok && l + 1 < sizes.size(); ++l) ok = (int64_t)sizes[l] * sizes[l + 1] <= ((int64_t)1 << 31);
     }
     if (ok) { table.resize(tb); ok = get(tb ? &table[0] : nullptr, 1, tb, f) == tb; }
+    if (ok && version >= 3) {
+        uint32_t nb = 0;
+        ok = fread(&nb, 4, 1, f) == 1 && nb < 4096;
+        if (ok) { netName.resize(nb); ok = get(nb ? &netName[0] : nullptr, 1, nb, f) == nb; named = true; }
+    }
     std::vector<std::vector<float> > W, B, SA, SB, ED;
     std::vector<std::vector<int32_t> > WC;
     for (int l = 0; ok && l < head[3]; ++l) {
@@ -556,6 +607,9 @@ bool NNetwork::loadCheckpoint(const std::string& path)
     const bool loaded = load(tmp);
     remove(tmp.c_str());
     if (!loaded) { lastError = "checkpoint holds no valid network table"; return false; }
+    // load() names the network after the file it read, here the temporary table: put the saved name back
+    // (older files have none: the checkpoint's own file name then)
+    skeleton->setName(named ? netName : path.substr(path.find_last_of('/') == std::string::npos ? 0 : path.find_last_of('/') + 1));
     clean();
     mode = head[0]; dtype = head[1]; epochs = head[2];
     initW = W; initB = B; initStateA = SA; initStateB = SB; initCounts = WC; initErrDer = ED;
@@ -657,6 +711,47 @@ void NNetwork::drawDropout()
     }
 }
 
+size_t NNetwork::dropoutDrawsPerEpoch() const
+{
+    if (!skeleton || mode != MODE_EXACT) return 0;
+    const int H = skeleton->numHiddenLayers();
+    size_t nodes = 0;
+    for (int l = 0; l <= H; ++l) {
+        const float p = l == 0 ? skeleton->getPInput() : skeleton->getPDropout(l - 1);
+        const int rate = p * 100.0f;  // layer.cpp:107-112: rates below 0 and from 100 up draw nothing
+        if (rate >= 0 && rate < 100) nodes += l == 0 ? nFeat : (size_t)skeleton->getHiddenLayerSize(l - 1);
+    }
+    return nodes * nRows;
+}
+
+void NNetwork::skipDropoutDraws(int64_t n)
+{
+    if (dropoutOn || n <= 0) return;  // with dropout the flags themselves are drawn (drawDropout)
+    const int64_t paid = prepaidDrawEpochs < n ? prepaidDrawEpochs : n;
+    prepaidDrawEpochs -= paid;
+    const size_t per = dropoutDrawsPerEpoch();
+    for (int64_t e = paid; e < n; ++e)
+        for (size_t k = 0; k < per; ++k) (void)rand();
+}
+
+void NNetwork::prepayDropoutDraws(int64_t n)
+{
+    if (dropoutOn || n <= 0) return;
+    const size_t per = dropoutDrawsPerEpoch();
+    for (int64_t e = 0; e < n; ++e)
+        for (size_t k = 0; k < per; ++k) (void)rand();
+    prepaidDrawEpochs += n;
+}
+
+bool NNetwork::samplesOnBuild() const
+{
+    if (dev || !skeleton) return false;
+    const int H = skeleton->numHiddenLayers();
+    for (int l = 0; l <= H; ++l)
+        if ((size_t)l >= initW.size() || initW[l].empty()) return true;
+    return false;
+}
+
 bool NNetwork::build()
 {
     std::vector<float> X, Y;
@@ -690,18 +785,19 @@ bool NNetwork::build()
     s.mode = mode == MODE_EXACT ? GHIP_MODE_EXACT : GHIP_MODE_CANONICAL;
     s.dtype = dtype == DTYPE_BF16 ? GHIP_BF16 : GHIP_F32;
     s.bias_mode = biasMode;
+    // weights: injected ones as they are; if any layer has none, the whole network is sampled in the
+    // reference's order (so libc's rand() moves as it does there) and injected layers replace their draw
+    std::vector<std::vector<float> > sampled;
+    bool allInjected = true;
+    for (int l = 0; l <= H; ++l)
+        allInjected = allInjected && (size_t)l < initW.size() && initW[l].size() == (size_t)s.sizes[l] * s.sizes[l + 1];
+    if (!allInjected && !sampleInitialWeights(skeleton, (int)nFeat, (int)nOut, sampled, &lastError)) return false;
     if (ghip_net_create(&s, &dev) != 0) { lastError = ghip_last_error(); dev = NULL; return false; }
     for (int l = 0; l <= H; ++l) {
         const int ni = s.sizes[l], no = s.sizes[l + 1];
         std::vector<float> W;
-        if ((size_t)l < initW.size() && initW[l].size() == (size_t)ni * no) {
-            W = initW[l];
-        } else {
-            W.resize((size_t)ni * no);
-            // the output layer is scaled by the activation type of index H-1 (LayerBuilder.cpp:243-265)
-            const int at = skeleton->getActivationType(l < H ? l : (H > 0 ? H - 1 : 0));
-            xavierLayer(ni, no, at, W.data());
-        }
+        if ((size_t)l < initW.size() && initW[l].size() == (size_t)ni * no) W = initW[l];
+        else W.swap(sampled[l]);
         const float* bp = NULL;
         int bl = 0;
         if ((size_t)l < initB.size() && !initB[l].empty()) { bp = initB[l].data(); bl = (int)initB[l].size(); }
@@ -1155,6 +1251,7 @@ void NNetwork::run(DataInput* newDataInput, int runType)
                 break;
             }
             if (ran <= 0) break;
+            skipDropoutDraws(ran);  // the darts the reference throws at rate 0 (train and test passes alike)
             for (int e = 0; e < ran; ++e) learningCurve.push_back(ms[e].accuracy);
             afterEpochs(&ms[ran - 1], ran, runType);
         } else {
@@ -1188,9 +1285,15 @@ void NNetwork::run(DataInput* newDataInput, int runType)
 // Subnets that are the same network in everything but their parameters (exact mode, equal tables,
 // equal epoch counters and stop conditions) train in ONE kernel launch per chunk of epochs, a
 // workgroup each; a subnet that meets its stop condition leaves the group.
-bool MetaNetwork::runGroup(DataInput* d, int runType)
+bool MetaNetwork::runGroup(DataInput* d, int runType, bool testsFollow)
 {
     std::vector<NNetwork*> act;
+    // The reference runs subnet after subnet, so a subnet that samples its weights finds libc's rand()
+    // where the runs of the subnets before it left it.  Here all subnets are built first: if a later
+    // one samples, the draws of the runs before it are taken ahead of time, which needs their number:
+    // known for an epoch-count stop, unknown for an accuracy stop (then the caller runs them in turn).
+    bool laterSamples = false;
+    for (size_t i = 1; i < subnets.size(); ++i) laterSamples = laterSamples || (subnets[i] && subnets[i]->samplesOnBuild());
     for (size_t i = 0; i < subnets.size(); ++i) {
         NNetwork* n = subnets[i];
         if (!n || !n->skeleton || n->mode != NNetwork::MODE_EXACT) return false;
@@ -1199,9 +1302,16 @@ bool MetaNetwork::runGroup(DataInput* d, int runType)
         if (n->epochs != a->epochs || n->biasMode != a->biasMode || n->skeleton->toTable() != a->skeleton->toTable()) return false;
         if (n->terminator.getEpoch() != a->terminator.getEpoch() || n->terminator.getAccuracy() != a->terminator.getAccuracy() ||
             n->terminator.getTimestamp() != 0) return false;
+        if (laterSamples && runType == NNetwork::RUN_TRAIN && (n->terminator.getAccuracy() > 0.0f || n->terminator.getEpoch() <= 0)) return false;
     }
     for (size_t i = 0; i < subnets.size(); ++i) {
         if (!subnets[i]->prepare(d)) return false;
+        if (laterSamples) {
+            NNetwork* n = subnets[i];
+            const int64_t e = n->terminator.getEpoch();
+            const int64_t ahead = (runType == NNetwork::RUN_TRAIN ? e - ((int64_t)n->epochs % e) : 1) + (testsFollow ? 1 : 0);
+            n->prepayDropoutDraws(ahead);
+        }
         subnets[i]->resetGraphs();
         subnets[i]->running = true;
         act.push_back(subnets[i]);
@@ -1221,6 +1331,7 @@ bool MetaNetwork::runGroup(DataInput* d, int runType)
         for (size_t i = 0; i < act.size(); ++i) {
             NNetwork* n = act[i];
             if (ran[i] <= 0) { n->running = false; continue; }
+            n->skipDropoutDraws(ran[i]);
             for (int e = 0; e < ran[i]; ++e) n->learningCurve.push_back(ms[i * chunk + e].accuracy);
             n->afterEpochs(&ms[i * chunk + ran[i] - 1], ran[i], runType);
             const bool done = !n->running || n->terminator.triggered(time(NULL), n->epochs, n->overallTotalAccuracy) || runType == NNetwork::RUN_TEST;
@@ -1283,8 +1394,11 @@ template <typename Fn>
 void for_each_subnet(MetaNetwork* m, Fn fn)
 {
     const std::vector<NNetwork*>& nets = m->getSubnets();
-    bool dropout = false;  // libc rand() is one stream: the reference's order is subnet after subnet
-    for (size_t i = 0; i < nets.size(); ++i) dropout = dropout || (nets[i] && nets[i]->hasDropout());
+    // libc rand() is one stream and the reference's order is subnet after subnet: subnets that draw
+    // dropout flags, or that sample their weights after another subnet's run, take their turn
+    bool dropout = false;
+    for (size_t i = 0; i < nets.size(); ++i)
+        dropout = dropout || (nets[i] && (nets[i]->hasDropout() || (i > 0 && nets[i]->samplesOnBuild())));
     if (!m->getConcurrent() || nets.size() < 2 || dropout) {
         for (size_t i = 0; i < nets.size(); ++i)
             if (nets[i]) fn(nets[i]);
@@ -1336,7 +1450,7 @@ NNetwork* MetaNetwork::getSubnetByName(const std::string& n) const
 float MetaNetwork::crossValidate(DataInput* newDataInput)
 {
     if (!newDataInput || subnets.empty()) return 0.0f;
-    if (concurrent && subnets.size() > 1 && runGroup(newDataInput, NNetwork::RUN_TRAIN)) {
+    if (concurrent && subnets.size() > 1 && runGroup(newDataInput, NNetwork::RUN_TRAIN, true)) {
         if (!runGroup(newDataInput, NNetwork::RUN_TEST))
             for_each_subnet(this, [newDataInput](NNetwork* n) { n->test(newDataInput); });
     } else {

@@ -364,6 +364,13 @@ class NNetwork
     std::vector<unsigned char> dropFlags;
     bool dropoutOn;
     void drawDropout();                              // one epoch's flags from libc rand()
+    // Layer::generateDropout draws one dart per node and row for every rate in 0..99, also at rate 0,
+    // where no dart can drop anything (layer.cpp:102-134): a run without dropout still moves libc's
+    // rand() by that many draws per epoch, which the next network's weight sampler then starts from
+    int64_t prepaidDrawEpochs;                       // epochs whose draws have been taken ahead of the run
+    size_t dropoutDrawsPerEpoch() const;
+    void skipDropoutDraws(int64_t epochs);           // exact mode, no flags: take the draws and throw them away
+    void prepayDropoutDraws(int64_t epochs);
 
     void run(DataInput*, int);
     bool prepare(DataInput*);                        // checks + build on first use
@@ -372,6 +379,7 @@ class NNetwork
 
 public:
     bool hasDropout() const;  // some layer's rate int(p*100) lies in 1..99
+    bool samplesOnBuild() const;  // not built yet and not every layer's weights injected: the first run draws weights from rand()
     static const int TYPE_DFF = 0, TYPE_RNN = 1;
     static const int RUN_TRAIN = 0, RUN_TEST = 1, RUN_VALIDATE = 2;
     static const int MODE_EXACT = 0, MODE_CANONICAL = 1;      // extension
@@ -467,7 +475,9 @@ public:
     // one kernel launch for all subnets where they allow it (see glades.cpp); false = not applicable.
     // Subnets trained this way keep their metrics, learning curve and weights; getResults() (the last
     // row's predictions) stays empty, since the grouped launch returns no predictions.
-    bool runGroup(DataInput*, int runType);
+    // testsFollow: every subnet's training is followed by its test pass before the next subnet trains
+    // (crossValidate), which matters to where libc's rand() stands when a later subnet samples weights.
+    bool runGroup(DataInput*, int runType, bool testsFollow = false);
     std::string getName() const { return name; }
     void setName(const std::string& v) { name = v; }
     int getCollectionType() const { return collectionType; }
@@ -494,6 +504,16 @@ MetaNetwork* test(MetaNetwork*, DataInput*);
 // The reference's weight sampler (ML/State/layer.cpp:196-217, ML/State/node.cpp:241-276): draws
 // from libc rand(), so srand(seed) reproduces the reference's initial weights for a layer.
 void xavierLayer(int fanIn, int nOut, int activationType, float* W);
+// The initial weights of a whole network in the order LayerBuilder::buildHiddenLayers / buildOutputLayer
+// sample them (ML/State/LayerBuilder.cpp:192-265), from libc rand(): W[l] is sizes[l+1] x sizes[l].
+// Includes the restart of the hidden layers: the first row whose activation is SIGMOID / RELU / LEAKY
+// (any row when the output is CLASSIFICATION) throws the layers built so far away, their draws spent,
+// and starts over WITHOUT resetting prevLayerSize (:196,213-222), so after a restart at row i >= 1
+// the first hidden layer is sampled with fan-in = size of hidden layer i-1: its scale is that fan-in's
+// and, if it is larger than the feature count, the surplus edges exist but are never visited.  A
+// stale fan-in SMALLER than the feature count leaves input columns without an edge in the reference;
+// that network is not modelled here: false, with a message.
+bool sampleInitialWeights(const NNInfo* skeleton, int nFeat, int nOut, std::vector<std::vector<float> >& W, std::string* err);
 
 }  // namespace glades
 #endif

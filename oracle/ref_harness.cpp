@@ -15,6 +15,8 @@
  * Usage:
  *   ref_harness gmath  <out.bin>                      grid of element-wise functions
  *   ref_harness xavier <seed> <fan_in> <n_out> <act> <out.bin>
+ *   ref_harness xavierseq <seed> <out.bin> <fan_in> <n_out> <act> [<fan_in> <n_out> <act> ...]
+ *       the layers one after the other under ONE srand(seed), then rand() % 65536 as a float
  *   ref_harness train  <case.bin> <out.bin>           see tests/golden/make_golden.py
  *   ref_harness term   <out.bin>                      Terminator truth table
  */
@@ -78,6 +80,23 @@ static int do_xavier(int seed, int fan_in, int n_out, int act, const char* out)
     if (!f) return 1;
     for (int o = 0; o < n_out; ++o)
         for (int i = 0; i < fan_in; ++i) wrf(f, layer[o]->getEdgeWeight(i));
+    fclose(f);
+    return 0;
+}
+
+static int do_xavier_seq(int seed, const char* out, int n, char** spec)
+{
+    srand(seed);
+    FILE* f = fopen(out, "wb");
+    if (!f) return 1;
+    for (int k = 0; k + 2 < n; k += 3) {
+        const int fan_in = atoi(spec[k]), n_out = atoi(spec[k + 1]), act = atoi(spec[k + 2]);
+        Layer layer(Layer::HIDDEN_TYPE);
+        layer.initWeights(fan_in, n_out, Node::INIT_XAVIER, act);
+        for (int o = 0; o < n_out; ++o)
+            for (int i = 0; i < fan_in; ++i) wrf(f, layer[o]->getEdgeWeight(i));
+    }
+    wrf(f, (float)(rand() % 65536));
     fclose(f);
     return 0;
 }
@@ -315,6 +334,8 @@ static int do_train(const char* in, const char* out)
 int main(int argc, char** argv)
 {
     if (argc >= 3 && !strcmp(argv[1], "gmath")) return do_gmath(argv[2]);
+    if (argc >= 7 && !strcmp(argv[1], "xavierseq"))
+        return do_xavier_seq(atoi(argv[2]), argv[3], argc - 4, argv + 4);
     if (argc >= 7 && !strcmp(argv[1], "xavier"))
         return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "train")) return do_train(argv[2], argv[3]);

@@ -9,6 +9,7 @@ mb 1 CLASSIFICATION).
 
     python tests/golden/make_golden.py            # everything
     python tests/golden/make_golden.py full       # only the full-schedule runs (about 5 minutes)
+    python tests/golden/make_golden.py init       # only the whole-network initialisations
 """
 import os
 import subprocess
@@ -112,6 +113,59 @@ def windows(series, lags=32):
     return X, series[lags:].reshape(n, 1).copy()
 
 
+# Whole-network initialisations: (name, seed, n_feat, hidden sizes, acts as NNInfo::getActivationType(i)
+# returns them for i = 0 .. H-1 (the input row, then the hidden rows but the last), n_out, output type)
+INIT_CASES = [
+    ("plain_tanh", 21, 4, [5, 3], [po.TANH, po.TANH], 2, po.REGRESSION),             # no restart
+    ("restart_row0", 22, 4, [5], [po.SIGMOID], 3, po.CLASSIFICATION),                 # restart at row 0: nothing thrown away
+    ("restart_row1_wider", 23, 3, [6, 4], [po.TANH, po.SIGMOID], 2, po.REGRESSION),   # row 1: layer 0 again, with fan-in 6
+    ("restart_row2_equal", 24, 5, [3, 5, 4], [po.TANH, po.TANH, po.RELU], 2, po.REGRESSION),   # row 2: layer 0 with fan-in 5 = features
+]
+
+
+def init_call_sequence(n_feat, hidden, acts, n_out, out_type):
+    """The Layer::initWeights calls of LayerBuilder::buildHiddenLayers + buildOutputLayer
+    (LayerBuilder.cpp:192-265) in order: (fan_in, n_out, act, kept layer index or -1).  A restart
+    (the first row whose activation is SIGMOID / RELU / LEAKY, any row for CLASSIFICATION) throws away
+    what was built and starts over without resetting prevLayerSize."""
+    calls, positive, prev, i = [], False, n_feat, 0
+    while i < len(hidden):
+        at = acts[i]
+        if not positive and (at in (po.SIGMOID, po.RELU, po.LEAKY) or out_type == po.CLASSIFICATION):
+            positive = True
+            calls = [(f, n, a, -1) for (f, n, a, _) in calls]
+            i = 0
+            continue
+        calls.append((prev, hidden[i], at, i))
+        prev = hidden[i]
+        i += 1
+    last = hidden[-1] if hidden else n_feat
+    calls.append((last, n_out, acts[len(hidden) - 1] if hidden else acts[0], len(hidden)))
+    return calls
+
+
+def init_sequences(td):
+    d = {}
+    for (name, seed, n_feat, hidden, acts, n_out, out_type) in INIT_CASES:
+        calls = init_call_sequence(n_feat, hidden, acts, n_out, out_type)
+        out = os.path.join(td, "seq.bin")
+        args = [str(v) for c in calls for v in c[:3]]
+        subprocess.check_call([po.REF_HARNESS, "xavierseq", str(seed), out] + args)
+        raw = np.fromfile(out, np.float32)
+        pos = 0
+        sizes = [n_feat] + hidden + [n_out]
+        for (fan, n, a, keep) in calls:
+            w = raw[pos:pos + fan * n].reshape(n, fan)
+            pos += fan * n
+            if keep >= 0:
+                assert fan >= sizes[keep]
+                d[f"{name}_W{keep}"] = w[:, :sizes[keep]].copy()   # surplus edges exist in the reference but are never visited
+        d[f"{name}_next"] = raw[pos:pos + 1].copy()
+        d[f"{name}_spec"] = np.array([seed, n_feat, n_out, out_type, len(hidden)] + hidden + acts, np.int32)
+        print("init", name, "calls", [(c[0], c[1], c[3]) for c in calls])
+    np.savez_compressed(os.path.join(HERE, "init_sequences.npz"), **d)
+
+
 def full_schedule_runs(td):
     for (name, sizes, acts, cost, mb, epochs, lr, mom, params, seed, data) in FULL_CASES:
         nl = len(sizes) - 1
@@ -178,6 +232,9 @@ def main():
     if not po.have_ref():
         raise SystemExit("oracle/_ref/ref_harness missing: run `make -C oracle ref` where /root/reference exists")
     with tempfile.TemporaryDirectory() as td:
+        if sys.argv[1:] == ["init"]:
+            return init_sequences(td)
+        init_sequences(td)
         full_schedule_runs(td)
         if sys.argv[1:] == ["full"]:
             return

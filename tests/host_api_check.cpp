@@ -4,6 +4,8 @@
 // Terminator, glades::train(&network, dataInput), read accuracy and epochs.
 //
 //   host_api_check xavier <seed> <fan_in> <n_out> <act> <out.bin>        (no GPU needed)
+//   host_api_check initseq <seed> <n_feat> <n_out> <output type> <out.bin> <input-row act> [<hidden size> <hidden-row act> ...]   (no GPU needed)
+//   host_api_check randpos <case.bin> <seed> <epochs> <k subnets> <concurrent 0|1> <out.bin>
 //   host_api_check nninfo <table.csv> <resaved.csv>                      (no GPU needed)
 //   host_api_check cmatrix <n> <pairs.bin> <out.bin>                     (no GPU needed)
 //   host_api_check ohe                                                   (no GPU needed)
@@ -34,6 +36,25 @@ static int do_xavier(int seed, int fi, int no, int act, const char* out)
     FILE* f = fopen(out, "wb");
     if (!f) return 1;
     put(W, f);
+    fclose(f);
+    return 0;
+}
+
+// the whole network's initial weights in the reference's sampling order, then rand() % 65536
+static int do_initseq(int seed, int nFeat, int nOut, int outType, const char* out, int n, char** spec)
+{
+    std::vector<HiddenLayerInfo*> hidden;
+    for (int k = 1; k + 1 < n; k += 2) hidden.push_back(new HiddenLayerInfo(atoi(spec[k]), 0.01f, 0.0f, 0.0f, 0.0f, 0.0f, atoi(spec[k + 1]), 0.0f));
+    NNInfo info("seq", new InputLayerInfo(1, 0.01f, 0.0f, 0.0f, 0.0f, 0.0f, atoi(spec[0]), 0.0f), hidden, new OutputLayerInfo(nOut, outType));
+    srand(seed);
+    std::vector<std::vector<float> > W;
+    std::string err;
+    if (!sampleInitialWeights(&info, nFeat, nOut, W, &err)) { printf("refused: %s\n", err.c_str()); return 7; }
+    FILE* f = fopen(out, "wb");
+    if (!f) return 1;
+    for (size_t l = 0; l < W.size(); ++l) put(W[l], f);
+    const float next = (float)(rand() % 65536);
+    fwrite(&next, 4, 1, f);
     fclose(f);
     return 0;
 }
@@ -488,8 +509,45 @@ static int do_meta(const char* in, int mode, int k, int epochs, const char* out)
     return 0;
 }
 
+// k subnets over one table whose weights are NOT injected, learning rate 0 (so that a trained network
+// still holds the weights it was built with), trained `epochs` epochs and tested once each, in the
+// reference's order or grouped: writes every subnet's weights and then rand() % 65536
+static int do_randpos(const char* in, int seed, int epochs, int k, int concurrent, const char* out)
+{
+    Case c;
+    int rc = read_case(in, c);
+    if (rc) return rc;
+    glades::init();
+    DenseInput di(c.X.data(), c.Y.data(), c.N, c.sizes[0], c.sizes[c.nl]);
+    for (int l = 0; l < c.nl; ++l) c.lr[l] = 0.0f;
+    srand(seed);
+    MetaNetwork meta("meta");
+    meta.setConcurrent(concurrent != 0);
+    for (int i = 0; i < k; ++i) {
+        meta.addSubnet(case_info(c));
+        NNetwork* n = meta.getSubnet(i);
+        n->setVerbose(false);
+        n->terminator.setEpoch(epochs);
+    }
+    meta.crossValidate(&di);   // every subnet: train, then its test pass
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    for (int i = 0; i < k; ++i) {
+        NNetwork* n = meta.getSubnet(i);
+        if (!n->getLastError().empty()) { fprintf(stderr, "subnet %d: %s\n", i, n->getLastError().c_str()); return 4; }
+        for (int l = 0; l < c.nl; ++l) { std::vector<float> w = n->getWeights(l); put(w, fo); }
+    }
+    const float next = (float)(rand() % 65536);
+    fwrite(&next, 4, 1, fo);
+    fclose(fo);
+    for (int i = 0; i < k; ++i) delete meta.getSubnet(i);
+    return 0;
+}
+
 int main(int argc, char** argv)
 {
+    if (argc >= 8 && !strcmp(argv[1], "initseq")) return do_initseq(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argc - 7, argv + 7);
+    if (argc >= 8 && !strcmp(argv[1], "randpos")) return do_randpos(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), atoi(argv[6]), argv[7]);
     if (argc >= 7 && !strcmp(argv[1], "xavier")) return do_xavier(atoi(argv[2]), atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6]);
     if (argc >= 4 && !strcmp(argv[1], "nninfo")) return do_nninfo(argv[2], argv[3]);
     if (argc >= 3 && !strcmp(argv[1], "nnedit")) return do_nnedit(argv[2]);

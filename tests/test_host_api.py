@@ -459,3 +459,73 @@ def test_dropout_through_the_class_api_follows_the_rand_stream():
         W = body[pos:pos + n].reshape(c["sizes"][l + 1], c["sizes"][l])
         pos += n + 1
         assert bits_equal(W, o.get_weights(l)), l
+
+
+@needs_bin
+def test_whole_network_initialisation_follows_the_reference_order():
+    """NNetwork::build's sampling (sampleInitialWeights) against sequences of the reference's compiled
+    Layer::initWeights under one srand: the order of LayerBuilder::buildHiddenLayers / buildOutputLayer
+    (LayerBuilder.cpp:192-265) with its restart -- layers thrown away with their draws spent, and the
+    first layer sampled again with the stale fan-in of the row the restart came from -- and where
+    libc's rand() stands afterwards."""
+    g = np.load(os.path.join(GOLDEN, "init_sequences.npz"), allow_pickle=False)
+    names = sorted(k[:-5] for k in g.files if k.endswith("_spec"))
+    assert len(names) == 4
+    with tempfile.TemporaryDirectory() as td:
+        for name in names:
+            spec = [int(v) for v in g[name + "_spec"]]
+            seed, n_feat, n_out, out_type, H = spec[:5]
+            hidden, acts = spec[5:5 + H], spec[5 + H:5 + 2 * H]
+            # rows of the table: the input row carries acts[0], hidden row k acts[k+1] (the last hidden row's is unused here)
+            args = [str(acts[0])]
+            for k in range(H):
+                args += [str(hidden[k]), str(acts[k + 1] if k + 1 < H else 0)]
+            out = os.path.join(td, "w.bin")
+            subprocess.check_call([BIN, "initseq", str(seed), str(n_feat), str(n_out), str(out_type), out] + args)
+            raw = np.fromfile(out, np.float32)
+            want = np.concatenate([g[f"{name}_W{l}"].ravel() for l in range(H + 1)] + [g[name + "_next"]])
+            assert bits_equal(raw, want), name
+
+
+@needs_bin
+def test_initialisation_the_reference_cannot_wire_is_refused():
+    """8 features, hidden rows TANH(4) then SIGMOID(5), regression: the reference restarts at row 1 and
+    samples the first layer with 4 of its 8 input edges (LayerBuilder.cpp:196-233).  Not modelled:
+    build says so instead of sampling something else."""
+    with tempfile.TemporaryDirectory() as td:
+        r = subprocess.run([BIN, "initseq", "5", "8", "2", "0", os.path.join(td, "w.bin"), "0", "4", "2", "5", "0"],
+                           stdout=subprocess.PIPE, text=True)
+    assert r.returncode == 7 and "4 of 8 input edges" in r.stdout
+
+
+@needs_bin
+@pytest.mark.gpu
+@pytest.mark.parametrize("concurrent", [0, 1])
+def test_rand_stream_between_subnets_follows_the_reference(concurrent):
+    """Three subnets that sample their own weights, cross-validated (train 3 epochs, test, next subnet)
+    with learning rate 0, so that each still holds its initial weights afterwards.  In the reference
+    every row of every pass throws one dart per input and hidden node even at dropout rate 0
+    (Layer::generateDropout, layer.cpp:102-134), so subnet k's sampler starts 4 x N x (nodes) draws after
+    subnet k-1's: the weights of all three, and rand() after the last, against the restated sampler
+    (bit-compared with the reference's compiled one) on the same libc stream.  One subnet after the
+    other and all in one launch give the same."""
+    c = load_case("window_4_5_3_1")
+    seed, epochs, k = 31, 3, 3
+    with tempfile.TemporaryDirectory() as td:
+        cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
+        write_case(cin, c)
+        subprocess.check_call([BIN, "randpos", cin, str(seed), str(epochs), str(k), str(concurrent), cout], stdout=subprocess.DEVNULL)
+        raw = np.fromfile(cout, np.float32)
+    sizes, nl = c["sizes"], c["nl"]
+    acts = [c["spec"].act[l] for l in range(nl)]
+    po.libc_srand(seed)
+    want = []
+    for _ in range(k):
+        for l in range(nl):    # all TANH, regression: no restart; the output layer takes the last hidden row's type
+            W = np.empty((sizes[l + 1], sizes[l]), np.float32)
+            po.lib().go_ref_xavier_layer(sizes[l], sizes[l + 1], acts[l] if l < nl - 1 else acts[nl - 2], W)
+            want.append(W.ravel())
+        for _ in range((epochs + 1) * c["N"] * sum(sizes[:-1])):
+            po.libc_rand()
+    want.append(np.array([po.libc_rand() % 65536], np.float32))
+    assert bits_equal(raw, np.concatenate(want))
