@@ -32,11 +32,23 @@ HBM_PEAK = 8000.0  # GB/s
 # (FETCH_SIZE x 2.000, WRITE_SIZE x 1.000); profiles/gemm_lowprec_pmc.md has the runs.  The
 # counters sit between L2 and the fabric, so lines re-fetched from the memory-side cache count again.
 # A workload / kernel pair that was not measured reports null.
-MEASURED_TRAFFIC_BYTES = {
-    # the 256 x 256-tile weight-gradient kernel (the four 4096 x 4096 layers): 328654.8 x 2 + 196608 KiB
-    ("cfg4", "gemm_bf16_wgrad_sgd"): int((328654.84 * 2.000 + 196608.0) * 1024),
-    ("cfg5", "gemm_fp8_forward"): int((789181.97 * 2.000 + 270336.0 * 1.000) * 1024),
-}
+TRAFFIC_PROFILE = "profiles/gemm_lowprec_pmc.md"
+
+
+def measured_traffic(workload, kernel):
+    """(bytes per launch, source) from the `traffic` lines of the committed counter summary, or (None, None):
+    `traffic <workload> <kernel> fetch_kib F write_kib W fetch_scale a write_scale b commit <hash>`."""
+    try:
+        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
+            t = line.split()
+            if len(t) >= 13 and t[0] == "traffic" and t[1] == workload and t[2] == kernel:
+                kv = dict(zip(t[3::2], t[4::2]))
+                byts = (float(kv["fetch_kib"]) * float(kv["fetch_scale"]) + float(kv["write_kib"]) * float(kv["write_scale"])) * 1024
+                return int(byts), f"{TRAFFIC_PROFILE}, rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of commit {kv['commit']} (not measured in this run)"
+    except (OSError, KeyError, ValueError):
+        pass
+    return None, None
+
 
 WORKLOADS = {
     "cfg4": dict(desc="bf16 train MLP 4096-4096-4096-4096-4096-1024 ReLU softmax-CE, batch 8192, SGD momentum 0.9, fp32 master",
@@ -139,7 +151,29 @@ def run_canonical(w, args):
     el = hip_timed(net, fn, args.steps)
     loss = net.last_metrics().loss if w["kind"] == "train" else None
     prof = kernel_profile(net, fn, min(args.steps, 5))
+    more = {}
+    if w["kind"] == "train" and getattr(args, "extras", False):
+        # the configuration's own schedule length, untouched by the short timed region's boost clocks
+        n_sus = 200
+        el_sus = hip_timed(net, fn, n_sus)
+        more["sustained"] = dict(steps=n_sus, ms_per_step=round(el_sus / n_sus * 1e3, 4), value=round(n_sus * B / el_sus, 1),
+                                 step_frac_of_peak=round(flops * B / (el_sus / n_sus) / 1e12 / PEAKS[w["dtype"]], 4))
     net.close()
+    if w["kind"] == "train" and w["dtype"] == "bf16" and getattr(args, "extras", False):
+        # the same warm-up + timed steps from the same start in fp32 (the path that is pinned to the CPU
+        # restatement): the low-precision run's last loss has to be the fp32 run's within 2e-2
+        ref = pg.Net(pg.make_spec(sizes, acts, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=pg.F32, batch=B, **hyper))
+        for l in range(nl):
+            ref.set_params(l, Ws[l])
+        ref.set_dataset_device(X.data_ptr(), Y.data_ptr(), N)
+        for s_ in range(args.warmup):
+            ref.train_step((s_ % nb) * B, B, want_metrics=False)
+        for s_ in range(args.steps):
+            ref.train_step((s_ % nb) * B, B, want_metrics=False)
+        ref_loss = ref.last_metrics().loss
+        ref.close()
+        rel = abs(loss - ref_loss) / abs(ref_loss)
+        more["loss_check"] = dict(bf16=loss, fp32=ref_loss, rel=round(rel, 6), tolerance=2e-2, ok=bool(rel <= 2e-2))
     # dominant kernel + its algorithmic FLOPs per launch
     gemm_names = {
         "bf16": {"gemm_bf16_forward": "fwd_hidden", "gemm_bf16_forward_out": "fwd_out", "gemm_bf16_dgrad": "dgrad",
@@ -163,16 +197,42 @@ def run_canonical(w, args):
     fl_launch = per_step[gemm_names[dom]] * psteps / kern[dom]["launches"]
     ach = fl_launch / (kern[dom]["avg_ms"] * 1e-3) / 1e12
     peak = PEAKS[w["dtype"]]
+    traffic, traffic_source = measured_traffic(w["name"], dom)
     roof = dict(bound="mfma", kernel=dom, achieved=round(ach, 2), peak=peak, unit="TFLOP/s", frac=round(ach / peak, 4),
-                traffic=MEASURED_TRAFFIC_BYTES.get((w["name"], dom)), flop_per_launch=fl_launch,
+                traffic=traffic, traffic_source=traffic_source, flop_per_launch=fl_launch,
                 avg_launch_ms=round(kern[dom]["avg_ms"], 4))
     total_ms = sum(k["total_ms"] for k in kern.values())
     breakdown = {n: round(k["total_ms"] / psteps, 4) for n, k in sorted(kern.items(), key=lambda kv: -kv[1]["total_ms"])}
     value = args.steps * B / el
     step_tflops = flops * B / (el / args.steps) / 1e12
     extra = dict(step_tflops=round(step_tflops, 2), step_frac_of_peak=round(step_tflops / peak, 4),
-                 kernel_ms_per_step=breakdown, kernel_ms_sum=round(total_ms / psteps, 4), final_loss=loss)
+                 kernel_ms_per_step=breakdown, kernel_ms_sum=round(total_ms / psteps, 4), final_loss=loss, **more)
     return value, el, roof, extra
+
+
+def vendor_gemm_rates(sizes, B, iters=30):
+    """The vendor library's plain bf16 GEMM (torch.matmul -> hipBLASLt: one output, no epilogue) on the
+    three product shapes of a hidden layer's training step: what this chip sustains on them under its
+    power limit, beside the published peak."""
+    import torch
+    dev = torch.device("cuda:0")
+    n = sizes[1]
+    shapes = {"forward / back-propagation (batch x n x n)": (B, n, n), "weight gradient (n x n x batch)": (n, n, B)}
+    out = {}
+    for name, (M, N, K) in shapes.items():
+        a = torch.randn((M, K), device=dev, dtype=torch.bfloat16)
+        b = torch.randn((N, K), device=dev, dtype=torch.bfloat16)
+        for _ in range(5):
+            torch.matmul(a, b.t())
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            torch.matmul(a, b.t())
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / iters
+        tf = 2.0 * M * N * K / dt / 1e12
+        out[name] = dict(ms=round(dt * 1e3, 4), tflops=round(tf, 1), frac_of_peak=round(tf / PEAKS["bf16"], 4))
+    return out
 
 
 def run_exact(w, args):
@@ -290,6 +350,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=None)
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS) + ["copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="cfg4: skip the untimed extras (fp32 loss check, 200-step sustained rate, cfg5 inference leg, vendor GEMM rates)")
     ap.add_argument("--subnets", type=int, default=1,
                     help="exact workloads: this many networks (MetaNetwork subnets) side by side in one launch; value is their sum")
     args = ap.parse_args()
@@ -320,12 +382,23 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    args.extras = args.workload == "cfg4" and not args.no_extras
     if w["kind"] == "exact":
         value, el, roof, extra = run_exact(w, args)
         unit_rows = w["rows"]
     else:
         value, el, roof, extra = run_canonical(w, args)
         unit_rows = w["batch"]
+    if args.extras:
+        # the metric's other half, inference samples/s, on its own configuration (cfg5), in the same run
+        w5 = dict(WORKLOADS["cfg5"], name="cfg5")
+        a5 = argparse.Namespace(steps=40, warmup=5, extras=False)
+        v5, el5, roof5, extra5 = run_canonical(w5, a5)
+        extra["infer"] = dict(metric="infer samples/sec", value=round(v5, 1), unit="samples/s", steps=a5.steps, warmup=a5.warmup,
+                              ms_per_step=round(el5 / a5.steps * 1e3, 4), dtype="fp8", workload="cfg5: " + w5["desc"],
+                              flop_per_sample=infer_flops_per_sample(w5["sizes"]), roofline=roof5,
+                              step_frac_of_peak=extra5["step_frac_of_peak"], kernel_ms_per_step=extra5["kernel_ms_per_step"])
+        extra["vendor_gemm"] = vendor_gemm_rates(w["sizes"], w["batch"])
     out = {
         "metric": "train samples/sec (fwd+bwd+update)" if w["kind"] != "infer" else "infer samples/sec",
         "value": round(value, 1), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

@@ -246,7 +246,9 @@ int check_spec(const ghip_net_spec* s)
         if (s->dtype < GHIP_F32 || s->dtype > GHIP_FP8_INFER) return fail(GHIP_EINVAL, "unknown dtype %d", s->dtype);
         if (s->dtype != GHIP_F32) {
             for (int l = 0; l <= s->n_layers; ++l)
-                if (s->sizes[l] % 256) return fail(GHIP_EINVAL, "bf16/fp8 paths need layer sizes that are multiples of 256 (layer %d is %d)", l, s->sizes[l]);
+                if (s->sizes[l] % 256)
+                    return fail(GHIP_EINVAL, "the bf16 / e4m3 paths tile layers in blocks of 256: layer %d has %d nodes; "
+                                "use dtype GHIP_F32 (any shape) or pad the layer to a multiple of 256", l, s->sizes[l]);
         }
     } else {
         return fail(GHIP_EINVAL, "unknown mode %d", s->mode);
@@ -1170,7 +1172,7 @@ int ghip_net_train_step(ghip_net* n, int64_t row0, int batch, ghip_metrics* host
     if (n->spec.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "fp8 networks are inference only");
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows [%lld,%lld) exceed the table (%lld rows)", (long long)row0, (long long)(row0 + batch), (long long)n->n_rows);
-    if (n->spec.dtype == GHIP_BF16 && (batch % 256)) return fail(GHIP_EINVAL, "bf16 path needs a batch that is a multiple of 256");
+    if (n->spec.dtype == GHIP_BF16 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 path takes batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     n->last_batch = batch;
     if (n->spec.dtype == GHIP_F32) TRY(step_f32(n, row0, batch));
@@ -1191,7 +1193,7 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
     const int64_t N = n->n_rows;
     if (batch > N) batch = (int)N;
     if (s.dtype != GHIP_F32 && ((batch % 256) || (N % batch) % 256))
-        return fail(GHIP_EINVAL, "bf16/fp8 paths need batches that are multiples of 256 (the last one, %lld rows, too)", (long long)(N % batch));
+        return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256, the last one (%lld rows here) too; use dtype GHIP_F32 or pad the table", (long long)(N % batch));
     TRY(reserve_batch(n, batch));
     if (s.dtype == GHIP_BF16) TRY(refresh_shadows(n));
     LAUNCH(n, "fill_pass_metrics", ghip_fill_f64(n->dAcc + 12, 4, 0.0, n->stream));
@@ -1266,7 +1268,7 @@ int ghip_net_forward(ghip_net* n, const float* host_X, int batch, float* host_ou
     HIP_TRY(hipSetDevice(g_device));
     if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
     const ghip_net_spec& s = n->spec;
-    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
+    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     HIP_TRY(hipMemcpyAsync(n->stageX, host_X, (size_t)batch * s.sizes[0] * 4, hipMemcpyHostToDevice, n->stream));
     uint16_t* xbf = nullptr;
@@ -1291,7 +1293,7 @@ int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_o
     if (!n->dX) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
     const ghip_net_spec& s = n->spec;
-    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
+    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     float* res = nullptr;
     TRY(forward_any(n, n->dX + row0 * s.sizes[0], n->Xbf ? n->Xbf + row0 * s.sizes[0] : nullptr, batch, &res));
@@ -1344,7 +1346,7 @@ int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* h
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
     const ghip_net_spec& s = n->spec;
-    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "bf16/fp8 paths need a batch that is a multiple of 256");
+    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     const int L = s.n_layers;
     float* P = nullptr;

@@ -180,6 +180,19 @@ def test_number_input_scaling_rules_by_hand():
         X, Y, _ = number_input(p)
         np.testing.assert_array_equal(X[:, 0], np.array([0.01, 0.99, np.float32(0.5) * np.float32(0.98) + np.float32(0.01)], np.float32))
         np.testing.assert_array_equal(Y, np.array([[0.99, 0.01], [0.01, 0.99], [0.99, 0.01]], np.float32))
+        # four rows, two numeric columns and a label, every expected cell worked out by hand from
+        # NumberInput.cpp:68-212: column 0 takes its own min / max (2, 8); column 1 starts both at 0, so
+        # its minimum is 0 and not 5 (5 / 20 = 0.25, not 0); cells go to x' * 0.98 + 0.01, labels to 0.99 / 0.01
+        open(p, "w").write("a,b,k\n2,5,u\n4,10,v\n6,15,u\n8,20,w\n")
+        X, Y, _ = number_input(p)
+        f = np.float32
+        third = (f(4) - f(2)) / f(6)
+        np.testing.assert_array_equal(X, np.array([
+            [f(0.01), f(0.25) * f(0.98) + f(0.01)],
+            [third * f(0.98) + f(0.01), f(0.5) * f(0.98) + f(0.01)],
+            [((f(6) - f(2)) / f(6)) * f(0.98) + f(0.01), f(0.75) * f(0.98) + f(0.01)],
+            [f(0.99), f(0.99)]], np.float32))
+        np.testing.assert_array_equal(Y, np.array([[0.99, 0.01, 0.01], [0.01, 0.99, 0.01], [0.99, 0.01, 0.01], [0.01, 0.01, 0.99]], np.float32))
         # z-score: mean over the rows, deviation with n - 1 (NumberInput.cpp:229-266)
         open(p, "w").write("a,b\n1,2\n2,4\n6,9\n")
         X, Y, _ = number_input(p, "zscore")
