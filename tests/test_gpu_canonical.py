@@ -157,3 +157,70 @@ def test_one_pass_call_equals_the_steps_one_by_one(sizes, acts, B, N):
     got_correct = int((want.argmax(1) == Y.argmax(1)).sum())
     assert ev.correct == got_correct
     a.close(); b.close()
+
+
+def test_cfg3_one_epoch_on_its_own_data():
+    """The medium benchmark configuration as written: 60 000 rows x 784 features U[0,1], labels = argmax of a
+    fixed random 784-256-10 ReLU teacher, network 784-1024-1024-10 ReLU + softmax cross-entropy, batch 512,
+    lr 0.05, momentum 0.9, L2 1e-4, one epoch = 117 steps.
+
+    Two fp32 runs of this schedule that sum in different orders drift apart (measured: 1e-4 relative in the
+    loss by step 13, 1e-3 by step 50, several per cent by step 100: lr 0.05 with momentum 0.9 is barely
+    stable here, the loss overshoots to 4.1 at step 3), so "equal after 117 free-running steps" is a
+    property no second implementation has.  What is checked instead holds every step of the epoch to the
+    bar: before each step the GPU network takes the CPU restatement's parameters and momentum, both take
+    the step, and the step's loss (1e-4 relative), its count of correct rows (within 1 of 512: a tie
+    between two nearly equal outputs may break either way) and, every tenth step, the updated weights
+    and biases (1e-4, plus the 3e-5 the L1/L2 terms' sign flips allow) must agree; then the logits of 512
+    held-out rows (1e-4 of their scale, same class on >= 99.5 % of all rows)."""
+    import pyglades as pg
+    print("cfg3 on its own data, one epoch, every step from the CPU run's state", flush=True)
+    rng = np.random.default_rng(1234)
+    sizes, acts = [784, 1024, 1024, 10], [po.RELU, po.RELU, po.SOFTMAX]
+    N, B = 60000, 512
+    X = rng.random((N, 784), dtype=np.float32)
+    T1 = rng.standard_normal((784, 256), dtype=np.float32) / np.float32(28.0)
+    T2 = rng.standard_normal((256, 10), dtype=np.float32) / np.float32(16.0)
+    Hc = X @ T1
+    Hc -= Hc.mean(0)                      # U[0,1] features have mean 1/2: centre the teacher's hidden layer so that all 10 classes occur
+    lab = (np.maximum(Hc, 0) @ T2).argmax(1)
+    assert len(np.unique(lab)) == 10
+    Y = np.eye(10, dtype=np.float32)[lab]
+    Ws = [rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l])) for l in range(3)]
+    kw = dict(lr=0.05, mom=0.9, wd2=1e-4, cost=po.CLASSIFICATION)
+    o = po.CanonNet(po.make_spec(sizes, acts, **kw))
+    g = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_CANONICAL, dtype=pg.F32, **kw))
+    for l in range(3):
+        o.set_params(l, Ws[l])
+    g.set_dataset(X, Y)
+    po.lib().go_set_threads(16)
+    steps = N // B
+    worst, differ, first = 0.0, 0, None
+    for s in range(steps):
+        for l in range(3):
+            W, b = o.get_params(l)
+            vW, vb = o.get_momentum(l)
+            g.set_params(l, W, b)
+            g.set_state(l, vW, vb)
+        mo = o.step(X[s * B:(s + 1) * B], Y[s * B:(s + 1) * B])
+        mg = g.train_step(s * B, B)
+        first = mo.loss if first is None else first
+        worst = max(worst, abs(mg.loss - mo.loss) / abs(mo.loss))
+        assert abs(mg.loss - mo.loss) <= 1e-4 * abs(mo.loss), (s, mg.loss, mo.loss)
+        assert abs(mg.correct - mo.correct) <= 1, (s, mg.correct, mo.correct)
+        differ += mg.correct != mo.correct
+        if s % 10 == 0 or s == steps - 1:
+            for l in range(3):
+                Wo, bo = o.get_params(l)
+                Wg, bg = g.get_params(l)
+                np.testing.assert_allclose(Wg, Wo, rtol=1e-4, atol=3e-5, err_msg=f"step {s} layer {l}")
+                np.testing.assert_allclose(bg, bo, rtol=1e-4, atol=3e-6, err_msg=f"step {s} layer {l} bias")
+    Xt = rng.random((512, 784), dtype=np.float32)
+    lo, lg = o.forward(Xt), g.forward(Xt)
+    agree = (lo.argmax(1) == lg.argmax(1)).mean()
+    print("steps", steps, "first / last loss %.4f / %.4f, worst relative loss gap of a step %.2e, steps whose correct count differs %d, "
+          "held-out max |dp| %.2e, class agreement %.4f" % (first, mo.loss, worst, differ, np.abs(lo - lg).max(), agree), flush=True)
+    assert mo.loss < first                                         # it trains
+    np.testing.assert_allclose(lg, lo, rtol=1e-4, atol=1e-4 * np.abs(lo).max())
+    assert agree >= 0.995
+    g.close()
