@@ -84,8 +84,9 @@ struct ghip_net {
     float* ownY = nullptr;
     int64_t n_rows = 0;
     uint16_t* Xbf = nullptr;  // bf16 copy of the table (BF16 / FP8_INFER)
-    uint16_t* XbfT = nullptr; // BF16 training: the same table transposed, [inputs][XbfT_ld]; a batch's columns are the
-    long long XbfT_ld = 0;    // B operand of the first layer's weight gradient as they lie (nullptr: transposed per step)
+    uint16_t* XbfT = nullptr; // BF16 training: the same table transposed and K-blocked, [rows / 64][inputs][64]: the planes of a
+                              // batch that starts on a multiple of 64 rows are the B operand of the first layer's weight
+                              // gradient as they lie (nullptr: the batch is transposed per step)
     // exact
     ExactLaunch ex;
     int ex_threads = 64;
@@ -555,7 +556,7 @@ int forward_bf16(ghip_net* n, const uint16_t* X, int B)
         g.fp8 = 0; g.bias = n->b[l];
         g.act = out_act(s, l, &g.act_param);
         if (l < L - 1) {
-            g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = n->HT[l + 1];
+            g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = n->HT[l + 1]; g.outT_blocked = 1;
             LAUNCH(n, "gemm_bf16_forward", ghip_gemm_lp(g, n->stream));
         } else {
             g.epilogue = LP_FWD_F32; g.out = n->logits;
@@ -586,7 +587,8 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
         if (l > 0) {
             memset(&g, 0, sizeof(g));
             g.A = n->D[l + 1]; g.B = n->WhT[l]; g.M = B; g.N = ni; g.K = no;
-            g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.aux = n->H[l]; g.colsum = n->csum[l];
+            g.ldb = 64; g.kstrideB = (long long)ni * 128;   // W^T is kept K-blocked: [n_out / 64][n_in][64]
+            g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.outT_blocked = 1; g.aux = n->H[l]; g.colsum = n->csum[l];
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1];
             LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));
         }
@@ -596,9 +598,12 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
         else
             LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
         memset(&g, 0, sizeof(g));
+        // both operands K-blocked over the batch: [B / 64][nodes][64], a tile's stage one contiguous block
         g.A = n->DT[l + 1]; g.B = n->HT[l]; g.M = no; g.N = ni; g.K = B;
-        if (l == 0 && inT) { g.B = n->XbfT + row0; g.ldb = (int)n->XbfT_ld; }
-        g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l];
+        g.lda = 64; g.kstrideA = (long long)no * 128;
+        g.ldb = 64; g.kstrideB = (long long)ni * 128;
+        if (l == 0 && inT) g.B = n->XbfT + (row0 / 64) * (long long)ni * 64;
+        g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l]; g.outT_blocked = 1;
         g.master = n->W[l]; g.mom = n->vW[l];
         g.lr = s.lr[l]; g.momf = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l]; g.gscale = 1.0f / (float)B;
         // the profile keeps the two tile sizes apart: they are different kernels with different rooflines
@@ -955,23 +960,20 @@ static int make_bf16_table(ghip_net* n)
     if (s.mode != GHIP_MODE_CANONICAL || s.dtype == GHIP_F32) return 0;
     dfree(n->Xbf);
     dfree(n->XbfT);
-    n->XbfT_ld = 0;
     TRY(dalloc(&n->Xbf, (size_t)n->n_rows * s.sizes[0]));
     // Training reads each batch transposed as well (the weight gradient of the first layer runs over the
-    // batch): the whole table is kept that way, rows padded by one cache line so that the rows of a tile do
-    // not all start in the same memory channel.  A table too large for that is transposed batch by batch.
-    const long long ldT = ((n->n_rows + 63) / 64) * 64 + 64;
-    const size_t bytesT = (size_t)s.sizes[0] * (size_t)ldT * 2;
+    // batch): the whole table is kept that way, in planes of 64 rows.  A table too large for that is
+    // transposed batch by batch.
+    const size_t bytesT = (size_t)s.sizes[0] * (size_t)(((n->n_rows + 63) / 64) * 64) * 2;
     if (s.dtype == GHIP_BF16 && n->n_rows >= 64 && bytesT <= ((size_t)16 << 30)) {
-        if (hipMalloc((void**)&n->XbfT, bytesT) == hipSuccess) n->XbfT_ld = ldT;
-        else { n->XbfT = nullptr; (void)hipGetLastError(); }
+        if (hipMalloc((void**)&n->XbfT, bytesT) != hipSuccess) { n->XbfT = nullptr; (void)hipGetLastError(); }
     }
     // convert in slabs of rows to keep the grid small
     const int64_t slab = 65536;
     for (int64_t r = 0; r < n->n_rows; r += slab) {
         const int rows = (int)((n->n_rows - r) < slab ? (n->n_rows - r) : slab);
-        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d_ld(n->dX + r * s.sizes[0], n->Xbf + r * s.sizes[0],
-                                                             n->XbfT ? n->XbfT + r : nullptr, ldT, rows, s.sizes[0], n->stream));
+        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d(n->dX + r * s.sizes[0], n->Xbf + r * s.sizes[0],
+                                                          n->XbfT ? n->XbfT + (r / 64) * s.sizes[0] * 64 : nullptr, rows, s.sizes[0], n->stream));
     }
     return 0;
 }

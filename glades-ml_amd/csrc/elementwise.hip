@@ -240,7 +240,7 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
     }
 }
 
-// bf16 delta^T [n][B]: one wavefront per channel, 16-byte loads (B is a multiple of 8)
+// bf16 delta^T, K-blocked [B / 64][n][64]: one wavefront per channel, 16-byte loads (B is a multiple of 64)
 __global__ void __launch_bounds__(256)
 bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* __restrict__ bias,
                          float* __restrict__ vb, float lr, float mom)
@@ -248,7 +248,8 @@ bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* _
     const int lane = threadIdx.x & 63;
     const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (o >= n) return;
-    const uint4* row = reinterpret_cast<const uint4*>(DT + (long long)o * B);
+    // eight 16-byte pieces per plane of 64 batch rows; plane p of channel o starts at (p * n + o) * 64
+    auto piece = [&](int k) { return *reinterpret_cast<const uint4*>(DT + ((long long)(k >> 3) * n + o) * 64 + (k & 7) * 8); };
     float s4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     const int nq = B >> 3;
     for (int k0 = 0; k0 < nq; k0 += 256) {  // four independent 16-byte loads in flight per lane
@@ -256,7 +257,7 @@ bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* _
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int k = k0 + u * 64 + lane;
-            q[u] = (k < nq) ? row[k] : make_uint4(0u, 0u, 0u, 0u);
+            q[u] = (k < nq) ? piece(k) : make_uint4(0u, 0u, 0u, 0u);
         }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
@@ -304,12 +305,12 @@ __global__ void __launch_bounds__(256) fill_kernel(T* p, long long n, T v)
     for (; i < n; i += stride) p[i] = v;
 }
 
-// 64x64 tile through LDS: dst[r][c] = bf16(src[r][c]) and dstT[c][r] (rows of dstT are ldT elements apart);
-// src fp32 or bf16
+// 64x64 tile through LDS: dst[r][c] = bf16(src[r][c]) and the K-blocked transposed copy
+// dstT[r / 64][c][r % 64]; src fp32 or bf16
 template <typename SrcT>
 __global__ void __launch_bounds__(256)
 convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ dst,
-                         uint16_t* __restrict__ dstT, int rows, int cols, long long ldT)
+                         uint16_t* __restrict__ dstT, int rows, int cols)
 {
     __shared__ uint16_t tile[64][64 + 2];
     const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
@@ -328,13 +329,14 @@ convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ ds
     if (dstT) {
         for (int j = ty; j < 64; j += 4) {
             const int c = c0 + j, r = r0 + tx;
-            if (r < rows && c < cols) dstT[(long long)c * ldT + r] = tile[tx][j];
+            if (r < rows && c < cols) dstT[((long long)blockIdx.y * cols + c) * 64 + tx] = tile[tx][j];
         }
     }
 }
 
-// bf16 transposition with 16-byte global accesses: a 64 x 64 tile enters LDS row by row (8 lanes
-// per source row) and leaves column by column (each lane gathers 8 values of one source column).
+// bf16 transposition (K-blocked destination, dstT[r / 64][c][r % 64]) with 16-byte global accesses: a
+// 64 x 64 tile enters LDS row by row (8 lanes per source row) and leaves column by column (each lane
+// gathers 8 values of one source column; a tile's 64 destination rows of 128 bytes are contiguous).
 // rows and cols are multiples of 64 here; other shapes take the kernel above.
 __global__ void __launch_bounds__(256)
 bf16_transpose64_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dstT, int rows, int cols)
@@ -357,7 +359,7 @@ bf16_transpose64_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__
 #pragma unroll
         for (int k = 0; k < 4; ++k)
             o[k] = (uint32_t)tile[sub * 8 + 2 * k][c] | ((uint32_t)tile[sub * 8 + 2 * k + 1][c] << 16);
-        *reinterpret_cast<uint4*>(dstT + (long long)(c0 + c) * rows + r0 + sub * 8) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4*>(dstT + ((long long)blockIdx.y * cols + c0 + c) * 64 + sub * 8) = make_uint4(o[0], o[1], o[2], o[3]);
     }
 }
 
@@ -555,13 +557,8 @@ hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream
 
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s)
 {
-    return ghip_f32_to_bf16_2d_ld(src, dst, dstT, rows, rows, cols, s);
-}
-
-hipError_t ghip_f32_to_bf16_2d_ld(const float* src, uint16_t* dst, uint16_t* dstT, long long ldT, int rows, int cols, hipStream_t s)
-{
     dim3 grid((cols + 63) / 64, (rows + 63) / 64);
-    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, dst, dstT, rows, cols, ldT);
+    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, dst, dstT, rows, cols);
     return hipGetLastError();
 }
 
@@ -572,7 +569,7 @@ hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, in
         hipLaunchKernelGGL(bf16_transpose64_kernel, grid, dim3(256), 0, s, src, dstT, rows, cols);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols, (long long)rows);
+    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols);
     return hipGetLastError();
 }
 

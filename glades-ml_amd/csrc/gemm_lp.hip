@@ -179,6 +179,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     const long long ldk = (long long)g.K * ES;                        // bytes of K per row
     const long long lda = (long long)(g.lda ? g.lda : g.K) * ES;      // row pitches in bytes
     const long long ldb = (long long)(g.ldb ? g.ldb : g.K) * ES;
+    const long long ksA = g.kstrideA ? g.kstrideA : SKB, ksB = g.kstrideB ? g.kstrideB : SKB;  // bytes from stage to stage
     const unsigned char* gA = (const unsigned char*)g.A + (long long)bm * lda;
     const unsigned char* gB = (const unsigned char*)g.B + (long long)bn * ldb;
 
@@ -215,11 +216,11 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     const unsigned char* const gAw = gA + (long long)(ws * PWA * 8) * lda;
     const unsigned char* const gBw = gB + (long long)(ws * PWB * 8) * ldb;
     auto dmaA = [&](int slot, int st, int jj) {
-        const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;  // past the end: refetch, never read
+        const long long kb = (long long)(st < nk ? st : nk - 1) * ksA;  // past the end: refetch, never read
         lds_direct_16s(gAw + (long long)(jj * 8) * lda + kb, voffA[jj & 1], smem_u + slot * SLOT + (ws * PWA + jj) * 1024);
     };
     auto dmaB = [&](int slot, int st, int jj) {
-        const long long kb = (long long)(st < nk ? st : nk - 1) * SKB;
+        const long long kb = (long long)(st < nk ? st : nk - 1) * ksB;
         lds_direct_16s(gBw + (long long)(jj * 8) * ldb + kb, voffB[jj & 1], smem_u + slot * SLOT + (ws * PWB + jj) * 1024);
     };
     // X is the operand with two stages of lead, Y the one with one: A and B, except in the 128 x 128-tile
@@ -492,13 +493,19 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_s_barrier();
             constexpr int LPR = TM / 8, RPI = 64 / LPR;   // lanes per transposed row, rows per instruction
-            unsigned char* dstT = (unsigned char*)g.outT + ((long long)bn * M + bm) * 2;
+            // plain: outT[n][m]; K-blocked for the weight gradient (K = m): outT[m / 64][n][m % 64], where
+            // the 128-byte pieces of a transposed row go to planes N x 128 bytes apart and the tile's rows
+            // follow one another within a plane
+            unsigned char* dstT = g.outT_blocked ? (unsigned char*)g.outT + ((long long)(bm >> 6) * N + bn) * 128
+                                                 : (unsigned char*)g.outT + ((long long)bn * M + bm) * 2;
+            const long long rowT = g.outT_blocked ? 128 : (long long)M * 2;
+            const long long planeT = g.outT_blocked ? (long long)N * 128 : 128;
 #pragma unroll
             for (int i = 0; i < (TN / 8) / RPI; ++i) {
                 const int nl = w * (TN / 8) + i * RPI + lane / LPR;
                 const int lc = (lane % LPR) << 4;
                 const v4i val = *reinterpret_cast<const v4i*>(smem + nl * PITCH_T + lc);
-                *reinterpret_cast<v4i*>(dstT + (long long)nl * M * 2 + lc) = val;
+                *reinterpret_cast<v4i*>(dstT + (long long)nl * rowT + (long long)(lc >> 7) * planeT + (lc & 127)) = val;
             }
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_s_barrier();
@@ -625,7 +632,10 @@ hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
     if (!ghip_gemm_lp_shape_ok(a_.M, a_.N, a_.K, a_.fp8)) return hipErrorInvalidValue;
     // the LDS-direct loads move 16 bytes per lane: operand rows start on 16-byte boundaries, pitches cover K
     const int es = a_.fp8 ? 1 : 2;
-    if ((a_.lda && (a_.lda < a_.K || ((long long)a_.lda * es) % 16)) || (a_.ldb && (a_.ldb < a_.K || ((long long)a_.ldb * es) % 16)) ||
+    // (a K-blocked operand's pitch is one stage's 128 bytes and its stages lie kstride bytes apart)
+    const bool pitchA_ok = a_.kstrideA ? ((long long)a_.lda * es == 128 && a_.kstrideA % 128 == 0) : (!a_.lda || a_.lda >= a_.K);
+    const bool pitchB_ok = a_.kstrideB ? ((long long)a_.ldb * es == 128 && a_.kstrideB % 128 == 0) : (!a_.ldb || a_.ldb >= a_.K);
+    if (!pitchA_ok || !pitchB_ok || (a_.lda && ((long long)a_.lda * es) % 16) || (a_.ldb && ((long long)a_.ldb * es) % 16) ||
         (((uintptr_t)a_.A | (uintptr_t)a_.B) % 16))
         return hipErrorInvalidValue;
     GemmLpArgs a = a_;

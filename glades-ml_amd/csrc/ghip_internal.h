@@ -339,6 +339,13 @@ struct GemmLpArgs {
     const void* A; const void* B;    // [M][K], [N][K], K contiguous; bf16 or e4m3
     int M, N, K;
     int lda, ldb;                     // row pitches of A and B in elements (0: K)
+    // K-blocked operands: bytes between one stage's 128 bytes of a row and the next stage's (0: they follow
+    // each other in the row).  With a pitch of 128 bytes and kstride = rows x 128 an operand lies as
+    // [K bytes / 128][rows][128 bytes]: every stage of a tile is ONE contiguous block of memory instead of
+    // 256 lines a row pitch apart.  The weight gradient's operands (activations and deltas transposed, K =
+    // the batch) are kept that way: they come from HBM, where scattered lines cost a DRAM page each.
+    long long kstrideA, kstrideB;
+    int outT_blocked;                 // outT is written K-blocked for the product that will read it: [M / 64][N][64]
     int fp8;                          // 0: bf16 operands, 1: e4m3 operands
     int epilogue;
     void* out; void* outT;            // see LpEpilogue; outT may be NULL
@@ -364,11 +371,12 @@ hipError_t ghip_gemm_lp(const GemmLpArgs& a, hipStream_t s);
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8);
 int ghip_gemm_lp_tile_m(int M, int N);  // rows per tile the launcher picks for this product
 
+// Transposed bf16 copies are K-blocked for the weight-gradient product (see GemmLpArgs::kstrideA):
+// element (row r, column c) of a [rows][cols] source lies at ((r / 64) * cols + c) * 64 + r % 64 of dstT,
+// i.e. dstT is [ceil(rows / 64)][cols][64].
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
-// the same with the rows of dstT ldT elements apart (a slab of rows of a table whose transposed copy is kept whole)
-hipError_t ghip_f32_to_bf16_2d_ld(const float* src, uint16_t* dst, uint16_t* dstT, long long ldT, int rows, int cols, hipStream_t s);
 hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s);
-// bias update from bf16 delta^T [n][B] rows (contiguous): gb[o] = sum_b
+// bias update from bf16 delta^T, K-blocked [B / 64][n][64]: gb[o] = sum_b
 hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vbias, float lr,
                                   float mom, hipStream_t s);
 // the same from per-tile-row partial column sums [tiles][n] (written by the LP_DGRAD epilogue)
