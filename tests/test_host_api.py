@@ -11,7 +11,8 @@ import pyoracle as po
 from helpers import GOLDEN, bits_equal, load_case
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-BIN = os.path.join(ROOT, "tests", "bin", "host_api_check")
+# GLADES_HOST_API_CHECK: another build of the driver (e.g. one with host-side sanitizers)
+BIN = os.environ.get("GLADES_HOST_API_CHECK", os.path.join(ROOT, "tests", "bin", "host_api_check"))
 needs_bin = pytest.mark.skipif(not os.path.exists(BIN), reason="tests/bin/host_api_check not built (python glades-ml_amd/build.py)")
 
 
