@@ -227,7 +227,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     // weight gradient, which runs 10 % faster with its B operand (the activations, a forward pass old)
     // in the place with more lead; the 256 x 256-tile kernels measure the same either way
     constexpr bool kSwap = !FP8 && EPI == LP_WGRAD_SGD && TM == 128;
-    static_assert(PWA == PWB, "either operand can take either place in the ring");
+    static_assert(!kSwap || PWA == PWB, "operands that change places in the ring have equally many slabs");
     auto dmaX = [&](int slot, int st, int jj) { if constexpr (kSwap) dmaB(slot, st, jj); else dmaA(slot, st, jj); };
     auto dmaY = [&](int slot, int st, int jj) { if constexpr (kSwap) dmaA(slot, st, jj); else dmaB(slot, st, jj); };
     constexpr int OA = kSwap ? 1 : 0, OB = kSwap ? 0 : 1;  // places of A and B within a stage's pair of slots
@@ -582,10 +582,21 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
 // 256 x 256 tiles when they give every CU at least one workgroup, else 128 x 128.
 constexpr int kCUs = 256;
 inline bool use_small_tile(int M, int N) { return (long long)(M / 256) * (N / 256) < kCUs; }
+// In between, for the fp32-output forward product of a narrow last layer: 256 x 128 tiles where those fill the
+// CUs.  Two 128 x 128 workgroups per CU ask the global->LDS path for 124 bytes per clock at the matrix
+// cores' rate, twice what it moves; one 256 x 128 workgroup asks for 46.
+inline bool use_tall_tile(int M, int N) { return (long long)(M / 256) * (N / 128) >= kCUs; }
 
 template <bool FP8, int EPI>
 hipError_t launch(const GemmLpArgs& a, hipStream_t s)
 {
+    if constexpr (!FP8 && EPI == LP_FWD_F32) {
+        if (use_small_tile(a.M, a.N) && use_tall_tile(a.M, a.N)) {
+            const int nb = (a.M / 256) * (a.N / 128);
+            hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI, 4, 1>), dim3(nb), dim3(NT), 0, s, a);
+            return hipGetLastError();
+        }
+    }
     if (use_small_tile(a.M, a.N)) {
         const int nb = (a.M / 128) * (a.N / 128);
         hipLaunchKernelGGL((gemm_lp_kernel<FP8, EPI, 2, 1>), dim3(nb), dim3(NT), 0, s, a);
