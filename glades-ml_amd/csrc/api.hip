@@ -77,6 +77,11 @@ struct ghip_net {
     ghip_net_spec spec;
     hipStream_t stream = nullptr;
     int L = 0;
+    // Layer widths as the device holds them.  The bf16 / e4m3 products work on tiles of 256: there every width is
+    // rounded up to a multiple of 256 and the units added are kept at zero (zero weights, zero bias, activation
+    // stored as 0), so they change no result.  fp32: the widths of the spec.
+    int ps[GHIP_MAX_LAYERS + 1] = {};
+    int64_t table_rows = 0;   // rows the bf16 table holds: those of the dataset plus zero rows a padded last batch may read
     // dataset
     const float* dX = nullptr;
     const float* dY = nullptr;
@@ -223,6 +228,21 @@ void prof_collect(ghip_net* n)
 }
 
 int pow2ceil(int v) { int p = 1; while (p < v) p <<= 1; return p; }
+int pad256(int v) { return (v + 255) / 256 * 256; }
+bool low_prec(const ghip_net* n) { return n->spec.mode == GHIP_MODE_CANONICAL && n->spec.dtype != GHIP_F32; }
+// rows a batch occupies on the device: low-precision products take whole tiles of 256 rows; the rows added
+// carry zero deltas, so they add nothing to a gradient, and their outputs are not read
+int pad_batch(const ghip_net* n, int B) { return low_prec(n) ? pad256(B) : B; }
+void set_padded_sizes(ghip_net* n)
+{
+    for (int l = 0; l <= n->spec.n_layers; ++l) n->ps[l] = low_prec(n) ? pad256(n->spec.sizes[l]) : n->spec.sizes[l];
+}
+// host <-> device copy of a rows x cols fp32 matrix whose device copy has row pitch dev_ld (>= cols)
+hipError_t copy_matrix(float* dev, int dev_ld, float* host, int rows, int cols, bool to_device, hipStream_t st)
+{
+    if (to_device) return hipMemcpy2DAsync(dev, (size_t)dev_ld * 4, host, (size_t)cols * 4, (size_t)cols * 4, rows, hipMemcpyHostToDevice, st);
+    return hipMemcpy2DAsync(host, (size_t)cols * 4, dev, (size_t)dev_ld * 4, (size_t)cols * 4, rows, hipMemcpyDeviceToHost, st);
+}
 int ilog2(int v) { int l = 0; while ((1 << l) < v) ++l; return l; }
 
 bool is_canon(const ghip_net* n) { return n->spec.mode == GHIP_MODE_CANONICAL; }
@@ -245,12 +265,6 @@ int check_spec(const ghip_net_spec* s)
         if (s->dtype != GHIP_F32) return fail(GHIP_EINVAL, "exact mode is fp32 only");
     } else if (s->mode == GHIP_MODE_CANONICAL) {
         if (s->dtype < GHIP_F32 || s->dtype > GHIP_FP8_INFER) return fail(GHIP_EINVAL, "unknown dtype %d", s->dtype);
-        if (s->dtype != GHIP_F32) {
-            for (int l = 0; l <= s->n_layers; ++l)
-                if (s->sizes[l] % 256)
-                    return fail(GHIP_EINVAL, "the bf16 / e4m3 paths tile layers in blocks of 256: layer %d has %d nodes; "
-                                "use dtype GHIP_F32 (any shape) or pad the layer to a multiple of 256", l, s->sizes[l]);
-        }
     } else {
         return fail(GHIP_EINVAL, "unknown mode %d", s->mode);
     }
@@ -325,17 +339,18 @@ int setup_exact(ghip_net* n)
 int setup_canon(ghip_net* n)
 {
     const ghip_net_spec& s = n->spec;
+    const int* ps = n->ps;
     for (int l = 0; l < s.n_layers; ++l) {
-        size_t cnt = (size_t)s.sizes[l] * s.sizes[l + 1];
+        size_t cnt = (size_t)ps[l] * ps[l + 1];
         TRY(dalloc(&n->W[l], cnt));
-        TRY(dalloc(&n->b[l], (size_t)s.sizes[l + 1]));
+        TRY(dalloc(&n->b[l], (size_t)ps[l + 1]));
         HIP_TRY(hipMemsetAsync(n->W[l], 0, cnt * 4, n->stream));
-        HIP_TRY(hipMemsetAsync(n->b[l], 0, (size_t)s.sizes[l + 1] * 4, n->stream));
+        HIP_TRY(hipMemsetAsync(n->b[l], 0, (size_t)ps[l + 1] * 4, n->stream));
         if (s.dtype != GHIP_FP8_INFER) {
             TRY(dalloc(&n->vW[l], cnt));
-            TRY(dalloc(&n->vb[l], (size_t)s.sizes[l + 1]));
+            TRY(dalloc(&n->vb[l], (size_t)ps[l + 1]));
             HIP_TRY(hipMemsetAsync(n->vW[l], 0, cnt * 4, n->stream));
-            HIP_TRY(hipMemsetAsync(n->vb[l], 0, (size_t)s.sizes[l + 1] * 4, n->stream));
+            HIP_TRY(hipMemsetAsync(n->vb[l], 0, (size_t)ps[l + 1] * 4, n->stream));
         }
         if (s.dtype == GHIP_BF16) {
             TRY(dalloc(&n->Wh[l], cnt));
@@ -343,7 +358,7 @@ int setup_canon(ghip_net* n)
         }
         if (s.dtype == GHIP_FP8_INFER) {
             TRY(dalloc(&n->Wq[l], cnt));
-            TRY(dalloc(&n->wscale[l], (size_t)s.sizes[l + 1]));
+            TRY(dalloc(&n->wscale[l], (size_t)ps[l + 1]));
         }
     }
     TRY(dalloc(&n->dAcc, 16));  // two alternating banks per step, one for softmax-only launches, one per pass over the table
@@ -364,15 +379,26 @@ void free_batch_buffers(ghip_net* n)
     n->cap_batch = 0;
 }
 
-int reserve_batch(ghip_net* n, int B)
+// zeroed device memory (the padded parts of low-precision buffers are read and never written)
+template <typename T>
+int dalloc_zero(ghip_net* n, T** p, size_t count)
 {
+    TRY(dalloc(p, count));
+    HIP_TRY(hipMemsetAsync(*p, 0, (count ? count : 1) * sizeof(T), n->stream));
+    return 0;
+}
+
+int reserve_batch(ghip_net* n, int batch)
+{
+    const int B = pad_batch(n, batch);
     if (B <= n->cap_batch) return 0;
     (void)hipStreamSynchronize(n->stream);
     free_batch_buffers(n);
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
+    const int* ps = n->ps;
     int maxw = 0;
-    for (int l = 0; l <= L; ++l) if (s.sizes[l] > maxw) maxw = s.sizes[l];
+    for (int l = 0; l <= L; ++l) if (ps[l] > maxw) maxw = ps[l];
     if (s.dtype == GHIP_F32) {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
         for (int l = 1; l <= L; ++l) {
@@ -387,27 +413,28 @@ int reserve_batch(ghip_net* n, int B)
         }
     } else if (s.dtype == GHIP_BF16) {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
-        TRY(dalloc(&n->HT[0], (size_t)B * s.sizes[0]));
+        TRY(dalloc_zero(n, &n->HT[0], (size_t)B * ps[0]));
         for (int l = 1; l <= L; ++l) {
             if (l < L) {
-                TRY(dalloc(&n->H[l], (size_t)B * s.sizes[l]));
-                TRY(dalloc(&n->HT[l], (size_t)B * s.sizes[l]));
+                TRY(dalloc_zero(n, &n->H[l], (size_t)B * ps[l]));
+                TRY(dalloc_zero(n, &n->HT[l], (size_t)B * ps[l]));
             }
-            TRY(dalloc(&n->D[l], (size_t)B * s.sizes[l]));
-            TRY(dalloc(&n->DT[l], (size_t)B * s.sizes[l]));
-            if (l < L) TRY(dalloc(&n->csum[l], (size_t)((B + 127) / 128) * s.sizes[l]));
+            // the output deltas are written for the units and rows the batch has; the rest of D[L] stays zero
+            TRY(dalloc_zero(n, &n->D[l], (size_t)B * ps[l]));
+            TRY(dalloc_zero(n, &n->DT[l], (size_t)B * ps[l]));
+            if (l < L) TRY(dalloc(&n->csum[l], (size_t)((B + 127) / 128) * ps[l]));
         }
-        TRY(dalloc(&n->logits, (size_t)B * s.sizes[L]));
+        TRY(dalloc_zero(n, &n->logits, (size_t)B * ps[L]));
     } else {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
-        TRY(dalloc(&n->Aq[0], (size_t)B * maxw));
-        TRY(dalloc(&n->Aq[1], (size_t)B * maxw));
+        TRY(dalloc_zero(n, &n->Aq[0], (size_t)B * maxw));
+        TRY(dalloc_zero(n, &n->Aq[1], (size_t)B * maxw));
         TRY(dalloc(&n->ascale[0], (size_t)B));
         TRY(dalloc(&n->ascale[1], (size_t)B));
         TRY(dalloc(&n->amax_bits, (size_t)B));
         n->amax_clean = false;
-        TRY(dalloc(&n->Hq, (size_t)B * maxw));
-        TRY(dalloc(&n->out8, (size_t)B * s.sizes[L]));
+        TRY(dalloc_zero(n, &n->Hq, (size_t)B * maxw));
+        TRY(dalloc_zero(n, &n->out8, (size_t)B * ps[L]));
     }
     n->cap_batch = B;
     return 0;
@@ -419,7 +446,7 @@ int refresh_shadows(ghip_net* n)
     if (!n->shadow_dirty) return 0;
     const ghip_net_spec& s = n->spec;
     for (int l = 0; l < s.n_layers; ++l)
-        LAUNCH(n, "f32_to_bf16_transpose", ghip_f32_to_bf16_2d(n->W[l], n->Wh[l], n->WhT[l], s.sizes[l + 1], s.sizes[l], n->stream));
+        LAUNCH(n, "f32_to_bf16_transpose", ghip_f32_to_bf16_2d(n->W[l], n->Wh[l], n->WhT[l], n->ps[l + 1], n->ps[l], n->stream));
     n->shadow_dirty = false;
     return 0;
 }
@@ -468,7 +495,7 @@ DeltaArgs delta_args(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
     DeltaArgs a;
     memset(&a, 0, sizeof(a));
     a.P = P; a.Y = Y; a.D = D; a.Dbf = Dbf; a.DbfT = nullptr;
-    a.B = B; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
+    a.B = B; a.n = s.sizes[L]; a.ldp = n->ps[L]; a.ldy = s.sizes[L]; a.ldd = n->ps[L];
     a.act = s.act[L - 1]; a.act_param = s.act_param[L - 1]; a.cost = s.cost;
     a.acc = n->dAcc + 4 * bank; a.acc_clear = n->dAcc + 4 * (bank ^ 1);
     a.cm = n->cm;
@@ -544,19 +571,23 @@ int step_f32(ghip_net* n, int64_t row0, int B)
 }
 
 // ---- canonical bf16 ----
-int forward_bf16(ghip_net* n, const uint16_t* X, int B)
+// X: the batch's rows in bf16 at pitch ps[0], pad_batch(batch) of them readable
+int forward_bf16(ghip_net* n, const uint16_t* X, int batch)
 {
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
+    const int* ps = n->ps;
+    const int B = pad_batch(n, batch);
     const uint16_t* in = X;
     for (int l = 0; l < L; ++l) {
         GemmLpArgs g;
         memset(&g, 0, sizeof(g));
-        g.A = in; g.B = n->Wh[l]; g.M = B; g.N = s.sizes[l + 1]; g.K = s.sizes[l];
+        g.A = in; g.B = n->Wh[l]; g.M = B; g.N = ps[l + 1]; g.K = ps[l];
         g.fp8 = 0; g.bias = n->b[l];
         g.act = out_act(s, l, &g.act_param);
         if (l < L - 1) {
             g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = n->HT[l + 1]; g.outT_blocked = 1;
+            g.n_valid = ps[l + 1] != s.sizes[l + 1] ? s.sizes[l + 1] : 0;
             LAUNCH(n, "gemm_bf16_forward", ghip_gemm_lp(g, n->stream));
         } else {
             g.epilogue = LP_FWD_F32; g.out = n->logits;
@@ -567,22 +598,27 @@ int forward_bf16(ghip_net* n, const uint16_t* X, int B)
     return 0;
 }
 
-int step_bf16(ghip_net* n, int64_t row0, int B)
+int step_bf16(ghip_net* n, int64_t row0, int batch)
 {
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
+    const int* ps = n->ps;
+    const int B = pad_batch(n, batch);   // rows of every product; the means below divide by the batch's own count
     TRY(refresh_shadows(n));
-    const uint16_t* X = n->Xbf + row0 * s.sizes[0];
+    const uint16_t* X = n->Xbf + row0 * ps[0];
     const float* Y = n->dY + row0 * s.sizes[L];
     // the batch transposed: its columns of the transposed table where that is kept and the batch starts on a
     // cache line of it, a copy made now otherwise
     const bool inT = n->XbfT && (row0 % 64) == 0;
-    if (!inT) LAUNCH(n, "bf16_transpose_input", ghip_bf16_transpose(X, n->HT[0], B, s.sizes[0], n->stream));
-    TRY(forward_bf16(n, X, B));
-    TRY(output_delta_f32(n, n->logits, Y, nullptr, n->D[L], B));
-    LAUNCH(n, "bf16_transpose_delta", ghip_bf16_transpose(n->D[L], n->DT[L], B, s.sizes[L], n->stream));
+    if (!inT) LAUNCH(n, "bf16_transpose_input", ghip_bf16_transpose(X, n->HT[0], B, ps[0], n->stream));
+    TRY(forward_bf16(n, X, batch));
+    // rows past the batch carry zero deltas: an earlier, longer batch may have left its own there
+    if (B != batch)
+        LAUNCH(n, "fill_pad_delta", ghip_fill_u32((unsigned int*)(n->D[L] + (size_t)batch * ps[L]), (long long)(B - batch) * ps[L] / 2, 0u, n->stream));
+    TRY(output_delta_f32(n, n->logits, Y, nullptr, n->D[L], batch));
+    LAUNCH(n, "bf16_transpose_delta", ghip_bf16_transpose(n->D[L], n->DT[L], B, ps[L], n->stream));
     for (int l = L - 1; l >= 0; --l) {
-        const int ni = s.sizes[l], no = s.sizes[l + 1];
+        const int ni = ps[l], no = ps[l + 1];
         GemmLpArgs g;
         if (l > 0) {
             memset(&g, 0, sizeof(g));
@@ -593,10 +629,10 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
             LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));
         }
         if (l + 1 < L)  // D[l+1] came from a back-propagation product, which left its column sums
-            LAUNCH(n, "bias_update_bf16", ghip_bias_update_partials(n->csum[l + 1], B / ghip_gemm_lp_tile_m(B, no), no, B, n->b[l], n->vb[l],
+            LAUNCH(n, "bias_update_bf16", ghip_bias_update_partials(n->csum[l + 1], B / ghip_gemm_lp_tile_m(B, no), no, batch, n->b[l], n->vb[l],
                                                                     s.lr[l], s.mom[l], n->stream));
         else
-            LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+            LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, batch, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
         memset(&g, 0, sizeof(g));
         // both operands K-blocked over the batch: [B / 64][nodes][64], a tile's stage one contiguous block
         g.A = n->DT[l + 1]; g.B = n->HT[l]; g.M = no; g.N = ni; g.K = B;
@@ -605,7 +641,7 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
         if (l == 0 && inT) g.B = n->XbfT + (row0 / 64) * (long long)ni * 64;
         g.epilogue = LP_WGRAD_SGD; g.out = n->Wh[l]; g.outT = n->WhT[l]; g.outT_blocked = 1;
         g.master = n->W[l]; g.mom = n->vW[l];
-        g.lr = s.lr[l]; g.momf = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l]; g.gscale = 1.0f / (float)B;
+        g.lr = s.lr[l]; g.momf = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l]; g.gscale = 1.0f / (float)batch;
         // the profile keeps the two tile sizes apart: they are different kernels with different rooflines
         if (ghip_gemm_lp_tile_m(g.M, g.N) == 128) LAUNCH(n, "gemm_bf16_wgrad_sgd_t128", ghip_gemm_lp(g, n->stream));
         else LAUNCH(n, "gemm_bf16_wgrad_sgd", ghip_gemm_lp(g, n->stream));
@@ -614,13 +650,16 @@ int step_bf16(ghip_net* n, int64_t row0, int B)
 }
 
 // ---- fp8 inference ----
-int forward_fp8(ghip_net* n, const uint16_t* Xbf, int B, float* dev_out)
+// Xbf: the batch's rows in bf16 at pitch ps[0], pad_batch(batch) of them readable; dev_out has pitch ps[L]
+int forward_fp8(ghip_net* n, const uint16_t* Xbf, int batch, float* dev_out)
 {
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
+    const int* ps = n->ps;
+    const int B = pad_batch(n, batch);
     if (!n->quantized) return fail(GHIP_ESTATE, "call ghip_net_quantize_fp8 first");
     int cur = 0;
-    LAUNCH(n, "quant_rows_e4m3", ghip_quant_rows_e4m3(Xbf, 1, B, s.sizes[0], n->Aq[0], n->ascale[0], nullptr, 0, n->stream));
+    LAUNCH(n, "quant_rows_e4m3", ghip_quant_rows_e4m3(Xbf, 1, B, ps[0], n->Aq[0], n->ascale[0], nullptr, 0, n->stream));
     // the row maxima start at zero and every re-quantisation puts the entries it has read back to
     // zero; they are only cleared here after a forward pass that stopped between the two
     if (!n->amax_clean) {
@@ -630,14 +669,15 @@ int forward_fp8(ghip_net* n, const uint16_t* Xbf, int B, float* dev_out)
     for (int l = 0; l < L; ++l) {
         GemmLpArgs g;
         memset(&g, 0, sizeof(g));
-        g.A = n->Aq[cur]; g.B = n->Wq[l]; g.M = B; g.N = s.sizes[l + 1]; g.K = s.sizes[l];
+        g.A = n->Aq[cur]; g.B = n->Wq[l]; g.M = B; g.N = ps[l + 1]; g.K = ps[l];
         g.fp8 = 1; g.row_scale = n->ascale[cur]; g.col_scale = n->wscale[l];
         g.act = out_act(s, l, &g.act_param);
         if (l < L - 1) {
             g.epilogue = LP_FP8_ACT; g.out = n->Hq; g.row_amax_bits = n->amax_bits;
+            g.n_valid = ps[l + 1] != s.sizes[l + 1] ? s.sizes[l + 1] : 0;
             n->amax_clean = false;
             LAUNCH(n, "gemm_fp8_forward", ghip_gemm_lp(g, n->stream));
-            LAUNCH(n, "requant_rows_e4m3", ghip_quant_rows_e4m3(n->Hq, 1, B, s.sizes[l + 1], n->Aq[cur ^ 1], n->ascale[cur ^ 1],
+            LAUNCH(n, "requant_rows_e4m3", ghip_quant_rows_e4m3(n->Hq, 1, B, ps[l + 1], n->Aq[cur ^ 1], n->ascale[cur ^ 1],
                                                                 n->amax_bits, 1, n->stream));
             n->amax_clean = true;
             cur ^= 1;
@@ -738,6 +778,7 @@ int ghip_net_create(const ghip_net_spec* spec, ghip_net** out)
     ghip_net* n = new ghip_net();
     n->spec = *spec;
     n->L = spec->n_layers;
+    set_padded_sizes(n);
     hipError_t e = hipStreamCreate(&n->stream);
     if (e != hipSuccess) { delete n; return fail(GHIP_EHIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
     int r = (spec->mode == GHIP_MODE_EXACT) ? setup_exact(n) : setup_canon(n);
@@ -791,9 +832,11 @@ int ghip_net_set_params(ghip_net* n, int layer, const float* host_W, const float
         return 0;
     }
     if (bias_len != 0 && bias_len != no) return fail(GHIP_EINVAL, "canonical bias has one entry per output channel (%d), got %d", no, bias_len);
-    const size_t cnt = (size_t)ni * no;
+    const int pni = n->ps[layer];
+    const size_t cnt = (size_t)pni * n->ps[layer + 1];
     if (host_W) {
-        HIP_TRY(hipMemcpyAsync(n->W[layer], host_W, cnt * 4, hipMemcpyHostToDevice, n->stream));
+        if (pni == ni) HIP_TRY(hipMemcpyAsync(n->W[layer], host_W, (size_t)ni * no * 4, hipMemcpyHostToDevice, n->stream));
+        else HIP_TRY(copy_matrix(n->W[layer], pni, const_cast<float*>(host_W), no, ni, true, n->stream));
         if (n->vW[layer]) HIP_TRY(hipMemsetAsync(n->vW[layer], 0, cnt * 4, n->stream));
         n->shadow_dirty = true;
         n->quantized = false;
@@ -821,7 +864,13 @@ int ghip_net_get_params(ghip_net* n, int layer, float* host_W, float* host_bias,
         if (host_bias && bias_len >= 1) HIP_TRY(hipMemcpy(host_bias, n->exBias + layer, 4, hipMemcpyDeviceToHost));
         return 0;
     }
-    if (host_W) HIP_TRY(hipMemcpy(host_W, n->W[layer], (size_t)ni * no * 4, hipMemcpyDeviceToHost));
+    if (host_W) {
+        if (n->ps[layer] == ni) HIP_TRY(hipMemcpy(host_W, n->W[layer], (size_t)ni * no * 4, hipMemcpyDeviceToHost));
+        else {
+            HIP_TRY(copy_matrix(n->W[layer], n->ps[layer], host_W, no, ni, false, n->stream));
+            HIP_TRY(hipStreamSynchronize(n->stream));
+        }
+    }
     if (host_bias) {
         if (bias_len != no) return fail(GHIP_EINVAL, "bias_len %d != %d", bias_len, no);
         HIP_TRY(hipMemcpy(host_bias, n->b[layer], (size_t)no * 4, hipMemcpyDeviceToHost));
@@ -854,8 +903,12 @@ static int move_state(ghip_net* n, int layer, float* a, float* b, int to_device)
         return 0;
     }
     if (s.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "an inference-only network has no optimiser state");
-    if (a) HIP_TRY(to_device ? hipMemcpy(n->vW[layer], a, (size_t)ni * no * 4, hipMemcpyHostToDevice)
-                             : hipMemcpy(a, n->vW[layer], (size_t)ni * no * 4, hipMemcpyDeviceToHost));
+    if (a && n->ps[layer] != ni) {
+        HIP_TRY(copy_matrix(n->vW[layer], n->ps[layer], a, no, ni, to_device != 0, n->stream));
+        HIP_TRY(hipStreamSynchronize(n->stream));
+    } else if (a)
+        HIP_TRY(to_device ? hipMemcpy(n->vW[layer], a, (size_t)ni * no * 4, hipMemcpyHostToDevice)
+                          : hipMemcpy(a, n->vW[layer], (size_t)ni * no * 4, hipMemcpyDeviceToHost));
     if (b) HIP_TRY(to_device ? hipMemcpy(n->vb[layer], b, (size_t)no * 4, hipMemcpyHostToDevice)
                              : hipMemcpy(b, n->vb[layer], (size_t)no * 4, hipMemcpyDeviceToHost));
     return 0;
@@ -960,20 +1013,25 @@ static int make_bf16_table(ghip_net* n)
     if (s.mode != GHIP_MODE_CANONICAL || s.dtype == GHIP_F32) return 0;
     dfree(n->Xbf);
     dfree(n->XbfT);
-    TRY(dalloc(&n->Xbf, (size_t)n->n_rows * s.sizes[0]));
+    const int n0 = s.sizes[0], pn0 = n->ps[0];
+    // a last batch that is not a multiple of 256 rows reads on into rows of zeros
+    n->table_rows = (n->n_rows + 255 + 63) / 64 * 64;
+    TRY(dalloc(&n->Xbf, (size_t)n->table_rows * pn0));
+    HIP_TRY(hipMemsetAsync(n->Xbf + (size_t)n->n_rows * pn0, 0, (size_t)(n->table_rows - n->n_rows) * pn0 * 2, n->stream));
     // Training reads each batch transposed as well (the weight gradient of the first layer runs over the
     // batch): the whole table is kept that way, in planes of 64 rows.  A table too large for that is
     // transposed batch by batch.
-    const size_t bytesT = (size_t)s.sizes[0] * (size_t)(((n->n_rows + 63) / 64) * 64) * 2;
+    const size_t bytesT = (size_t)pn0 * (size_t)n->table_rows * 2;
     if (s.dtype == GHIP_BF16 && n->n_rows >= 64 && bytesT <= ((size_t)16 << 30)) {
         if (hipMalloc((void**)&n->XbfT, bytesT) != hipSuccess) { n->XbfT = nullptr; (void)hipGetLastError(); }
+        else HIP_TRY(hipMemsetAsync(n->XbfT + (size_t)(n->n_rows / 64) * pn0 * 64, 0, (size_t)(n->table_rows / 64 - n->n_rows / 64) * pn0 * 128, n->stream));
     }
     // convert in slabs of rows to keep the grid small
     const int64_t slab = 65536;
     for (int64_t r = 0; r < n->n_rows; r += slab) {
         const int rows = (int)((n->n_rows - r) < slab ? (n->n_rows - r) : slab);
-        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d(n->dX + r * s.sizes[0], n->Xbf + r * s.sizes[0],
-                                                          n->XbfT ? n->XbfT + (r / 64) * s.sizes[0] * 64 : nullptr, rows, s.sizes[0], n->stream));
+        LAUNCH(n, "f32_to_bf16_table", ghip_f32_to_bf16_2d_pad(n->dX + r * n0, rows, n0, n->Xbf + r * pn0,
+                                                              n->XbfT ? n->XbfT + (r / 64) * pn0 * 64 : nullptr, rows, pn0, n->stream));
     }
     return 0;
 }
@@ -1174,7 +1232,6 @@ int ghip_net_train_step(ghip_net* n, int64_t row0, int batch, ghip_metrics* host
     if (n->spec.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "fp8 networks are inference only");
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows [%lld,%lld) exceed the table (%lld rows)", (long long)row0, (long long)(row0 + batch), (long long)n->n_rows);
-    if (n->spec.dtype == GHIP_BF16 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 path takes batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     n->last_batch = batch;
     if (n->spec.dtype == GHIP_F32) TRY(step_f32(n, row0, batch));
@@ -1194,8 +1251,6 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
     if (train && s.dtype == GHIP_FP8_INFER) return fail(GHIP_ESTATE, "fp8 networks are inference only");
     const int64_t N = n->n_rows;
     if (batch > N) batch = (int)N;
-    if (s.dtype != GHIP_F32 && ((batch % 256) || (N % batch) % 256))
-        return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256, the last one (%lld rows here) too; use dtype GHIP_F32 or pad the table", (long long)(N % batch));
     TRY(reserve_batch(n, batch));
     if (s.dtype == GHIP_BF16) TRY(refresh_shadows(n));
     LAUNCH(n, "fill_pass_metrics", ghip_fill_f64(n->dAcc + 12, 4, 0.0, n->stream));
@@ -1208,8 +1263,8 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
         } else {
             float* P = nullptr;
             if (s.dtype == GHIP_F32) { rc = forward_f32(n, n->dX + r0 * s.sizes[0], b, L); P = n->act[L]; }
-            else if (s.dtype == GHIP_BF16) { rc = forward_bf16(n, n->Xbf + r0 * s.sizes[0], b); P = n->logits; }
-            else { rc = forward_fp8(n, n->Xbf + r0 * s.sizes[0], b, n->out8); P = n->out8; }
+            else if (s.dtype == GHIP_BF16) { rc = forward_bf16(n, n->Xbf + r0 * n->ps[0], b); P = n->logits; }
+            else { rc = forward_fp8(n, n->Xbf + r0 * n->ps[0], b, n->out8); P = n->out8; }
             if (rc == 0) rc = output_delta_f32(n, P, n->dY + r0 * s.sizes[L], nullptr, nullptr, b);
         }
         n->last_batch = b;
@@ -1252,7 +1307,7 @@ static int forward_any(ghip_net* n, const float* dev_X32, const uint16_t* dev_Xb
         if (s.act[L - 1] == GHIP_SOFTMAX) {
             DeltaArgs a;
             memset(&a, 0, sizeof(a));
-            a.P = n->logits; a.B = batch; a.n = s.sizes[L]; a.ldp = s.sizes[L]; a.ldy = s.sizes[L];
+            a.P = n->logits; a.B = batch; a.n = s.sizes[L]; a.ldp = n->ps[L]; a.ldy = s.sizes[L];
             a.act = GHIP_SOFTMAX; a.cost = s.cost; a.acc = n->dAcc + 8; a.store_p = 1;
             LAUNCH(n, "softmax", ghip_output_delta(a, n->stream));
         }
@@ -1270,7 +1325,6 @@ int ghip_net_forward(ghip_net* n, const float* host_X, int batch, float* host_ou
     HIP_TRY(hipSetDevice(g_device));
     if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
     const ghip_net_spec& s = n->spec;
-    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     HIP_TRY(hipMemcpyAsync(n->stageX, host_X, (size_t)batch * s.sizes[0] * 4, hipMemcpyHostToDevice, n->stream));
     uint16_t* xbf = nullptr;
@@ -1278,11 +1332,13 @@ int ghip_net_forward(ghip_net* n, const float* host_X, int batch, float* host_ou
         // the bf16 copy of the staged rows goes to a buffer the forward pass only overwrites after
         // having consumed it (transposed-input buffer for bf16, activation scratch for fp8)
         xbf = (s.dtype == GHIP_BF16) ? n->HT[0] : n->Hq;
-        LAUNCH(n, "f32_to_bf16_input", ghip_f32_to_bf16_2d(n->stageX, xbf, nullptr, batch, s.sizes[0], n->stream));
+        LAUNCH(n, "f32_to_bf16_input", ghip_f32_to_bf16_2d_pad(n->stageX, batch, s.sizes[0], xbf, nullptr, pad_batch(n, batch), n->ps[0], n->stream));
     }
     float* res = nullptr;
     TRY(forward_any(n, n->stageX, xbf, batch, &res));
-    HIP_TRY(hipMemcpyAsync(host_out, res, (size_t)batch * s.sizes[s.n_layers] * 4, hipMemcpyDeviceToHost, n->stream));
+    const int nout = s.sizes[s.n_layers];
+    if (n->ps[s.n_layers] == nout) HIP_TRY(hipMemcpyAsync(host_out, res, (size_t)batch * nout * 4, hipMemcpyDeviceToHost, n->stream));
+    else HIP_TRY(copy_matrix(res, n->ps[s.n_layers], host_out, batch, nout, false, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
     return 0;
 }
@@ -1295,11 +1351,13 @@ int ghip_net_forward_resident(ghip_net* n, int64_t row0, int batch, float* dev_o
     if (!n->dX) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
     const ghip_net_spec& s = n->spec;
-    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     float* res = nullptr;
-    TRY(forward_any(n, n->dX + row0 * s.sizes[0], n->Xbf ? n->Xbf + row0 * s.sizes[0] : nullptr, batch, &res));
-    if (dev_out) HIP_TRY(hipMemcpyAsync(dev_out, res, (size_t)batch * s.sizes[s.n_layers] * 4, hipMemcpyDeviceToDevice, n->stream));
+    TRY(forward_any(n, n->dX + row0 * s.sizes[0], n->Xbf ? n->Xbf + row0 * n->ps[0] : nullptr, batch, &res));
+    const int nout = s.sizes[s.n_layers];
+    if (dev_out && n->ps[s.n_layers] == nout) HIP_TRY(hipMemcpyAsync(dev_out, res, (size_t)batch * nout * 4, hipMemcpyDeviceToDevice, n->stream));
+    else if (dev_out)
+        HIP_TRY(hipMemcpy2DAsync(dev_out, (size_t)nout * 4, res, (size_t)n->ps[s.n_layers] * 4, (size_t)nout * 4, batch, hipMemcpyDeviceToDevice, n->stream));
     return 0;
 }
 
@@ -1327,6 +1385,7 @@ int ghip_forward_noalloc(const ghip_net_spec* spec, const float* const* dev_W, c
     ghip_net n;
     n.spec = *spec;
     n.L = L;
+    set_padded_sizes(&n);
     n.stream = (hipStream_t)hip_stream;
     for (int l = 0; l < L; ++l) {
         n.W[l] = const_cast<float*>(dev_W[l]);
@@ -1348,13 +1407,12 @@ int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* h
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
     if (row0 + batch > n->n_rows) return fail(GHIP_EINVAL, "rows exceed the table");
     const ghip_net_spec& s = n->spec;
-    if (s.dtype != GHIP_F32 && (batch % 256)) return fail(GHIP_EINVAL, "the bf16 / e4m3 paths take batches that are multiples of 256; use dtype GHIP_F32 (any batch) or pad the batch");
     TRY(reserve_batch(n, batch));
     const int L = s.n_layers;
     float* P = nullptr;
     if (s.dtype == GHIP_F32) { TRY(forward_f32(n, n->dX + row0 * s.sizes[0], batch, L)); P = n->act[L]; }
-    else if (s.dtype == GHIP_BF16) { TRY(refresh_shadows(n)); TRY(forward_bf16(n, n->Xbf + row0 * s.sizes[0], batch)); P = n->logits; }
-    else { TRY(forward_fp8(n, n->Xbf + row0 * s.sizes[0], batch, n->out8)); P = n->out8; }
+    else if (s.dtype == GHIP_BF16) { TRY(refresh_shadows(n)); TRY(forward_bf16(n, n->Xbf + row0 * n->ps[0], batch)); P = n->logits; }
+    else { TRY(forward_fp8(n, n->Xbf + row0 * n->ps[0], batch, n->out8)); P = n->out8; }
     TRY(output_delta_f32(n, P, n->dY + row0 * s.sizes[L], nullptr, nullptr, batch));
     n->last_batch = batch;
     return fetch_metrics(n, host_metrics);
@@ -1410,12 +1468,13 @@ int ghip_net_quantize_fp8(ghip_net* n, float* const* host_scales, uint8_t* const
     const ghip_net_spec& s = n->spec;
     if (!is_canon(n) || s.dtype != GHIP_FP8_INFER) return fail(GHIP_ESTATE, "network was not created with GHIP_FP8_INFER");
     for (int l = 0; l < s.n_layers; ++l)
-        LAUNCH(n, "quant_weights_e4m3", ghip_quant_rows_e4m3(n->W[l], 0, s.sizes[l + 1], s.sizes[l], n->Wq[l], n->wscale[l], nullptr, 0, n->stream));
+        LAUNCH(n, "quant_weights_e4m3", ghip_quant_rows_e4m3(n->W[l], 0, n->ps[l + 1], n->ps[l], n->Wq[l], n->wscale[l], nullptr, 0, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
     n->quantized = true;
     for (int l = 0; l < s.n_layers; ++l) {
         if (host_scales && host_scales[l]) HIP_TRY(hipMemcpy(host_scales[l], n->wscale[l], (size_t)s.sizes[l + 1] * 4, hipMemcpyDeviceToHost));
-        if (host_codes && host_codes[l]) HIP_TRY(hipMemcpy(host_codes[l], n->Wq[l], (size_t)s.sizes[l + 1] * s.sizes[l], hipMemcpyDeviceToHost));
+        if (host_codes && host_codes[l])
+            HIP_TRY(hipMemcpy2D(host_codes[l], (size_t)s.sizes[l], n->Wq[l], (size_t)n->ps[l], (size_t)s.sizes[l], s.sizes[l + 1], hipMemcpyDeviceToHost));
     }
     return 0;
 }

@@ -58,7 +58,7 @@ __device__ __forceinline__ float ghip_delta_row64(const DeltaArgs& a, int b, int
         if (pv > bp) { bp = pv; ip = o; }
         if (yv > by) { by = yv; iy = o; }
         if (a.D) a.D[(long long)b * a.n + o] = d;
-        if (a.Dbf) a.Dbf[(long long)b * a.n + o] = ghip_f32_to_bf16(d);
+        if (a.Dbf) a.Dbf[(long long)b * (a.ldd ? a.ldd : a.n) + o] = ghip_f32_to_bf16(d);
     }
     // argmax across lanes: largest value, lowest index on ties; "no element above 0" = none
 #pragma unroll

@@ -104,7 +104,7 @@ __global__ void __launch_bounds__(256) output_delta_kernel(DeltaArgs a)
             if (pv > bp) { bp = pv; ip = o; }
             if (yv > by) { by = yv; iy = o; }
             if (a.D) a.D[(long long)b * a.n + o] = d;
-            if (a.Dbf) a.Dbf[(long long)b * a.n + o] = ghip_f32_to_bf16(d);
+            if (a.Dbf) a.Dbf[(long long)b * (a.ldd ? a.ldd : a.n) + o] = ghip_f32_to_bf16(d);
         };
         if (kInRegs) {
 #pragma unroll
@@ -213,7 +213,7 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
                     uint2 h;
                     h.x = (uint32_t)ghip_f32_to_bf16(d.x) | ((uint32_t)ghip_f32_to_bf16(d.y) << 16);
                     h.y = (uint32_t)ghip_f32_to_bf16(d.z) | ((uint32_t)ghip_f32_to_bf16(d.w) << 16);
-                    *reinterpret_cast<uint2*>(a.Dbf + (long long)b * a.n + o) = h;
+                    *reinterpret_cast<uint2*>(a.Dbf + (long long)b * (a.ldd ? a.ldd : a.n) + o) = h;
                 }
             }
         }
@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
 
 // bf16 delta^T, K-blocked [B / 64][n][64]: one wavefront per channel, 16-byte loads (B is a multiple of 64)
 __global__ void __launch_bounds__(256)
-bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* __restrict__ bias,
+bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, int batch, float* __restrict__ bias,
                          float* __restrict__ vb, float lr, float mom)
 {
     const int lane = threadIdx.x & 63;
@@ -268,7 +268,7 @@ bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, float* _
     }
     float s = wave_sum((s4[0] + s4[1]) + (s4[2] + s4[3]));
     if (lane == 0) {
-        const float g = s / (float)B;
+        const float g = s / (float)batch;
         const float d = lr * g + mom * vb[o];
         vb[o] = d;
         bias[o] = bias[o] - d;
@@ -307,9 +307,10 @@ __global__ void __launch_bounds__(256) fill_kernel(T* p, long long n, T v)
 
 // 64x64 tile through LDS: dst[r][c] = bf16(src[r][c]) and the K-blocked transposed copy
 // dstT[r / 64][c][r % 64]; src fp32 or bf16
+// The source has src_rows x src_cols elements (row pitch src_cols); what lies outside it is written as zero.
 template <typename SrcT>
 __global__ void __launch_bounds__(256)
-convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ dst,
+convert_transpose_kernel(const SrcT* __restrict__ src, int src_rows, int src_cols, uint16_t* __restrict__ dst,
                          uint16_t* __restrict__ dstT, int rows, int cols)
 {
     __shared__ uint16_t tile[64][64 + 2];
@@ -319,8 +320,10 @@ convert_transpose_kernel(const SrcT* __restrict__ src, uint16_t* __restrict__ ds
         const int r = r0 + j, c = c0 + tx;
         uint16_t v = 0;
         if (r < rows && c < cols) {
-            if (sizeof(SrcT) == 4) v = ghip_f32_to_bf16(((const float*)src)[(long long)r * cols + c]);
-            else v = ((const uint16_t*)src)[(long long)r * cols + c];
+            if (r < src_rows && c < src_cols) {
+                if (sizeof(SrcT) == 4) v = ghip_f32_to_bf16(((const float*)src)[(long long)r * src_cols + c]);
+                else v = ((const uint16_t*)src)[(long long)r * src_cols + c];
+            }
             if (dst) dst[(long long)r * cols + c] = v;
         }
         tile[j][tx] = v;
@@ -525,10 +528,10 @@ hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vb, float lr,
+hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, int batch, float* bias, float* vb, float lr,
                                   float mom, hipStream_t s)
 {
-    hipLaunchKernelGGL(bias_update_bf16T_kernel, dim3((n + 3) / 4), dim3(256), 0, s, DT, n, B, bias, vb, lr, mom);
+    hipLaunchKernelGGL(bias_update_bf16T_kernel, dim3((n + 3) / 4), dim3(256), 0, s, DT, n, B, batch, bias, vb, lr, mom);
     return hipGetLastError();
 }
 
@@ -558,7 +561,14 @@ hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s)
 {
     dim3 grid((cols + 63) / 64, (rows + 63) / 64);
-    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, dst, dstT, rows, cols);
+    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, rows, cols, dst, dstT, rows, cols);
+    return hipGetLastError();
+}
+
+hipError_t ghip_f32_to_bf16_2d_pad(const float* src, int src_rows, int src_cols, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s)
+{
+    dim3 grid((cols + 63) / 64, (rows + 63) / 64);
+    hipLaunchKernelGGL(convert_transpose_kernel<float>, grid, dim3(256), 0, s, src, src_rows, src_cols, dst, dstT, rows, cols);
     return hipGetLastError();
 }
 
@@ -569,7 +579,7 @@ hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, in
         hipLaunchKernelGGL(bf16_transpose64_kernel, grid, dim3(256), 0, s, src, dstT, rows, cols);
         return hipGetLastError();
     }
-    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, (uint16_t*)nullptr, dstT, rows, cols);
+    hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, rows, cols, (uint16_t*)nullptr, dstT, rows, cols);
     return hipGetLastError();
 }
 

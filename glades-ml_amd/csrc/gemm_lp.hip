@@ -405,6 +405,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     }
     // Two copies of the element loop, chosen once per launch: piecewise-linear activations
     // (ReLU, leaky, linear, step) take four instructions per element, the general form a dozen.
+    const bool pad_tile = g.n_valid > 0 && bn + TN > g.n_valid;   // only the tiles of the last columns can hold padding
     auto finish = [&](auto plain_c) {
         constexpr bool PLAIN = decltype(plain_c)::value;
 #pragma unroll
@@ -441,6 +442,10 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                             o[r] = v;
                         }
                         if constexpr (EPI == LP_FWD_F32 || EPI == LP_FP8_F32) ((float*)g.out)[idx] = o[r];
+                    }
+                    if constexpr (EPI == LP_FWD_ACT || EPI == LP_FP8_ACT) {
+                        // units past the layer's width are padding: they stay zero whatever the activation makes of 0
+                        if (pad_tile && col >= g.n_valid) { o[0] = 0.0f; o[1] = 0.0f; o[2] = 0.0f; o[3] = 0.0f; }
                     }
                     if constexpr (EPI == LP_FP8_ACT) {
                         // single output: straight into the row-major staging area

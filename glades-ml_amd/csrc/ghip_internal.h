@@ -309,6 +309,7 @@ hipError_t ghip_narrow_forward(const NarrowOutArgs& a, hipStream_t s);
 struct DeltaArgs {
     float* P; const float* Y; float* D; uint16_t* Dbf; uint16_t* DbfT;
     int B, n, ldp, ldy;
+    int ldd;       // row pitch of Dbf in elements (0: n): the bf16 deltas of a padded low-precision network
     int act; float act_param; int cost;
     double* acc;
     double* acc_clear;  // 4 doubles set to zero by this launch (the next launch's accumulators), or NULL
@@ -346,6 +347,7 @@ struct GemmLpArgs {
     // the batch) are kept that way: they come from HBM, where scattered lines cost a DRAM page each.
     long long kstrideA, kstrideB;
     int outT_blocked;                 // outT is written K-blocked for the product that will read it: [M / 64][N][64]
+    int n_valid;                      // LP_FWD_ACT / LP_FP8_ACT: columns from here on are padding and are stored as 0 (0: none)
     int fp8;                          // 0: bf16 operands, 1: e4m3 operands
     int epilogue;
     void* out; void* outT;            // see LpEpilogue; outT may be NULL
@@ -375,9 +377,13 @@ int ghip_gemm_lp_tile_m(int M, int N);  // rows per tile the launcher picks for 
 // element (row r, column c) of a [rows][cols] source lies at ((r / 64) * cols + c) * 64 + r % 64 of dstT,
 // i.e. dstT is [ceil(rows / 64)][cols][64].
 hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
+// the same from a source of src_rows x src_cols (row pitch src_cols) into destinations of rows x cols: what lies
+// outside the source is zero (the padded copy of a table)
+hipError_t ghip_f32_to_bf16_2d_pad(const float* src, int src_rows, int src_cols, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
 hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s);
 // bias update from bf16 delta^T, K-blocked [B / 64][n][64]: gb[o] = sum_b
-hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, float* bias, float* vbias, float lr,
+// (B rows of deltas, of which the first batch are the batch's; the rest are padding and zero)
+hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, int batch, float* bias, float* vbias, float lr,
                                   float mom, hipStream_t s);
 // the same from per-tile-row partial column sums [tiles][n] (written by the LP_DGRAD epilogue)
 hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B, float* bias, float* vbias, float lr,
