@@ -35,6 +35,7 @@
 namespace {
 
 constexpr int kPrefetch = 4;  // values per lane of the next row held in registers
+template <int V> struct IC { static constexpr int value = V; };
 
 // The reference updates the scalar layer bias once per (input, output) pair (network.cpp:654-656):
 // bias -= lr*d[o] for o = 0..n_out-1, repeated n_in times -- one dependent chain of n_in*n_out fp32
@@ -92,8 +93,38 @@ __device__ __forceinline__ float fold8(float z, const float* x, int xs, const fl
         if (nb - b == 2) { fetch(xb, yb, b + 1); run(xa, ya); run(xb, yb); }
         else run(xa, ya);
     }
-    for (int i = nb * B; i < n; ++i) z = step(z, x[i * xs], y[i * ys]);
+    // the last n % 8 steps: blocks of 4, 2 and 1, each block's operands asked for together (a loop would pay
+    // an LDS round trip per step, which for the 4-input layer of a small network is the whole dot product)
+    int i = nb * B;
+    auto block = [&](auto cnt) {
+        constexpr int C = decltype(cnt)::value;
+        float xv[C], yv[C];
+#pragma unroll
+        for (int j = 0; j < C; ++j) { xv[j] = x[(i + j) * xs]; yv[j] = y[(i + j) * ys]; }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < C; ++j) z = step(z, xv[j], yv[j]);
+        i += C;
+    };
+    if (n & 4) block(IC<4>{});
+    if (n & 2) block(IC<2>{});
+    if (n & 1) block(IC<1>{});
     return z;
+}
+
+// Inclusive scan over the 64 lanes of a wavefront with an associative op: shifts within the rows of 16 lanes,
+// then the last lane of row 0 / 2 into rows 1 / 3 and the last lane of the lower half into the upper half.
+// A lane without a source keeps `identity`.
+template <typename Op>
+__device__ __forceinline__ int wave_scan(int v, int identity, Op op)
+{
+    v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x111, 0xf, 0xf, false));  // row_shr:1
+    v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x112, 0xf, 0xf, false));  // row_shr:2
+    v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x114, 0xf, 0xf, false));  // row_shr:4
+    v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x118, 0xf, 0xf, false));  // row_shr:8
+    v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x142, 0xa, 0xf, false));  // row_bcast:15 into rows 1 and 3
+    v = op(v, __builtin_amdgcn_update_dpp(identity, v, 0x143, 0xc, 0xf, false));  // row_bcast:31 into rows 2 and 3
+    return v;
 }
 
 // The same chain without walking it, where that is provably the same.  While the bias stays in one
@@ -123,21 +154,13 @@ __device__ __forceinline__ bool bias_chain_grid(float b, float xk, int ni, int l
     const bool tie = fabs(t - q) == 0.5;
     if (__ballot(!in_range || tie) != 0ull) return false;
     const int qi = (int)q;
-    // inclusive prefix sums over the lanes, their extremes, and the total
-    int pre = qi;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const int up = __shfl_up(pre, o, 64);
-        if (lane >= o) pre += up;
-    }
-    int pmin = pre, pmax = pre;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const int a = __shfl_xor(pmin, o, 64), c = __shfl_xor(pmax, o, 64);
-        pmin = a < pmin ? a : pmin;
-        pmax = c > pmax ? c : pmax;
-    }
-    const long long Q = (long long)__shfl(pre, 63, 64);
+    // inclusive prefix sums over the lanes, their extremes, and the total: scans on the cross-lane data path
+    // (a shuffle through LDS is a round trip of a hundred clocks per step, and this wavefront runs alone)
+    const int pre = wave_scan(qi, 0, [](int a, int c) { return a + c; });
+    const int pmin = __builtin_amdgcn_readlane(wave_scan(pre, 0x7fffffff, [](int a, int c) { return a < c ? a : c; }), 63);
+    const int pmax = __builtin_amdgcn_readlane(wave_scan(pre, (int)0x80000000, [](int a, int c) { return a > c ? a : c; }), 63);
+    const long long Q = (long long)__builtin_amdgcn_readlane(pre, 63);
+    (void)lane;
     const long long span = (long long)(ni - 1) * Q;
     const long long lo = (span < 0 ? span : 0) + pmin;      // smallest and largest amount subtracted so far,
     const long long hi = (span > 0 ? span : 0) + pmax;      // over every step of every round
@@ -155,10 +178,16 @@ constexpr int kGridChainMin = 512;
 // another, so the wait covers LDS operations alone: __syncthreads() would also wait for the global
 // loads that prefetch the next row and for the confusion-matrix atomics, a trip to memory per row.
 // With the state in global memory the full barrier stays.
-template <bool kLds>
+// A workgroup of one wavefront (kWave) needs no barrier at all: its LDS operations execute in the order
+// they were issued, so a value one lane stored is there when another lane's later load reads it.  What is
+// left is a fence that keeps the compiler from moving memory operations across the hand-over.
+template <bool kLds, bool kWave = false>
 __device__ __forceinline__ void row_barrier()
 {
-    if (kLds) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (kWave) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    } else if (kLds) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else __syncthreads();
 }
 
@@ -166,16 +195,25 @@ __device__ __forceinline__ void row_barrier()
 // table; with `multi` each workgroup b takes its own parameter / result pointers from multi[b]
 // (the subnets of a MetaNetwork train at the same time, one per compute unit), without it the
 // single network's pointers are the ones in `p`.
-template <bool kLds, bool kDrop>
-__global__ void __launch_bounds__(1024)
+// kL: the number of layers where it is known at compile time (0: read from p).  With it the loops over the layers
+// unroll, every p.x[l] becomes a fixed kernel-argument slot that is read once into a scalar register, and the
+// per-layer code is laid out straight.  The arithmetic and its order are the same.
+// kMaxT: the most threads a launch of this instantiation has.  The register file is shared by the wavefronts a
+// workgroup may have: 128 registers per lane at 1024 threads, 256 at 512, 512 at 256.  At 128 the row loop keeps
+// addresses in scratch memory, and every reload waits for the next row's prefetch as well.
+template <bool kLds, bool kDrop, int kL, int kMaxT>
+__global__ void __launch_bounds__(kMaxT)
 exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 {
     extern __shared__ float smem[];
     const ExactPointers own = multi ? multi[blockIdx.x] : p.ptr;
+    // one wavefront per network (the small networks: LDS-resident, at most 64 lanes of work per phase)
+    constexpr bool kWave = kLds && kMaxT == 64;
     const int tid = threadIdx.x;
-    const int T = blockDim.x;
+    const int T = kWave ? 64 : (int)blockDim.x;
     const int serial = T - 1;  // lane that carries the order-dependent scalar chains
-    const int L = p.n_layers;
+    const int L = kL > 0 ? kL : p.n_layers;
+    constexpr int kLayerUnroll = kL > 0 ? kL : 1;
     const int n0 = p.sizes[0];
     const int nout = p.sizes[L];
     const int S = p.state_floats;
@@ -237,12 +275,14 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 
     const float data_size = (float)((unsigned)p.n_rows * (unsigned)nout);
     const float fmb = (float)p.mb;
-    const bool small_row = (n0 <= kPrefetch * T) && (nout <= kPrefetch * T);
+    // (the single-wavefront instantiation is launched for layers of at most 64 nodes: one value per lane)
+    constexpr int kPf = kWave ? 1 : kPrefetch;
+    const bool small_row = kWave || ((n0 <= kPrefetch * T) && (nout <= kPrefetch * T));
 
     // first row into registers
-    float px[kPrefetch], py[kPrefetch];
+    float px[kPf], py[kPf];
 #pragma unroll
-    for (int j = 0; j < kPrefetch; ++j) {
+    for (int j = 0; j < kPf; ++j) {
         int i = tid + j * T;
         px[j] = (small_row && i < n0) ? p.X[i] : 0.0f;
         py[j] = (small_row && i < nout) ? p.Y[i] : 0.0f;
@@ -264,7 +304,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
             // ---- stage the row (prefetched) and start fetching the next one
             if (small_row) {
 #pragma unroll
-                for (int j = 0; j < kPrefetch; ++j) {
+                for (int j = 0; j < kPf; ++j) {
                     int i = tid + j * T;
                     if (i < n0) sa[i] = px[j];
                     if (i < nout) sy[i] = py[j];
@@ -274,7 +314,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 const float* xn = p.X + rn * n0;
                 const float* yn = p.Y + rn * nout;
 #pragma unroll
-                for (int j = 0; j < kPrefetch; ++j) {
+                for (int j = 0; j < kPf; ++j) {
                     int i = tid + j * T;
                     px[j] = (i < n0) ? xn[i] : 0.0f;
                     py[j] = (i < nout) ? yn[i] : 0.0f;
@@ -287,9 +327,10 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 const unsigned char* mr = own.masks + ((long long)ep * p.n_rows + r) * mask_len;
                 for (int k = tid; k < mask_len; k += T) sm[k] = mr[k];
             }
-            row_barrier<kLds>();
+            row_barrier<kLds, kWave>();
 
             // ---- ForwardPass (network.cpp:457-516)
+#pragma unroll kLayerUnroll
             for (int l = 0; l < L; ++l) {
                 const int ni = p.sizes[l], no = p.sizes[l + 1], ld = p.ld[l];
                 const float* Wl = sW + p.woff[l];
@@ -320,8 +361,9 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         rp[fill + o] = a;
                         re[fill + o] = sy[o];
                     }
+                    if (kWave) break;  // at most one node per lane there
                 }
-                row_barrier<kLds>();
+                row_barrier<kLds, kWave>();
             }
             fill += nout;
             const float* pred = sa + p.aoff[L];
@@ -329,7 +371,19 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 for (int o = tid; o < nout; o += T) own.preds[r * nout + o] = pred[o];
 
             // ---- output metrics (network.cpp:519-559): the class of the row now, ...
-            if (tid == serial) {
+            if (kWave) {
+                // The scan "strictly greater than the best so far, starting from 0" ends on the first index that
+                // holds the largest value above 0 (none: -1); a NaN never compares greater.  Across the lanes:
+                // the maximum (the hardware's max ignores a NaN operand), then the lowest lane that holds it.
+                const float pr = tid < nout ? pred[tid] : 0.0f, ex = tid < nout ? sy[tid] : 0.0f;
+                auto fmax_op = [](int a, int c) { return __float_as_int(fmaxf(__int_as_float(a), __int_as_float(c))); };
+                const float mp = __int_as_float(__builtin_amdgcn_readlane(wave_scan(__float_as_int(pr), 0, fmax_op), 63));
+                const float my = __int_as_float(__builtin_amdgcn_readlane(wave_scan(__float_as_int(ex), 0, fmax_op), 63));
+                const unsigned long long bp = __ballot(pr == mp && pr > 0.0f), by = __ballot(ex == my && ex > 0.0f);
+                const int ip = bp ? __builtin_ctzll(bp) : -1, iy = by ? __builtin_ctzll(by) : -1;
+                if (ip == iy) ++correct;   // every lane counts alike; lane `serial` reports
+                if (tid == serial && own.cm && ip >= 0 && iy >= 0) atomicAdd(&own.cm[iy * nout + ip], 1);
+            } else if (tid == serial) {
                 float mp = 0.0f, my = 0.0f;
                 int ip = -1, iy = -1;
                 for (int o = 0; o < nout; ++o) {
@@ -350,7 +404,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     rp[k] = ghip_cost<true>(ex, pr, data_size, p.cost);
                     re[k] = ghip_accuracy_term(pr, ex);
                 }
-                row_barrier<kLds>();
+                row_barrier<kLds, kWave>();
                 if (tid == serial) {
                     for (int k = 0; k < fill; ++k) {
                         tot_err = __fadd_rn(tot_err, rp[k]);
@@ -371,10 +425,12 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         dl[o] = e;
                         bs[o] = __fmul_rn(lr, e);
                         if (kDrop) sE[p.aoff[L] + o] = e;
+                        if (kWave) break;
                     }
                 }
-                row_barrier<kLds>();
+                row_barrier<kLds, kWave>();
                 const bool apply = rmod == 0;
+#pragma unroll kLayerUnroll
                 for (int Lo = L; Lo > 0; --Lo) {
                     const int l = Lo - 1;
                     const int ni = p.sizes[l], no = p.sizes[Lo], ld = p.ld[l];
@@ -393,46 +449,61 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     {
                         const int sh = p.tw_log2[l];
                         const int tw = 1 << sh;
-                        const int i0 = tid & (tw - 1), o0 = tid >> sh, rpp = T >> sh;
+                        // The last wavefront walks this layer's bias chain (below), which depends on nothing
+                        // done here: where there are other wavefronts it starts on the chain at once and
+                        // they share the edges (lane groups of at most a wavefront, so that they divide
+                        // what is left).
+                        const bool chain_apart = l != 0 && T >= 128 && tw <= 64;
+                        const int Tp = chain_apart ? T - 64 : T;
+                        const int i0 = tid & (tw - 1), o0 = tid >> sh, rpp = Tp >> sh;
+                        if (tid < Tp) {
                         // an edge that sat out an applying row can hold more than mb pending deltas;
                         // applyDeltas reads the first mb only (node.cpp:299-301), so their number is kept
                         int* Cl = (kDrop && p.mb > 1) ? own.wcnt + p.woff[l] : nullptr;
                         if (!kDrop) {
-                            // four edges of a lane at a time: their operands are asked for together
-                            for (int i = i0; i < ni; i += tw) {
-                                const float a = ain[i];
-                                const float t1 = __fmul_rn(w1, fabsf(a));
-                                const float t2 = __fmul_rn(w2, a);
-                                for (int o = o0; o < no; o += 4 * rpp) {
-                                    float bv[4], lv[4], sv[4], wv[4];
-                                    int kk[4];
+                            // U edges of a lane at a time, their operands asked for together: four where a
+                            // lane has several outputs per input column, one where it has at most one
+                            // (the narrow layers of a small network, where three of four would be idle repeats
+                            // and a lone wavefront pays for every instruction)
+                            auto push = [&](auto uc) {
+                                constexpr int U = decltype(uc)::value;
+                                for (int i = i0; i < ni; i += tw) {
+                                    const float a = ain[i];
+                                    const float t1 = __fmul_rn(w1, fabsf(a));
+                                    const float t2 = __fmul_rn(w2, a);
+                                    for (int o = o0; o < no; o += U * rpp) {
+                                        float bv[U], lv[U], sv[U], wv[U];
+                                        int kk[U];
 #pragma unroll
-                                    for (int j = 0; j < 4; ++j) {
-                                        const int oj = o + j * rpp;
-                                        const int oc = oj < no ? oj : no - 1;  // past the end: a repeat that is not stored
-                                        kk[j] = oc * ld + i;
-                                        bv[j] = bs[oc]; lv[j] = Ll[kk[j]]; sv[j] = Sl[kk[j]]; wv[j] = Wl[kk[j]];
-                                    }
-                                    __builtin_amdgcn_sched_barrier(0);
+                                        for (int j = 0; j < U; ++j) {
+                                            const int oj = o + j * rpp;
+                                            const int oc = oj < no ? oj : no - 1;  // past the end: a repeat that is not stored
+                                            kk[j] = oc * ld + i;
+                                            bv[j] = bs[oc]; lv[j] = Ll[kk[j]]; sv[j] = Sl[kk[j]]; wv[j] = Wl[kk[j]];
+                                        }
+                                        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                                    for (int j = 0; j < 4; ++j) {
-                                        if (o + j * rpp < no) {
-                                            float dW = __fadd_rn(__fmul_rn(bv[j], a), __fmul_rn(mom, lv[j]));
-                                            dW = __fadd_rn(dW, t1);
-                                            dW = __fadd_rn(dW, t2);
-                                            const float sn = __fadd_rn(sv[j], dW);
-                                            if (apply) {
-                                                Wl[kk[j]] = __fsub_rn(wv[j], __fdiv_rn(sn, fmb));
-                                                Sl[kk[j]] = 0.0f;
-                                                Ll[kk[j]] = 0.0f;
-                                            } else {
-                                                Sl[kk[j]] = sn;
-                                                Ll[kk[j]] = dW;
+                                        for (int j = 0; j < U; ++j) {
+                                            if (o + j * rpp < no) {
+                                                float dW = __fadd_rn(__fmul_rn(bv[j], a), __fmul_rn(mom, lv[j]));
+                                                dW = __fadd_rn(dW, t1);
+                                                dW = __fadd_rn(dW, t2);
+                                                const float sn = __fadd_rn(sv[j], dW);
+                                                if (apply) {
+                                                    Wl[kk[j]] = __fsub_rn(wv[j], __fdiv_rn(sn, fmb));
+                                                    Sl[kk[j]] = 0.0f;
+                                                    Ll[kk[j]] = 0.0f;
+                                                } else {
+                                                    Sl[kk[j]] = sn;
+                                                    Ll[kk[j]] = dW;
+                                                }
                                             }
                                         }
                                     }
                                 }
-                            }
+                            };
+                            if (no <= rpp) push(IC<1>{});
+                            else push(IC<4>{});
                         } else
                         for (int i = i0; i < ni; i += tw) {
                             if (kDrop && mi[i]) continue;
@@ -461,6 +532,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                                 }
                             }
                         }
+                        }
                     }
                     // ---- scalar bias of the in-layer (network.cpp:654-656)
                     // The n_in*n_out subtractions are one dependent chain; it runs in the last
@@ -482,7 +554,9 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         }
                         if (walked) {
                         } else if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
-                            if (no <= 4) b = bias_chain<4>(b, bs, no, nv, mk);
+                            if (no == 1) b = bias_chain<1>(b, bs, no, nv, mk);
+                            else if (no == 2) b = bias_chain<2>(b, bs, no, nv, mk);
+                            else if (no <= 4) b = bias_chain<4>(b, bs, no, nv, mk);
                             else if (no <= 8) b = bias_chain<8>(b, bs, no, nv, mk);
                             else if (no <= 16) b = bias_chain<16>(b, bs, no, nv, mk);
                             else if (no <= 32) b = bias_chain<32>(b, bs, no, nv, mk);
@@ -500,7 +574,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         }
                         if (tid == serial) sbias[l] = b;
                     }
-                    row_barrier<kLds>();
+                    row_barrier<kLds, kWave>();
                     // ---- error partials of the in-layer with the UPDATED weights
                     //      (network.cpp:660-662), then its own d and lr*d for the next round
                     if (l != 0) {
@@ -529,8 +603,9 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                             float d = __fmul_rn(e, ghip_act_der_ref(ain[i], actp, 0.01f));
                             dn[i] = d;
                             bn[i] = __fmul_rn(lrn, d);
+                            if (kWave) break;
                         }
-                        row_barrier<kLds>();
+                        row_barrier<kLds, kWave>();
                     }
                     if (kDrop && Lo < L) {
                         // clearErrDer of the out-layer's nodes: only by a valid pair with the last
@@ -538,11 +613,11 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                         if (!mi[ni - 1])
                             for (int o = tid; o < no; o += T)
                                 if (!mo[o]) sE[p.aoff[Lo] + o] = 0.0f;
-                        row_barrier<kLds>();
+                        row_barrier<kLds, kWave>();
                     }
                 }
             } else {
-                row_barrier<kLds>();  // the metrics lane reads this row's outputs and targets: the next row waits
+                row_barrier<kLds, kWave>();  // the metrics lane reads this row's outputs and targets: the next row waits
             }
             if (++rmod == p.mb) rmod = 0;
         }
@@ -574,6 +649,305 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     if (tid == 0) own.epochs_run[0] = ep;
     if (kDrop)
         for (int k = tid; k < p.node_floats; k += T) own.errder[k] = sE[k];
+}
+
+// ---------------------------------------------------------------- one wavefront per network
+// The same rows, the same arithmetic in the same order, for the networks this is about most often: a few layers
+// of at most 64 nodes, state in LDS, no dropout.  One wavefront runs alone on its SIMD and issues an instruction
+// every other issue slot at best (each step of a row depends on the one before), so what a row costs is the
+// number of instructions it executes.  Here that number is kept down: the layers are unrolled (kL of them), a
+// lane owns one node of every layer and one column of edges, nothing is a loop that is known to run once, the
+// layer biases and the row's targets stay in registers, the predicted class is found across the lanes, the kind
+// of bias chain is decided once per launch, and there is no barrier: LDS operations of one wavefront execute
+// in order.
+template <int NP>
+__device__ __forceinline__ float bias_chain_exact(float b, const float* bs, int ni)
+{
+    float x[NP];
+#pragma unroll
+    for (int k = 0; k < NP; ++k) x[k] = bs[k];
+    for (int i = 0; i < ni; ++i) {
+#pragma unroll
+        for (int k = 0; k < NP; ++k) b = __fsub_rn(b, x[k]);
+    }
+    return b;
+}
+
+__device__ __forceinline__ void wave_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+template <int kL>
+__global__ void __launch_bounds__(64)
+exact_wave_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
+{
+    extern __shared__ float smem[];
+    const ExactPointers own = multi ? multi[blockIdx.x] : p.ptr;
+    const int lane = threadIdx.x;
+    constexpr int L = kL;
+    const int n0 = p.sizes[0];
+    const int nout = p.sizes[L];
+    const int S = p.state_floats;
+    // the layout of exact_kernel's LDS-resident instantiation (ghip_exact_lds_bytes sizes it)
+    float* sW = smem;
+    float* sSum = smem + S;
+    float* sLast = smem + 2 * S;
+    float* nodes = smem + 3 * S;
+    float* sa = nodes;
+    float* sd = nodes + p.node_floats;
+    float* sbase = nodes + 2 * p.node_floats;
+    float* sy = nodes + 3 * p.node_floats;
+    float* sbias = sy + nout;
+    int* sflag = (int*)(sbias + GHIP_MAX_LAYERS);
+    const int cap = p.metric_cap;
+    unsigned long long* sT = (unsigned long long*)(((uintptr_t)(sflag + 4) + 7) & ~(uintptr_t)7);
+    float* rp = (float*)(sT + 32);
+    float* re = rp + cap;
+    int fill = 0;
+
+    for (int k = lane; k < S; k += 64) {
+        sW[k] = own.W[k];
+        sSum[k] = own.wsum[k];
+        sLast[k] = own.wlast[k];
+    }
+    if (lane == 0) sflag[0] = 0;
+    if (lane < 32) {
+        const unsigned long long tab[32] = GLM_EXP2_TAB;
+        sT[lane] = tab[lane];
+    }
+    float bias[kL];   // the scalar layer biases: every lane holds the same values
+#pragma unroll
+    for (int l = 0; l < kL; ++l) bias[l] = own.bias[l];
+
+    // how layer l's bias chain is walked: 0 the closed form of the other bias mode, 1..8 / 16 / 32 / 64 that many
+    // values per round held in registers; +128: first see whether the integer-grid shortcut applies
+    int chain[kL];
+#pragma unroll
+    for (int l = 1; l < kL; ++l) {
+        const int ni = p.sizes[l], no = p.sizes[l + 1];
+        int c = 0;
+        if (p.bias_mode == GHIP_BIAS_SEQUENTIAL) {
+            c = no <= 8 ? no : (no <= 16 ? 16 : (no <= 32 ? 32 : 64));
+            if ((long long)ni * no >= kGridChainMin) c += 128;
+        }
+        chain[l] = c;
+    }
+
+    const float data_size = (float)((unsigned)p.n_rows * (unsigned)nout);
+    const float fmb = (float)p.mb;
+    float px = lane < n0 ? p.X[lane] : 0.0f;
+    float py = lane < nout ? p.Y[lane] : 0.0f;
+    __syncthreads();
+
+    int ep = 0;
+    for (; ep < p.n_epochs; ++ep) {
+        float tot_err = 0.0f, tot_acc = 0.0f;
+        long long correct = 0;
+        const bool last_epoch = (ep == p.n_epochs - 1) || (p.stop_accuracy > 0.0f);
+        if (own.cm) {  // CMatrix::reset at the head of every epoch (network.cpp:183-185)
+            for (int k = lane; k < nout * nout; k += 64) own.cm[k] = 0;
+            __threadfence();
+            __syncthreads();
+        }
+        int rmod = 0;  // r % mb
+        for (long long r = 0; r < p.n_rows; ++r) {
+            // ---- the row (fetched while the row before was worked on) and the request for the next one
+            if (lane < n0) sa[lane] = px;
+            const float yv = py;   // lane o: expected value of output o
+            {
+                long long rn = r + 1;
+                if (rn == p.n_rows) rn = 0;
+                px = lane < n0 ? p.X[rn * n0 + lane] : 0.0f;
+                py = lane < nout ? p.Y[rn * nout + lane] : 0.0f;
+            }
+            wave_sync();
+
+            // ---- ForwardPass (network.cpp:457-516)
+            float pv = 0.0f;       // lane o: output o
+#pragma unroll
+            for (int l = 0; l < kL; ++l) {
+                const int ni = p.sizes[l], no = p.sizes[l + 1], ld = p.ld[l];
+                if (lane < no) {
+                    float z = fold8(0.0f, sW + p.woff[l] + lane * ld, 1, sa + p.aoff[l], 1, ni,
+                                    [](float acc, float wv, float av) { return __fadd_rn(acc, __fmul_rn(wv, av)); });
+                    if (l != 0) z = __fadd_rn(z, bias[l]);
+                    const float a = ghip_squash<true>(z, p.act[l], p.act_param[l], (const uint64_t*)sT);
+                    sa[p.aoff[l + 1] + lane] = a;
+                    if (l == kL - 1) {
+                        rp[fill + lane] = a;
+                        re[fill + lane] = yv;
+                        pv = a;
+                    }
+                }
+                wave_sync();
+            }
+            fill += nout;
+            if (own.preds && last_epoch && lane < nout) own.preds[r * nout + lane] = pv;
+
+            // ---- output metrics (network.cpp:519-559).  The scan "strictly greater than the best so far, starting
+            // from 0" ends on the first index that holds the largest value above 0 (none: -1), and a NaN never
+            // compares greater: across the lanes that is the maximum (the hardware's max passes over a NaN operand),
+            // then the lowest lane that holds it.
+            {
+                const float pr = lane < nout ? pv : 0.0f, ex = lane < nout ? yv : 0.0f;
+                auto fmax_op = [](int a, int c) { return __float_as_int(fmaxf(__int_as_float(a), __int_as_float(c))); };
+                const float mp = __int_as_float(__builtin_amdgcn_readlane(wave_scan(__float_as_int(pr), 0, fmax_op), 63));
+                const float my = __int_as_float(__builtin_amdgcn_readlane(wave_scan(__float_as_int(ex), 0, fmax_op), 63));
+                const unsigned long long bp = __ballot(pr == mp && pr > 0.0f), by = __ballot(ex == my && ex > 0.0f);
+                const int ip = bp ? __builtin_ctzll(bp) : -1, iy = by ? __builtin_ctzll(by) : -1;
+                if (ip == iy) ++correct;
+                // CMatrix::addResult (cmatrix.cpp:57-98): row = expected class, column = predicted
+                if (lane == 63 && own.cm && ip >= 0 && iy >= 0) atomicAdd(&own.cm[iy * nout + ip], 1);
+            }
+            // cost and accuracy once the ring of (predicted, expected) pairs is full: the terms a lane each, the two
+            // running sums in visiting order
+            if (fill + nout > cap || r == p.n_rows - 1) {
+                wave_sync();
+                for (int k = lane; k < fill; k += 64) {
+                    const float pr = rp[k], ex = re[k];
+                    rp[k] = ghip_cost<true>(ex, pr, data_size, p.cost);
+                    re[k] = ghip_accuracy_term(pr, ex);
+                }
+                wave_sync();
+                for (int k = 0; k < fill; ++k) {   // every lane walks the same sums
+                    tot_err = __fadd_rn(tot_err, rp[k]);
+                    tot_acc = __fadd_rn(tot_acc, re[k]);
+                }
+                wave_sync();
+                fill = 0;
+            }
+
+            if (p.train) {
+                // output layer: errDer = 0 + costErrDer, derivative 1 (network.cpp:599-612)
+                if (lane < nout) {
+                    const float e = __fadd_rn(0.0f, ghip_cost_der(yv, pv, p.cost));
+                    sd[p.aoff[L] + lane] = e;
+                    sbase[p.aoff[L] + lane] = __fmul_rn(p.lr[L - 1], e);
+                }
+                wave_sync();
+                const bool apply = rmod == 0;
+#pragma unroll
+                for (int Lo = kL; Lo > 0; --Lo) {
+                    const int l = Lo - 1;
+                    const int ni = p.sizes[l], no = p.sizes[Lo], ld = p.ld[l];
+                    float* Wl = sW + p.woff[l];
+                    float* Sl = sSum + p.woff[l];
+                    float* Ll = sLast + p.woff[l];
+                    const float* ain = sa + p.aoff[l];
+                    const float* dl = sd + p.aoff[Lo];
+                    const float* bs = sbase + p.aoff[Lo];
+                    const float lr = p.lr[l], mom = p.mom[l];
+                    const float w1 = __fmul_rn(p.wd1[l], lr), w2 = __fmul_rn(p.wd2[l], lr);
+                    // ---- per-edge delta push and conditional apply (node.cpp:278-307): lane groups of tw lanes
+                    //      walk a row of edges each (tw = the layer's width rounded up to a power of two)
+                    {
+                        const int sh = p.tw_log2[l];
+                        const int i = lane & ((1 << sh) - 1), o0 = lane >> sh, rpp = 64 >> sh;
+                        if (i < ni) {
+                            const float a = ain[i];
+                            const float t1 = __fmul_rn(w1, fabsf(a));
+                            const float t2 = __fmul_rn(w2, a);
+                            auto edge = [&](int o) {
+                                const int k = o * ld + i;
+                                const float bv = bs[o], lv = Ll[k], sv = Sl[k];
+                                float dW = __fadd_rn(__fmul_rn(bv, a), __fmul_rn(mom, lv));
+                                dW = __fadd_rn(dW, t1);
+                                dW = __fadd_rn(dW, t2);
+                                const float sn = __fadd_rn(sv, dW);
+                                if (apply) {
+                                    Wl[k] = __fsub_rn(Wl[k], __fdiv_rn(sn, fmb));
+                                    Sl[k] = 0.0f;
+                                    Ll[k] = 0.0f;
+                                } else {
+                                    Sl[k] = sn;
+                                    Ll[k] = dW;
+                                }
+                            };
+                            if (no <= rpp) {
+                                if (o0 < no) edge(o0);
+                            } else {
+                                for (int o = o0; o < no; o += rpp) edge(o);
+                            }
+                        }
+                    }
+                    // ---- scalar bias of the in-layer (network.cpp:654-656): n_in rounds of n_out subtractions
+                    if (l != 0) {
+                        float b = bias[l];
+                        int c = chain[l];
+                        bool walked = false;
+                        if (c & 128) {
+                            walked = bias_chain_grid(b, lane < no ? bs[lane] : 0.0f, ni, lane, &b);
+                            c &= 127;
+                        }
+                        if (!walked) {
+                            switch (c) {
+                            case 1: b = bias_chain_exact<1>(b, bs, ni); break;
+                            case 2: b = bias_chain_exact<2>(b, bs, ni); break;
+                            case 3: b = bias_chain_exact<3>(b, bs, ni); break;
+                            case 4: b = bias_chain_exact<4>(b, bs, ni); break;
+                            case 5: b = bias_chain_exact<5>(b, bs, ni); break;
+                            case 6: b = bias_chain_exact<6>(b, bs, ni); break;
+                            case 7: b = bias_chain_exact<7>(b, bs, ni); break;
+                            case 8: b = bias_chain_exact<8>(b, bs, ni); break;
+                            case 16: b = bias_chain<16>(b, bs, no, ni); break;
+                            case 32: b = bias_chain<32>(b, bs, no, ni); break;
+                            case 64: b = bias_chain<64>(b, bs, no, ni); break;
+                            default: {
+                                float sum = 0.0f;
+                                for (int o = 0; o < no; ++o) sum = __fadd_rn(sum, bs[o]);
+                                b = __fsub_rn(b, __fmul_rn((float)ni, sum));
+                            }
+                            }
+                        }
+                        bias[l] = b;
+                    }
+                    wave_sync();
+                    // ---- error partials of the in-layer with the UPDATED weights (network.cpp:660-662), then its
+                    //      own d and lr*d for the next round
+                    if (l != 0) {
+                        if (lane < ni) {
+                            const float e = fold8(0.0f, dl, 1, Wl + lane, ld, no,
+                                                  [](float acc, float dv, float wv) { return __fadd_rn(acc, __fadd_rn(acc, __fmul_rn(dv, wv))); });
+                            // the reference always passes 0.01 here (network.cpp:617-618)
+                            const float d = __fmul_rn(e, ghip_act_der_ref(ain[lane], p.act[l - 1], 0.01f));
+                            sd[p.aoff[l] + lane] = d;
+                            sbase[p.aoff[l] + lane] = __fmul_rn(p.lr[l - 1], d);
+                        }
+                        wave_sync();
+                    }
+                }
+            }
+            if (++rmod == p.mb) rmod = 0;
+        }
+        // ---- end of epoch (network.cpp:193-195, Terminator.cpp:73-74)
+        if (lane == 63) {
+            const float acc = __fdiv_rn(tot_acc, __fmul_rn((float)(unsigned)p.n_rows, (float)(unsigned)nout));
+            ghip_metrics* m = ((ghip_metrics*)own.metrics) + ep;
+            m->loss = tot_err;
+            m->accuracy = acc;
+            m->correct = correct;
+            if (own.cm && own.class_metrics) {  // network.cpp:218-224, read back through the atomics' path
+                __threadfence();
+                ghip_cmatrix_overall(own.cm, nout, own.class_metrics + 5 * ep);
+            }
+            if (p.stop_accuracy > 0.0f && acc >= p.stop_accuracy) sflag[0] = 1;
+        }
+        __syncthreads();
+        if (sflag[0]) { ++ep; break; }
+    }
+
+    for (int k = lane; k < S; k += 64) {
+        own.W[k] = sW[k];
+        own.wsum[k] = sSum[k];
+        own.wlast[k] = sLast[k];
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int l = 0; l < kL; ++l) own.bias[l] = bias[l];
+        own.epochs_run[0] = ep;
+    }
 }
 
 // GMath::squash / activationErrDer / outputNodeCost / costErrDer over arrays, with exact mode's arithmetic
@@ -638,17 +1012,46 @@ size_t ghip_exact_lds_bytes(const ExactLaunch& p, bool state_in_lds, bool dropou
     return f * sizeof(float);
 }
 
+template <bool kLds, bool kDrop, int kL, int kMaxT>
+static hipError_t launch_sized(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads,
+                               size_t lds_bytes, hipStream_t s)
+{
+    if (kLds) {
+        hipError_t e = hipFuncSetAttribute((const void*)exact_kernel<kLds, kDrop, kL, kMaxT>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+    }
+    hipLaunchKernelGGL((exact_kernel<kLds, kDrop, kL, kMaxT>), dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
+    return hipGetLastError();
+}
+
+template <bool kLds, bool kDrop, int kL>
+static hipError_t launch_layers(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads,
+                                size_t lds_bytes, hipStream_t s)
+{
+    bool narrow = true;   // every layer fits the lanes of one wavefront
+    for (int l = 0; l <= p.n_layers; ++l) narrow = narrow && p.sizes[l] <= 64;
+    if (kL > 0 && kLds && !kDrop && threads == 64 && narrow) {
+        hipError_t e = hipFuncSetAttribute((const void*)exact_wave_kernel<(kL > 0 ? kL : 1)>,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL((exact_wave_kernel<(kL > 0 ? kL : 1)>), dim3(count), dim3(64), lds_bytes, s, p, dev_multi);
+        return hipGetLastError();
+    }
+    if (kL > 0 && kLds && threads == 64 && narrow) return launch_sized<kLds, kDrop, kL, 64>(p, dev_multi, count, threads, lds_bytes, s);
+    if (kL > 0 && threads <= 256) return launch_sized<kLds, kDrop, kL, 256>(p, dev_multi, count, threads, lds_bytes, s);
+    if (kL > 0 && threads <= 512) return launch_sized<kLds, kDrop, kL, 512>(p, dev_multi, count, threads, lds_bytes, s);
+    return launch_sized<kLds, kDrop, kL, 1024>(p, dev_multi, count, threads, lds_bytes, s);
+}
+
 template <bool kLds, bool kDrop>
 static hipError_t launch_variant(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads,
                                  size_t lds_bytes, hipStream_t s)
 {
-    if (kLds) {
-        hipError_t e = hipFuncSetAttribute((const void*)exact_kernel<kLds, kDrop>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return e;
-    }
-    hipLaunchKernelGGL((exact_kernel<kLds, kDrop>), dim3(count), dim3(threads), lds_bytes, s, p, dev_multi);
-    return hipGetLastError();
+    // the common depths have their own instantiation (one and two hidden layers)
+    if (kLds && p.n_layers == 2) return launch_layers<kLds, kDrop, 2>(p, dev_multi, count, threads, lds_bytes, s);
+    if (kLds && p.n_layers == 3) return launch_layers<kLds, kDrop, 3>(p, dev_multi, count, threads, lds_bytes, s);
+    return launch_layers<kLds, kDrop, 0>(p, dev_multi, count, threads, lds_bytes, s);
 }
 
 hipError_t ghip_launch_exact(const ExactLaunch& p, const ExactPointers* dev_multi, int count, int threads, size_t lds_bytes,
