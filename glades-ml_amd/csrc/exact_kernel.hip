@@ -93,22 +93,22 @@ __device__ __forceinline__ float fold8(float z, const float* x, int xs, const fl
         if (nb - b == 2) { fetch(xb, yb, b + 1); run(xa, ya); run(xb, yb); }
         else run(xa, ya);
     }
-    // the last n % 8 steps: blocks of 4, 2 and 1, each block's operands asked for together (a loop would pay
-    // an LDS round trip per step, which for the 4-input layer of a small network is the whole dot product)
-    int i = nb * B;
-    auto block = [&](auto cnt) {
-        constexpr int C = decltype(cnt)::value;
-        float xv[C], yv[C];
+    // the last n % 8 steps: their operands asked for together (a loop would pay an LDS round trip per step,
+    // which for the 4-input layer of a small network is the whole dot product); past the end the last pair is
+    // read again and not used
+    const int rem = n - nb * B;
+    if (rem > 0) {
+        float xv[B - 1], yv[B - 1];
 #pragma unroll
-        for (int j = 0; j < C; ++j) { xv[j] = x[(i + j) * xs]; yv[j] = y[(i + j) * ys]; }
+        for (int j = 0; j < B - 1; ++j) {
+            const int i = nb * B + (j < rem ? j : rem - 1);
+            xv[j] = x[i * xs]; yv[j] = y[i * ys];
+        }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < C; ++j) z = step(z, xv[j], yv[j]);
-        i += C;
-    };
-    if (n & 4) block(IC<4>{});
-    if (n & 2) block(IC<2>{});
-    if (n & 1) block(IC<1>{});
+        for (int j = 0; j < B - 1; ++j)
+            if (j < rem) z = step(z, xv[j], yv[j]);
+    }
     return z;
 }
 
@@ -205,7 +205,7 @@ template <bool kLds, bool kDrop, int kL, int kMaxT>
 __global__ void __launch_bounds__(kMaxT)
 exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 {
-    extern __shared__ float smem[];
+    extern __shared__ __align__(16) float smem[];
     const ExactPointers own = multi ? multi[blockIdx.x] : p.ptr;
     // one wavefront per network (the small networks: LDS-resident, at most 64 lanes of work per phase)
     constexpr bool kWave = kLds && kMaxT == 64;
@@ -245,7 +245,9 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     // are computed a ring-full at a time, one lane each, and summed in visiting order afterwards
     const int cap = p.metric_cap;
     // the 2^(i/32) table of expf, so that a sigmoid costs an LDS read instead of a trip to memory
-    unsigned long long* sT = (unsigned long long*)(((uintptr_t)(sflag + 4) + 7) & ~(uintptr_t)7);
+    // (8-byte aligned; found by index arithmetic: a pointer that went through an integer is a generic one to the
+    // compiler, and a generic load also waits for every global load in flight, the next row's prefetch included)
+    unsigned long long* sT = (unsigned long long*)(smem + ((((float*)(sflag + 4) - smem) + 1) & ~(ptrdiff_t)1));
     float* rp = (float*)(sT + 32);
     float* re = rp + cap;
     int fill = 0;
@@ -405,11 +407,9 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     re[k] = ghip_accuracy_term(pr, ex);
                 }
                 row_barrier<kLds, kWave>();
-                if (tid == serial) {
-                    for (int k = 0; k < fill; ++k) {
-                        tot_err = __fadd_rn(tot_err, rp[k]);
-                        tot_acc = __fadd_rn(tot_acc, re[k]);
-                    }
+                if (tid == serial) {   // eight terms per LDS round trip
+                    tot_err = fold8(tot_err, rp, 1, rp, 1, fill, [](float acc, float v, float) { return __fadd_rn(acc, v); });
+                    tot_acc = fold8(tot_acc, re, 1, re, 1, fill, [](float acc, float v, float) { return __fadd_rn(acc, v); });
                 }
                 fill = 0;
             }
@@ -666,6 +666,7 @@ __device__ __forceinline__ float bias_chain_exact(float b, const float* bs, int 
     float x[NP];
 #pragma unroll
     for (int k = 0; k < NP; ++k) x[k] = bs[k];
+#pragma unroll 4
     for (int i = 0; i < ni; ++i) {
 #pragma unroll
         for (int k = 0; k < NP; ++k) b = __fsub_rn(b, x[k]);
@@ -683,7 +684,7 @@ template <int kL>
 __global__ void __launch_bounds__(64)
 exact_wave_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 {
-    extern __shared__ float smem[];
+    extern __shared__ __align__(16) float smem[];
     const ExactPointers own = multi ? multi[blockIdx.x] : p.ptr;
     const int lane = threadIdx.x;
     constexpr int L = kL;
@@ -702,7 +703,9 @@ exact_wave_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     float* sbias = sy + nout;
     int* sflag = (int*)(sbias + GHIP_MAX_LAYERS);
     const int cap = p.metric_cap;
-    unsigned long long* sT = (unsigned long long*)(((uintptr_t)(sflag + 4) + 7) & ~(uintptr_t)7);
+    // (8-byte aligned; found by index arithmetic: a pointer that went through an integer is a generic one to the
+    // compiler, and a generic load also waits for every global load in flight, the next row's prefetch included)
+    unsigned long long* sT = (unsigned long long*)(smem + ((((float*)(sflag + 4) - smem) + 1) & ~(ptrdiff_t)1));
     float* rp = (float*)(sT + 32);
     float* re = rp + cap;
     int fill = 0;
@@ -811,10 +814,9 @@ exact_wave_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     re[k] = ghip_accuracy_term(pr, ex);
                 }
                 wave_sync();
-                for (int k = 0; k < fill; ++k) {   // every lane walks the same sums
-                    tot_err = __fadd_rn(tot_err, rp[k]);
-                    tot_acc = __fadd_rn(tot_acc, re[k]);
-                }
+                // every lane walks the same two sums, eight terms per LDS round trip
+                tot_err = fold8(tot_err, rp, 1, rp, 1, fill, [](float acc, float v, float) { return __fadd_rn(acc, v); });
+                tot_acc = fold8(tot_acc, re, 1, re, 1, fill, [](float acc, float v, float) { return __fadd_rn(acc, v); });
                 wave_sync();
                 fill = 0;
             }
@@ -845,30 +847,33 @@ exact_wave_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                     {
                         const int sh = p.tw_log2[l];
                         const int i = lane & ((1 << sh) - 1), o0 = lane >> sh, rpp = 64 >> sh;
-                        if (i < ni) {
+                        auto edge = [&](int k, float a, float t1, float t2, float bv, float lv, float sv) {
+                            float dW = __fadd_rn(__fmul_rn(bv, a), __fmul_rn(mom, lv));
+                            dW = __fadd_rn(dW, t1);
+                            dW = __fadd_rn(dW, t2);
+                            const float sn = __fadd_rn(sv, dW);
+                            if (apply) {
+                                Wl[k] = __fsub_rn(Wl[k], __fdiv_rn(sn, fmb));
+                                Sl[k] = 0.0f;
+                                Ll[k] = 0.0f;
+                            } else {
+                                Sl[k] = sn;
+                                Ll[k] = dW;
+                            }
+                        };
+                        if (no <= rpp) {
+                            // one edge per lane: its four operands in one LDS round trip (an idle lane reads edge 0)
+                            const bool mine = i < ni && o0 < no;
+                            const int ic = mine ? i : 0, oc = mine ? o0 : 0, k = oc * ld + ic;
+                            const float a = ain[ic], bv = bs[oc], lv = Ll[k], sv = Sl[k];
+                            if (mine) edge(k, a, __fmul_rn(w1, fabsf(a)), __fmul_rn(w2, a), bv, lv, sv);
+                        } else if (i < ni) {
                             const float a = ain[i];
                             const float t1 = __fmul_rn(w1, fabsf(a));
                             const float t2 = __fmul_rn(w2, a);
-                            auto edge = [&](int o) {
+                            for (int o = o0; o < no; o += rpp) {
                                 const int k = o * ld + i;
-                                const float bv = bs[o], lv = Ll[k], sv = Sl[k];
-                                float dW = __fadd_rn(__fmul_rn(bv, a), __fmul_rn(mom, lv));
-                                dW = __fadd_rn(dW, t1);
-                                dW = __fadd_rn(dW, t2);
-                                const float sn = __fadd_rn(sv, dW);
-                                if (apply) {
-                                    Wl[k] = __fsub_rn(Wl[k], __fdiv_rn(sn, fmb));
-                                    Sl[k] = 0.0f;
-                                    Ll[k] = 0.0f;
-                                } else {
-                                    Sl[k] = sn;
-                                    Ll[k] = dW;
-                                }
-                            };
-                            if (no <= rpp) {
-                                if (o0 < no) edge(o0);
-                            } else {
-                                for (int o = o0; o < no; o += rpp) edge(o);
+                                edge(k, a, t1, t2, bs[o], Ll[k], Sl[k]);
                             }
                         }
                     }
