@@ -198,9 +198,9 @@ __device__ __forceinline__ void row_barrier()
 // kL: the number of layers where it is known at compile time (0: read from p).  With it the loops over the layers
 // unroll, every p.x[l] becomes a fixed kernel-argument slot that is read once into a scalar register, and the
 // per-layer code is laid out straight.  The arithmetic and its order are the same.
-// kMaxT: the most threads a launch of this instantiation has.  The register file is shared by the wavefronts a
-// workgroup may have: 128 registers per lane at 1024 threads, 256 at 512, 512 at 256.  At 128 the row loop keeps
-// addresses in scratch memory, and every reload waits for the next row's prefetch as well.
+// kMaxT: the most threads a launch of this instantiation has: 1024, or 64 for the networks that one wavefront
+// serves (below).  Instantiations for 256 and 512 threads, which may use two and four times the registers, gained
+// nothing for one network and halved the networks a compute unit holds in a launch over many.
 template <bool kLds, bool kDrop, int kL, int kMaxT>
 __global__ void __launch_bounds__(kMaxT)
 exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
@@ -680,8 +680,11 @@ __device__ __forceinline__ void wave_sync()
     __builtin_amdgcn_wave_barrier();
 }
 
-template <int kL>
-__global__ void __launch_bounds__(64)
+// kOcc: wavefronts per SIMD the register budget must allow.  2 (all the registers the code likes) is fastest for
+// a launch that leaves SIMDs idle anyway; 4 costs one network 10 % and lets a launch over thousands of them
+// keep four per SIMD, whose instructions fill each other's waiting slots.
+template <int kL, int kOcc>
+__global__ void __launch_bounds__(64, kOcc)
 exact_wave_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
 {
     extern __shared__ __align__(16) float smem[];
@@ -1036,16 +1039,19 @@ static hipError_t launch_layers(const ExactLaunch& p, const ExactPointers* dev_m
 {
     bool narrow = true;   // every layer fits the lanes of one wavefront
     for (int l = 0; l <= p.n_layers; ++l) narrow = narrow && p.sizes[l] <= 64;
-    if (kL > 0 && kLds && !kDrop && threads == 64 && narrow) {
-        hipError_t e = hipFuncSetAttribute((const void*)exact_wave_kernel<(kL > 0 ? kL : 1)>,
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL((exact_wave_kernel<(kL > 0 ? kL : 1)>), dim3(count), dim3(64), lds_bytes, s, p, dev_multi);
-        return hipGetLastError();
-    }
-    if (kL > 0 && kLds && threads == 64 && narrow) return launch_sized<kLds, kDrop, kL, 64>(p, dev_multi, count, threads, lds_bytes, s);
-    if (kL > 0 && threads <= 256) return launch_sized<kLds, kDrop, kL, 256>(p, dev_multi, count, threads, lds_bytes, s);
-    if (kL > 0 && threads <= 512) return launch_sized<kLds, kDrop, kL, 512>(p, dev_multi, count, threads, lds_bytes, s);
+    if constexpr (kL > 0 && kLds && !kDrop)
+        if (threads == 64 && narrow) {
+            // 256 compute units x 4 SIMDs x 2 wavefronts hold 2048 networks at the larger register budget
+            const bool crowded = count > 2048;
+            const void* fn = crowded ? (const void*)exact_wave_kernel<kL, 4> : (const void*)exact_wave_kernel<kL, 2>;
+            hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return e;
+            if (crowded) hipLaunchKernelGGL((exact_wave_kernel<kL, 4>), dim3(count), dim3(64), lds_bytes, s, p, dev_multi);
+            else hipLaunchKernelGGL((exact_wave_kernel<kL, 2>), dim3(count), dim3(64), lds_bytes, s, p, dev_multi);
+            return hipGetLastError();
+        }
+    if constexpr (kL > 0 && kLds)
+        if (threads == 64 && narrow) return launch_sized<kLds, kDrop, kL, 64>(p, dev_multi, count, threads, lds_bytes, s);
     return launch_sized<kLds, kDrop, kL, 1024>(p, dev_multi, count, threads, lds_bytes, s);
 }
 

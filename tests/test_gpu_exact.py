@@ -193,6 +193,39 @@ def test_error_paths():
     net.close()
 
 
+def test_a_crowded_launch_equals_the_solo_runs():
+    """More than 2048 small networks in one launch run the instantiation with the smaller register budget
+    (four wavefronts per SIMD): 2100 copies of four differently initialised networks, every one of which
+    must end bit for bit where its solo run (the other instantiation) ends."""
+    import pyglades as pg
+    c = load_case("window_4_5_3_1")
+    rng = np.random.default_rng(22)
+    K, E, V = 2100, 3, 4
+    variants = [[(c["W0"][l] + rng.normal(0, 0.05, c["W0"][l].shape)).astype(np.float32) for l in range(c["nl"])] for _ in range(V)]
+    want, want_W = [], []
+    for Ws in variants:
+        n = gpu_net(c)
+        for l in range(c["nl"]):
+            n.set_params(l, Ws[l], c["bias0"][l])
+        want.append(n.run_epochs_exact(E)[0])
+        want_W.append([n.get_params(l) for l in range(c["nl"])])
+        n.close()
+    group = []
+    for k in range(K):
+        n = gpu_net(c)
+        for l in range(c["nl"]):
+            n.set_params(l, variants[k % V][l], c["bias0"][l])
+        group.append(n)
+    got = pg.run_epochs_exact_multi(group, E)
+    assert all(got[k] == want[k % V] for k in range(K))
+    for k in list(range(0, K, 97)) + [K - 1]:
+        for l in range(c["nl"]):
+            W, b = group[k].get_params(l)
+            assert np.array_equal(W, want_W[k % V][l][0]) and np.array_equal(b, want_W[k % V][l][1]), (k, l)
+    for n in group:
+        n.close()
+
+
 def test_many_networks_in_one_launch_equal_their_solo_runs():
     """ghip_net_run_epochs_exact_multi: one workgroup per network; every network ends exactly where
     it ends when it runs alone (metrics of every epoch, weights, biases, delta windows)."""
