@@ -19,6 +19,9 @@ The default run adds, outside the timed region and under "detail" (--no-extras l
                its own roofline entry
   vendor_gemm  the vendor library's plain bf16 GEMM on the step's two product shapes: what the chip
                sustains on them, beside the published peak
+  other_configs  BASELINE.json's other configurations at their default step counts, value and ms per
+               step each: cfg3 (fp32 training), cfg1 and cfg2 (exact mode, one network), and cfg1 with
+               1024 networks side by side in one launch
 """
 import argparse
 import ctypes
@@ -360,7 +363,7 @@ def main():
     ap.add_argument("--workload", default="cfg4", choices=sorted(WORKLOADS) + ["copy"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
-                    help="cfg4: skip the untimed extras (fp32 loss check, 200-step sustained rate, cfg5 inference leg, vendor GEMM rates)")
+                    help="cfg4: skip the untimed extras (fp32 loss check, 200-step sustained rate, cfg5 inference leg, vendor GEMM rates, the other configurations)")
     ap.add_argument("--subnets", type=int, default=1,
                     help="exact workloads: this many networks (MetaNetwork subnets) side by side in one launch; value is their sum")
     args = ap.parse_args()
@@ -415,6 +418,20 @@ def main():
             extra["vendor_gemm"] = vendor_gemm_rates(w["sizes"], w["batch"])
         except Exception as e:  # noqa: BLE001
             extra["vendor_gemm"] = dict(error=repr(e))
+        others = {}
+        for name, subnets in (("cfg3", 1), ("cfg1", 1), ("cfg2", 1), ("cfg1", 1024)):
+            key = name if subnets == 1 else f"{name}_x{subnets}"
+            try:
+                wo = dict(WORKLOADS[name], name=name)
+                ao = argparse.Namespace(steps={"cfg3": 200, "cfg2": 5, "cfg1": 200}[name], warmup={"cfg3": 20, "cfg2": 1, "cfg1": 5}[name],
+                                        extras=False, subnets=subnets)
+                vo, elo, roofo, _ = run_exact(wo, ao) if wo["kind"] == "exact" else run_canonical(wo, ao)
+                others[key] = dict(value=round(vo, 1), unit="samples/s", steps=ao.steps, ms_per_step=round(elo / ao.steps * 1e3, 4),
+                                   dtype=wo["dtype"], workload=f"{name}: {wo['desc']}" + (f", {subnets} subnets side by side" if subnets > 1 else ""),
+                                   kernel=roofo["kernel"], kernel_avg_launch_ms=roofo["avg_launch_ms"])
+            except Exception as e:  # noqa: BLE001
+                others[key] = dict(error=repr(e))
+        extra["other_configs"] = others
     out = {
         "metric": "train samples/sec (fwd+bwd+update)" if w["kind"] != "infer" else "infer samples/sec",
         "value": round(value, 1), "unit": "samples/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
