@@ -280,6 +280,8 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
     // (the single-wavefront instantiation is launched for layers of at most 64 nodes: one value per lane)
     constexpr int kPf = kWave ? 1 : kPrefetch;
     const bool small_row = kWave || ((n0 <= kPrefetch * T) && (nout <= kPrefetch * T));
+    // chunks of T values a row and its targets really have (the rest of the kPf slots is skipped, not masked)
+    const int nchunk = kWave ? 1 : ((n0 > nout ? n0 : nout) + T - 1) / T;
 
     // first row into registers
     float px[kPf], py[kPf];
@@ -307,6 +309,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
             if (small_row) {
 #pragma unroll
                 for (int j = 0; j < kPf; ++j) {
+                    if (j >= nchunk) break;
                     int i = tid + j * T;
                     if (i < n0) sa[i] = px[j];
                     if (i < nout) sy[i] = py[j];
@@ -317,6 +320,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                 const float* yn = p.Y + rn * nout;
 #pragma unroll
                 for (int j = 0; j < kPf; ++j) {
+                    if (j >= nchunk) break;
                     int i = tid + j * T;
                     px[j] = (i < n0) ? xn[i] : 0.0f;
                     py[j] = (i < nout) ? yn[i] : 0.0f;
