@@ -182,6 +182,44 @@ def test_bf16_steps_off_the_tile_grid(B):
     g.close()
 
 
+def test_bf16_off_grid_state_round_trip():
+    """Momentum of a padded network out and in again (what a checkpoint does): two copies of a network off the
+    tile grid take two steps; one hands its parameters and optimiser state to the host and takes them
+    back (setting parameters clears the momentum, so the state has to arrive for the next step to agree);
+    after a third step both hold the same bits."""
+    import pyglades as pg
+    print("bf16 off-grid state", flush=True)
+    rng = np.random.default_rng(31)
+    sizes, acts, B = [100, 300, 70], [po.RELU, po.SOFTMAX], 200
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * np.sqrt(2.0 / sizes[l])).astype(np.float32) for l in range(2)]
+    X = rng.standard_normal((3 * B, sizes[0])).astype(np.float32)
+    Y = teacher_labels(rng, X, sizes[-1])
+    nets = []
+    for _ in range(2):
+        g = pg.Net(pg.make_spec(sizes, acts, lr=0.1, mom=0.9, wd2=1e-4, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=pg.BF16))
+        for l in range(2):
+            g.set_params(l, Ws[l])
+        g.set_dataset(X, Y)
+        for s_ in range(2):
+            g.train_step(s_ * B, B)
+        nets.append(g)
+    a, b = nets
+    for l in range(2):
+        W, bias = b.get_params(l)
+        vW, vb = b.get_state(l)
+        assert vW.shape == Ws[l].shape and vb.shape == (sizes[l + 1],) and np.any(vW != 0) and np.any(vb != 0)
+        b.set_params(l, W, bias)
+        b.set_state(l, vW, vb)
+    la, lb = a.train_step(2 * B, B).loss, b.train_step(2 * B, B).loss
+    assert la == lb
+    for l in range(2):
+        (Wa, ba), (Wb, bb) = a.get_params(l), b.get_params(l)
+        assert np.array_equal(Wa, Wb) and np.array_equal(ba, bb), l
+        (va, vba), (vb_, vbb) = a.get_state(l), b.get_state(l)
+        assert np.array_equal(va, vb_) and np.array_equal(vba, vbb), l
+    a.close(); b.close()
+
+
 def test_bf16_pass_with_a_short_last_batch():
     """One training pass over 700 rows in batches of 256: 256, 256 and 188 rows.  The short batch follows
     two full ones in the same buffers, whose rows past 188 then hold the earlier batches' deltas unless
