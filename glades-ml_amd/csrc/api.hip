@@ -617,6 +617,8 @@ int step_bf16(ghip_net* n, int64_t row0, int batch)
         LAUNCH(n, "fill_pad_delta", ghip_fill_u32((unsigned int*)(n->D[L] + (size_t)batch * ps[L]), (long long)(B - batch) * ps[L] / 2, 0u, n->stream));
     TRY(output_delta_f32(n, n->logits, Y, nullptr, n->D[L], batch));
     LAUNCH(n, "bf16_transpose_delta", ghip_bf16_transpose(n->D[L], n->DT[L], B, ps[L], n->stream));
+    BiasStepArgs bias_args;
+    memset(&bias_args, 0, sizeof(bias_args));
     for (int l = L - 1; l >= 0; --l) {
         const int ni = ps[l], no = ps[l + 1];
         GemmLpArgs g;
@@ -628,11 +630,14 @@ int step_bf16(ghip_net* n, int64_t row0, int batch)
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1];
             LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));
         }
-        if (l + 1 < L)  // D[l+1] came from a back-propagation product, which left its column sums
-            LAUNCH(n, "bias_update_bf16", ghip_bias_update_partials(n->csum[l + 1], B / ghip_gemm_lp_tile_m(B, no), no, batch, n->b[l], n->vb[l],
-                                                                    s.lr[l], s.mom[l], n->stream));
-        else
-            LAUNCH(n, "bias_update_bf16", ghip_bias_update_bf16T(n->DT[l + 1], no, B, batch, n->b[l], n->vb[l], s.lr[l], s.mom[l], n->stream));
+        // the layer's bias update: from the column sums the back-propagation product that made D[l+1] left, or
+        // for the output layer from the transposed deltas; all of the step's in one launch after the products
+        {
+            BiasStepArgs::Entry& e = bias_args.e[bias_args.count++];
+            if (l + 1 < L) { e.part = n->csum[l + 1]; e.tiles = B / ghip_gemm_lp_tile_m(B, no); }
+            else { e.DT = n->DT[l + 1]; e.rows = B; }
+            e.n = no; e.batch = batch; e.bias = n->b[l]; e.vb = n->vb[l]; e.lr = s.lr[l]; e.mom = s.mom[l];
+        }
         memset(&g, 0, sizeof(g));
         // both operands K-blocked over the batch: [B / 64][nodes][64], a tile's stage one contiguous block
         g.A = n->DT[l + 1]; g.B = n->HT[l]; g.M = no; g.N = ni; g.K = B;
@@ -646,6 +651,7 @@ int step_bf16(ghip_net* n, int64_t row0, int batch)
         if (ghip_gemm_lp_tile_m(g.M, g.N) == 128) LAUNCH(n, "gemm_bf16_wgrad_sgd_t128", ghip_gemm_lp(g, n->stream));
         else LAUNCH(n, "gemm_bf16_wgrad_sgd", ghip_gemm_lp(g, n->stream));
     }
+    LAUNCH(n, "bias_update_bf16", ghip_bias_update_step(bias_args, n->stream));
     return 0;
 }
 

@@ -241,12 +241,11 @@ __global__ void __launch_bounds__(256) output_delta_vec4_kernel(DeltaArgs a)
 }
 
 // bf16 delta^T, K-blocked [B / 64][n][64]: one wavefront per channel, 16-byte loads (B is a multiple of 64)
-__global__ void __launch_bounds__(256)
-bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, int batch, float* __restrict__ bias,
-                         float* __restrict__ vb, float lr, float mom)
+__device__ __forceinline__ void bias_from_deltaT(int block, const uint16_t* __restrict__ DT, int n, int B, int batch,
+                                                 float* __restrict__ bias, float* __restrict__ vb, float lr, float mom)
 {
     const int lane = threadIdx.x & 63;
-    const int o = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int o = block * 4 + (threadIdx.x >> 6);
     if (o >= n) return;
     // eight 16-byte pieces per plane of 64 batch rows; plane p of channel o starts at (p * n + o) * 64
     auto piece = [&](int k) { return *reinterpret_cast<const uint4*>(DT + ((long long)(k >> 3) * n + o) * 64 + (k & 7) * 8); };
@@ -276,11 +275,9 @@ bias_update_bf16T_kernel(const uint16_t* __restrict__ DT, int n, int B, int batc
 }
 
 // bias update from per-tile-row partial column sums [tiles][n]: a thread per channel adds them in order
-__global__ void __launch_bounds__(64)
-bias_update_partials_kernel(const float* __restrict__ part, int tiles, int n, int B, float* __restrict__ bias,
-                            float* __restrict__ vb, float lr, float mom)
+__device__ __forceinline__ void bias_from_partials(int o, const float* __restrict__ part, int tiles, int n, int B,
+                                                   float* __restrict__ bias, float* __restrict__ vb, float lr, float mom)
 {
-    const int o = blockIdx.x * 64 + threadIdx.x;
     if (o >= n) return;
     float s = 0.0f;
     int k = 0;
@@ -295,6 +292,17 @@ bias_update_partials_kernel(const float* __restrict__ part, int tiles, int n, in
     const float d = lr * g + mom * vb[o];
     vb[o] = d;
     bias[o] = bias[o] - d;
+}
+
+// every layer's bias update of a step: a workgroup finds its layer by its index in the grid
+__global__ void __launch_bounds__(256) bias_update_step_kernel(BiasStepArgs a)
+{
+    int k = 0;
+    while (k + 1 < a.count && (int)blockIdx.x >= a.e[k + 1].first_block) ++k;
+    const BiasStepArgs::Entry& e = a.e[k];
+    const int block = blockIdx.x - e.first_block;
+    if (e.part) bias_from_partials(block * 256 + threadIdx.x, e.part, e.tiles, e.n, e.batch, e.bias, e.vb, e.lr, e.mom);
+    else bias_from_deltaT(block, e.DT, e.n, e.rows, e.batch, e.bias, e.vb, e.lr, e.mom);
 }
 
 template <typename T>
@@ -528,17 +536,18 @@ hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
     return hipGetLastError();
 }
 
-hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, int batch, float* bias, float* vb, float lr,
-                                  float mom, hipStream_t s)
-{
-    hipLaunchKernelGGL(bias_update_bf16T_kernel, dim3((n + 3) / 4), dim3(256), 0, s, DT, n, B, batch, bias, vb, lr, mom);
-    return hipGetLastError();
-}
 
-hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B, float* bias, float* vb, float lr,
-                                     float mom, hipStream_t s)
+
+hipError_t ghip_bias_update_step(BiasStepArgs& a, hipStream_t s)
 {
-    hipLaunchKernelGGL(bias_update_partials_kernel, dim3((n + 63) / 64), dim3(64), 0, s, part, tiles, n, B, bias, vb, lr, mom);
+    int blocks = 0;
+    for (int k = 0; k < a.count; ++k) {
+        a.e[k].first_block = blocks;
+        blocks += a.e[k].part ? (a.e[k].n + 255) / 256 : (a.e[k].n + 3) / 4;
+    }
+    a.blocks = blocks;
+    if (blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(bias_update_step_kernel, dim3(blocks), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 

@@ -381,13 +381,21 @@ hipError_t ghip_f32_to_bf16_2d(const float* src, uint16_t* dst, uint16_t* dstT, 
 // outside the source is zero (the padded copy of a table)
 hipError_t ghip_f32_to_bf16_2d_pad(const float* src, int src_rows, int src_cols, uint16_t* dst, uint16_t* dstT, int rows, int cols, hipStream_t s);
 hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, int cols, hipStream_t s);
-// bias update from bf16 delta^T, K-blocked [B / 64][n][64]: gb[o] = sum_b
-// (B rows of deltas, of which the first batch are the batch's; the rest are padding and zero)
-hipError_t ghip_bias_update_bf16T(const uint16_t* DT, int n, int B, int batch, float* bias, float* vbias, float lr,
-                                  float mom, hipStream_t s);
-// the same from per-tile-row partial column sums [tiles][n] (written by the LP_DGRAD epilogue)
-hipError_t ghip_bias_update_partials(const float* part, int tiles, int n, int B, float* bias, float* vbias, float lr,
-                                     float mom, hipStream_t s);
+// All bias updates of a bf16 step in one launch (a launch of its own per layer, between the products, costs the
+// step its few microseconds plus the gap each time): per layer either the partial column sums the
+// back-propagation product left ([tiles][n], a thread per channel adds them in order) or, for the output layer, the
+// transposed deltas, K-blocked [rows / 64][n][64] (a wavefront per channel; rows past the batch are zero).
+struct BiasStepArgs {
+    struct Entry {
+        const float* part; int tiles;      // partial sums [tiles][n], or NULL
+        const uint16_t* DT; int rows;      // else delta^T, K-blocked, of `rows` batch rows (a multiple of 64)
+        int n, batch;                      // channels; the divisor of the mean
+        float* bias; float* vb; float lr, mom;
+        int first_block;                   // this entry's first workgroup in the grid
+    } e[GHIP_MAX_LAYERS];
+    int count, blocks;
+};
+hipError_t ghip_bias_update_step(BiasStepArgs& a, hipStream_t s);   // fills first_block / blocks, launches
 // per-row e4m3 quantisation: src fp32/bf16 [rows][cols]; scale = amax/448 (1 if row is zero).
 // amax_bits: if non-NULL the row amax is taken from there (uint bits of a non-negative float)
 // instead of being reduced from the row; with consume_amax the entry is set back to zero once read
