@@ -21,7 +21,7 @@ The default run adds, outside the timed region and under "detail" (--no-extras l
                sustains on them, beside the published peak
   other_configs  BASELINE.json's other configurations at their default step counts, value and ms per
                step each: cfg3 (fp32 training), cfg1 and cfg2 (exact mode, one network), and cfg1 with
-               1024 networks side by side in one launch
+               1024 and 4096 networks side by side in one launch
 """
 import argparse
 import ctypes
@@ -419,7 +419,7 @@ def main():
         except Exception as e:  # noqa: BLE001
             extra["vendor_gemm"] = dict(error=repr(e))
         others = {}
-        for name, subnets in (("cfg3", 1), ("cfg1", 1), ("cfg2", 1), ("cfg1", 1024)):
+        for name, subnets in (("cfg3", 1), ("cfg1", 1), ("cfg2", 1), ("cfg1", 1024), ("cfg1", 4096)):
             key = name if subnets == 1 else f"{name}_x{subnets}"
             try:
                 wo = dict(WORKLOADS[name], name=name)
