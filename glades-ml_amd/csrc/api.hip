@@ -572,7 +572,8 @@ int step_f32(ghip_net* n, int64_t row0, int B)
 
 // ---- canonical bf16 ----
 // X: the batch's rows in bf16 at pitch ps[0], pad_batch(batch) of them readable
-int forward_bf16(ghip_net* n, const uint16_t* X, int batch)
+// for_training: also leave the transposed activations the weight gradients read (a forward-only pass skips those stores)
+int forward_bf16(ghip_net* n, const uint16_t* X, int batch, bool for_training = false)
 {
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
@@ -586,7 +587,7 @@ int forward_bf16(ghip_net* n, const uint16_t* X, int batch)
         g.fp8 = 0; g.bias = n->b[l];
         g.act = out_act(s, l, &g.act_param);
         if (l < L - 1) {
-            g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = n->HT[l + 1]; g.outT_blocked = 1;
+            g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = for_training ? n->HT[l + 1] : nullptr; g.outT_blocked = 1;
             g.n_valid = ps[l + 1] != s.sizes[l + 1] ? s.sizes[l + 1] : 0;
             LAUNCH(n, "gemm_bf16_forward", ghip_gemm_lp(g, n->stream));
         } else {
@@ -611,7 +612,7 @@ int step_bf16(ghip_net* n, int64_t row0, int batch)
     // cache line of it, a copy made now otherwise
     const bool inT = n->XbfT && (row0 % 64) == 0;
     if (!inT) LAUNCH(n, "bf16_transpose_input", ghip_bf16_transpose(X, n->HT[0], B, ps[0], n->stream));
-    TRY(forward_bf16(n, X, batch));
+    TRY(forward_bf16(n, X, batch, true));
     // rows past the batch carry zero deltas: an earlier, longer batch may have left its own there
     if (B != batch)
         LAUNCH(n, "fill_pad_delta", ghip_fill_u32((unsigned int*)(n->D[L] + (size_t)batch * ps[L]), (long long)(B - batch) * ps[L] / 2, 0u, n->stream));
