@@ -14,15 +14,22 @@
 // Tile: a workgroup of 8 wavefronts laid out 2 (M) x 4 (N); each wavefront owns MI x NI
 // accumulators of 32x32.  MI = 4, NI = 2 gives the 256 x 256 tile (128 x 64 per wavefront, 128
 // accumulator VGPRs) used whenever it fills the 256 CUs; MI = 2, NI = 1 gives a 128 x 128 tile for
-// the products that would otherwise leave most CUs idle (the 1024-wide output layer).
-// K advances in stages of 128 bytes per row (64 bf16 / 128 e4m3: whole cache lines).  LDS holds
-// two stages filled by LDS-direct global loads (global_load_lds_dwordx4: no VGPR staging, no
-// ds_write): stage s+1 is in flight while stage s is consumed.  (A ring of four 64-byte-row stages
-// with three in flight was measured too: same loop time, because every 128-byte line then travels
-// from L2 twice.)  16-byte chunks are XOR-swizzled with the row index so that the per-lane
-// 16-byte operand reads spread over all 64 banks.
-// Workgroup ids are remapped so that each XCD (ids congruent mod 8 share an L2) walks a compact
-// block of tiles.
+// the products that would otherwise leave most CUs idle (the 1024-wide output layer), MI = 4, NI = 1
+// a 256 x 128 tile for that layer's fp32-output forward product.
+// K advances in stages of 128 bytes per row (64 bf16 / 128 e4m3: whole cache lines).  The 160 KB of
+// LDS are a ring of five 32 KB operand half-stages (one operand of one stage each) filled by
+// LDS-direct global loads (global_load_lds_dwordx4 from inline assembly: no VGPR staging, no
+// ds_write, and no waits but the explicit s_waitcnt vmcnt(N) in front of the barriers).  The
+// half-stages go round the ring as X0 Y0 X1 Y1 ...: X (A, as a rule) is requested two stages ahead
+// of its use, its loads spread one by one between the MFMAs of the stage in between; Y (B) one stage
+// ahead, its loads back to back right behind the barrier that frees their slot.  The wait that
+// closes a stage leaves X's loads in flight.  (A ring of 64-byte-row stages with more of them in
+// flight was measured too: same loop time, because every 128-byte line then travels from L2 twice.)
+// Operands whose K runs over the batch (the weight gradient's, back-propagation's W^T) are read from
+// K-blocked copies, [K / 64][rows][64], where a tile's stage is one contiguous block.
+// 16-byte chunks are XOR-swizzled with the row index so that the per-lane 16-byte operand reads
+// spread over all 64 banks.  Workgroup ids are remapped so that each XCD (ids congruent mod 8 share
+// an L2) walks a compact block of tiles.
 
 #include "ghip_internal.h"
 
