@@ -141,6 +141,56 @@ def test_edge_shapes_against_oracle(sizes, N, mb):
     net.close()
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_small_networks_against_oracle(seed):
+    """Two- and three-layer networks of at most 64 nodes per layer (the shapes the single-wavefront kernel
+    serves) with activations, cost, batch size, momentum and both decays drawn at random: losses, accuracies,
+    class counts, predictions, weights, biases and delta windows of three epochs bit for bit against the CPU
+    restatement.  Widths around the power-of-two lane groups (1, 2, 3, 17, 33, 64) are in the draw."""
+    import pyglades as pg
+    rng = np.random.default_rng(1000 + seed)
+    widths = [1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 31, 33, 48, 64]
+    nl = int(rng.integers(2, 4))
+    sizes = [int(rng.choice(widths)) for _ in range(nl + 1)]
+    hidden = [po.TANH, po.SIGMOID, po.RELU, po.LEAKY, po.TANHP, po.SIGMOIDP, po.LINEAR]
+    cost = int(rng.choice([po.REGRESSION, po.CLASSIFICATION, po.KL]))
+    acts = [int(rng.choice(hidden)) for _ in range(nl - 1)] + [po.SIGMOID if cost != po.REGRESSION else int(rng.choice(hidden))]
+    params = [float(rng.choice([0.0, 0.01, 0.3, 1.0])) for _ in range(nl)]
+    N = int(rng.integers(5, 40))
+    mb = int(rng.choice([1, 2, 3, N, N + 5]))
+    kw = dict(lr=[float(rng.choice([0.01, 0.05])) for _ in range(nl)], mom=[float(rng.choice([0.0, 0.5, 0.9])) for _ in range(nl)],
+              wd1=float(rng.choice([0.0, 1e-3])), wd2=float(rng.choice([0.0, 1e-3])), act_params=params, batch=mb, cost=cost)
+    print("random net", seed, sizes, acts, cost, N, mb, flush=True)
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (0.5 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(nl)]
+    bs = [float(np.float32(rng.normal(0, 0.1))) for _ in range(nl)]
+    X = rng.random((N, sizes[0])).astype(np.float32)
+    Y = (rng.random((N, sizes[-1])) * 0.98 + 0.01).astype(np.float32)
+    o = po.ExactNet(po.make_spec(sizes, acts, **kw))
+    net = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_EXACT, **kw))
+    for l in range(nl):
+        o.set_weights(l, Ws[l]); o.set_bias(l, bs[l]); net.set_params(l, Ws[l], bs[l])
+    net.set_dataset(X, Y)
+    E = 3
+    om = [o.epoch(X, Y) for _ in range(E)]
+    ms, preds = net.run_epochs_exact(E, want_preds=True)
+    assert bits_equal([m[0] for m in ms], [m.loss for m, _ in om])
+    assert bits_equal([m[1] for m in ms], [m.accuracy for m, _ in om])
+    assert [m[2] for m in ms] == [m.correct for m, _ in om]
+    assert bits_equal(preds, om[-1][1])
+    for l in range(nl):
+        W, b = net.get_params(l)
+        assert bits_equal(W, o.get_weights(l)), l
+        assert bits_equal(np.float32(b), o.get_bias(l)), l
+        sa, sb = net.get_state(l)
+        wa, wb = o.get_window(l)
+        assert bits_equal(sa, wa) and bits_equal(sb, wb), l
+    # a test pass over the same rows leaves everything as it is and reports the same figures as the restatement's
+    mt, _ = net.run_epochs_exact(1, train=False)
+    ot, _ = o.epoch(X, Y, train=False)
+    assert bits_equal([mt[0][0]], [ot.loss]) and mt[0][2] == ot.correct
+    net.close()
+
+
 def test_network_too_large_for_lds_keeps_its_state_in_global_memory():
     """1100-40-3: three floats per edge are 529 KB, more than a compute unit's LDS, so weights and
     delta windows stay in global memory (L2) and every phase ends with a full barrier; alone and as
