@@ -49,6 +49,9 @@ __device__ __forceinline__ float bias_chain(float b, const float* bs, int no, in
     float x[NP];
 #pragma unroll
     for (int k = 0; k < NP; ++k) x[k] = (k < no && !(mo && mo[k])) ? bs[k] : 0.0f;
+    // (short rounds are unrolled so that the chain, not the loop around it, sets the pace)
+    constexpr int kRounds = NP >= 16 ? 1 : 16 / NP;
+#pragma unroll kRounds
     for (int i = 0; i < ni; ++i) {
 #pragma unroll
         for (int k = 0; k < NP; ++k) b = __fsub_rn(b, x[k]);
