@@ -182,6 +182,55 @@ def test_bf16_steps_off_the_tile_grid(B):
     g.close()
 
 
+@pytest.mark.parametrize("seed", range(5))
+def test_low_precision_random_shapes(seed):
+    """Widths from 1 to 700 and batches from 1 to 600 drawn at random, two or three layers, random hidden
+    activations: two bf16 training steps against the pipeline statement (losses 1e-4, updates 1e-2 of their
+    norm) and an e4m3 forward pass of the same shape against the restated quantised pipeline (2e-2 relative
+    RMS; codes and scales bit for bit)."""
+    import pyglades as pg
+    from helpers import bf16_pipeline_steps
+    rng = np.random.default_rng(500 + seed)
+    nl = int(rng.integers(2, 4))
+    sizes = [int(rng.integers(1, 701)) for _ in range(nl)] + [int(rng.integers(2, 300))]
+    acts = [int(rng.choice([po.TANH, po.RELU, po.SIGMOID])) for _ in range(nl - 1)] + [po.SOFTMAX]
+    B = int(rng.integers(1, 601))
+    print("random low-precision shape", seed, sizes, acts, B, flush=True)
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * np.sqrt(1.0 / sizes[l])).astype(np.float32) for l in range(nl)]
+    bs = [(rng.standard_normal(sizes[l + 1]) * 0.05).astype(np.float32) for l in range(nl)]
+    X = rng.standard_normal((2 * B, sizes[0])).astype(np.float32)
+    Y = teacher_labels(rng, X, sizes[-1])
+    lr, mom, wd2 = 0.3, 0.9, 1e-3
+    g = pg.Net(pg.make_spec(sizes, acts, lr=lr, mom=mom, wd2=wd2, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=pg.BF16))
+    for l in range(nl):
+        g.set_params(l, Ws[l], bs[l])
+    g.set_dataset(X, Y)
+    losses = [g.train_step(s_ * B, B).loss for s_ in range(2)]
+    Wm, bm, ref_losses = bf16_pipeline_steps(sizes, acts, Ws, bs, X, Y, B, 2, lr, mom, wd2)
+    np.testing.assert_allclose(losses, ref_losses, rtol=1e-4)
+    for l in range(nl):
+        Wg, bg = g.get_params(l)
+        fro = np.linalg.norm(Wg - Wm[l]) / np.linalg.norm(Wm[l] - Ws[l])
+        frob = np.linalg.norm(bg - bm[l]) / np.linalg.norm(bm[l] - bs[l])
+        assert fro <= 1e-2 and frob <= 1e-2, (l, fro, frob)
+    g.close()
+    # the same shape as an e4m3 inference network (ReLU / sigmoid hidden layers, linear output)
+    facts = [po.RELU if a == po.TANH else a for a in acts[:-1]] + [po.LINEAR]
+    q = pg.Net(pg.make_spec(sizes, facts, act_params=1.0, mode=pg.MODE_CANONICAL, dtype=pg.FP8_INFER))
+    for l in range(nl):
+        q.set_params(l, Ws[l])
+    codes, scales = q.quantize_fp8()
+    for l in range(nl):
+        c, sc = po.e4m3_quant_rows(Ws[l])
+        assert np.array_equal(codes[l], c) and np.array_equal(scales[l].view(np.uint32), sc.view(np.uint32)), l
+    Xq = po.bf16_round(X[:B])
+    out = q.forward(Xq)
+    emu = po.fp8_forward(po.make_spec(sizes, facts, act_params=1.0), codes, scales, Xq)
+    err = np.sqrt(np.mean((out - emu) ** 2)) / max(np.sqrt(np.mean(emu ** 2)), 1e-30)
+    assert err < 2e-2, err
+    q.close()
+
+
 def test_bf16_off_grid_state_round_trip():
     """Momentum of a padded network out and in again (what a checkpoint does): two copies of a network off the
     tile grid take two steps; one hands its parameters and optimiser state to the host and takes them
