@@ -479,14 +479,14 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                                     const float t1 = __fmul_rn(w1, fabsf(a));
                                     const float t2 = __fmul_rn(w2, a);
                                     for (int o = o0; o < no; o += U * rpp) {
-                                        float bv[U], lv[U], sv[U], wv[U];
+                                        float bv[U], lv[U], sv[U];   // (the weight is only read by the row that applies)
                                         int kk[U];
 #pragma unroll
                                         for (int j = 0; j < U; ++j) {
                                             const int oj = o + j * rpp;
                                             const int oc = oj < no ? oj : no - 1;  // past the end: a repeat that is not stored
                                             kk[j] = oc * ld + i;
-                                            bv[j] = bs[oc]; lv[j] = Ll[kk[j]]; sv[j] = Sl[kk[j]]; wv[j] = Wl[kk[j]];
+                                            bv[j] = bs[oc]; lv[j] = Ll[kk[j]]; sv[j] = Sl[kk[j]];
                                         }
                                         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -497,7 +497,7 @@ exact_kernel(ExactLaunch p, const ExactPointers* __restrict__ multi)
                                                 dW = __fadd_rn(dW, t2);
                                                 const float sn = __fadd_rn(sv[j], dW);
                                                 if (apply) {
-                                                    Wl[kk[j]] = __fsub_rn(wv[j], __fdiv_rn(sn, fmb));
+                                                    Wl[kk[j]] = __fsub_rn(Wl[kk[j]], __fdiv_rn(sn, fmb));
                                                     Sl[kk[j]] = 0.0f;
                                                     Ll[kk[j]] = 0.0f;
                                                 } else {
