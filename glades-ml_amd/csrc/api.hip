@@ -524,6 +524,11 @@ int step_f32(ghip_net* n, int64_t row0, int B)
     const bool narrow = n->narrowPart && ((uintptr_t)(L == 1 ? X : n->act[L - 1]) % 16) == 0;
     TRY(forward_f32(n, X, B, narrow ? L - 1 : L));
     if (!narrow) TRY(output_delta_f32(n, n->act[L], Y, n->dlt[L], nullptr, B));
+    // The weight gradients (with their updates) only need the deltas, which the back-propagation products
+    // leave layer by layer, and write what those products read (the weights): so they wait until the
+    // back-propagation below them is through and then run as one launch.
+    GemmF32Args wgrads[GHIP_GEMM_F32_GROUP_MAX];
+    int n_wgrads = 0;
     for (int l = L - 1; l >= 0; --l) {
         const int ni = s.sizes[l], no = s.sizes[l + 1];
         const float* Ain = (l == 0) ? X : n->act[l];
@@ -565,7 +570,11 @@ int step_f32(ghip_net* n, int64_t row0, int B)
         g.epilogue = EPI_SGD; g.alpha = 1.0f / (float)B;
         g.V = n->vW[l]; g.lr = s.lr[l]; g.mom = s.mom[l]; g.wd1 = s.wd1[l]; g.wd2 = s.wd2[l];
         g.bias_w = n->b[l]; g.bias_v = n->vb[l];
-        LAUNCH(n, "gemm_f32_wgrad_sgd", ghip_gemm_f32(g, n->stream));
+        wgrads[n_wgrads++] = g;
+        if (n_wgrads == GHIP_GEMM_F32_GROUP_MAX || l == 0) {
+            LAUNCH(n, "gemm_f32_wgrad_sgd", ghip_gemm_f32_group(wgrads, n_wgrads, n->stream));
+            n_wgrads = 0;
+        }
     }
     return 0;
 }

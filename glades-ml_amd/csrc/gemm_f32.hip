@@ -23,6 +23,8 @@
 // slabs (slab kt feeds the matrix cores, slab kt+1 waits, slab kt+2 is being written) and two
 // register sets holding the slabs after those on their way from memory.
 
+#include <cstring>
+
 #include "ghip_internal.h"
 
 namespace {
@@ -98,8 +100,9 @@ __device__ __forceinline__ void stage(float* dst, const Frag<UNITS>& f, int kmaj
     }
 }
 
+// one tile (bx, by) of the product g
 template <bool FAST, bool AKM, bool BKM, int BM>
-__global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
+__device__ __forceinline__ void gemm_f32_tile(const GemmF32Args& g, const int bx, const int by)
 {
     constexpr int UA = BM * BK / 4 / NTHR, UB = BN * BK / 4 / NTHR;  // float4 units per thread and slab
     constexpr int SUBS = (BM / 32) * (BN / 32);  // 32x32 accumulators of the tile
@@ -113,14 +116,14 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
     constexpr int skb = BKM ? LDT : 1, srb = BKM ? 1 : PITCH_ROWS;
     const int t = threadIdx.x;
     const int lane = t & 63, w = t >> 6;
-    const int bm = blockIdx.y * BM, bn = blockIdx.x * BN;
+    const int bm = by * BM, bn = bx * BN;
     const int sub = w % SUBS, kpart = w / SUBS;
     const int wm = (sub >> 1) * 32, wn = (sub & 1) * 32, kh = kpart * KW;
 
     v16f acc;
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
-    const bool row_sums = g.epilogue == EPI_SGD && g.bias_w && blockIdx.x == 0;
+    const bool row_sums = g.epilogue == EPI_SGD && g.bias_w && bx == 0;
     float rs = 0.0f;  // this lane's share of the sum over K of its A row (the bias gradient)
 
     const int nk = (g.K + BK - 1) / BK;
@@ -236,18 +239,96 @@ __global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
     }
 }
 
+template <bool FAST, bool AKM, bool BKM, int BM>
+__global__ void __launch_bounds__(NTHR) gemm_f32_kernel(GemmF32Args g)
+{
+    gemm_f32_tile<FAST, AKM, BKM, BM>(g, blockIdx.x, blockIdx.y);
+}
+
+// Several independent products of one kind in one launch (the weight gradients of a step): a workgroup finds
+// its product by its index in the grid.  Products of this size are mostly a launch's fixed part, which is paid
+// once here, and together their tiles fill the compute units that one of them alone leaves idle.
+template <bool FAST, bool AKM, bool BKM, int BM>
+__global__ void __launch_bounds__(NTHR) gemm_f32_group_kernel(GemmF32Group grp)
+{
+    int k = 0;
+    while (k + 1 < grp.count && (int)blockIdx.x >= grp.first[k + 1]) ++k;
+    const GemmF32Args g = grp.p[k];
+    const int local = (int)blockIdx.x - grp.first[k];
+    gemm_f32_tile<FAST, AKM, BKM, BM>(g, local % grp.gx[k], local / grp.gx[k]);
+}
+
+struct Variant { int bm; bool fast, akm, bkm; dim3 grid; };
+Variant variant_of(const GemmF32Args& a)
+{
+    Variant v;
+    // 64 x 64 tiles unless they would leave compute units without a workgroup
+    const long long tiles64 = (long long)((a.N + BN - 1) / BN) * ((a.M + 63) / 64);
+    v.bm = (tiles64 <= 128 && a.M > 32) ? 32 : 64;  // one workgroup per compute unit at a time (its LDS)
+    v.grid = dim3((a.N + BN - 1) / BN, (a.M + v.bm - 1) / v.bm);
+    const bool a_fast = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((a.a_kmajor ? a.M : a.K) % 4) == 0;
+    const bool b_fast = (a.ldb % 4) == 0 && ((uintptr_t)a.B % 16) == 0 && ((a.b_kmajor ? a.N : a.K) % 4) == 0;
+    v.fast = a_fast && b_fast;
+    v.akm = a.a_kmajor != 0;
+    v.bkm = a.b_kmajor != 0;
+    return v;
+}
+constexpr size_t kLdsBytes = sizeof(float) * 2 * NST * SLAB;  // 104 448 B: above the 64 KiB default
+
 }  // namespace
+
+hipError_t ghip_gemm_f32_group(const GemmF32Args* a, int count, hipStream_t s)
+{
+    if (count < 1 || count > GHIP_GEMM_F32_GROUP_MAX) return hipErrorInvalidValue;
+    bool alike = count > 1;
+    const Variant v0 = variant_of(a[0]);
+    for (int k = 0; k < count; ++k) {
+        if (a[k].M <= 0 || a[k].N <= 0 || a[k].K <= 0) return hipErrorInvalidValue;
+        const Variant v = variant_of(a[k]);
+        alike = alike && v.bm == v0.bm && v.fast == v0.fast && v.akm == v0.akm && v.bkm == v0.bkm;
+    }
+    if (!alike) {  // one launch each
+        for (int k = 0; k < count; ++k) {
+            hipError_t e = ghip_gemm_f32(a[k], s);
+            if (e != hipSuccess) return e;
+        }
+        return hipSuccess;
+    }
+    GemmF32Group grp;
+    memset(&grp, 0, sizeof(grp));
+    grp.count = count;
+    int blocks = 0;
+    for (int k = 0; k < count; ++k) {
+        const Variant v = variant_of(a[k]);
+        grp.p[k] = a[k];
+        grp.first[k] = blocks;
+        grp.gx[k] = (int)v.grid.x;
+        blocks += (int)(v.grid.x * v.grid.y);
+    }
+    grp.first[count] = blocks;
+    typedef void (*kernel_t)(GemmF32Group);
+#define GF32_ROW(F, BMV)                                                                                   \
+    {{gemm_f32_group_kernel<F, false, false, BMV>, gemm_f32_group_kernel<F, false, true, BMV>},            \
+     {gemm_f32_group_kernel<F, true, false, BMV>, gemm_f32_group_kernel<F, true, true, BMV>}}
+    static const kernel_t table[2][2][2][2] = {{GF32_ROW(false, 64), GF32_ROW(true, 64)}, {GF32_ROW(false, 32), GF32_ROW(true, 32)}};
+#undef GF32_ROW
+    static bool raised = false;
+    if (!raised) {
+        for (int i = 0; i < 16; ++i) {
+            hipError_t e = hipFuncSetAttribute((const void*)table[i >> 3][(i >> 2) & 1][(i >> 1) & 1][i & 1],
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+            if (e != hipSuccess) return e;
+        }
+        raised = true;
+    }
+    hipLaunchKernelGGL(table[v0.bm == 32][v0.fast][v0.akm ? 1 : 0][v0.bkm ? 1 : 0], dim3(blocks), dim3(NTHR), kLdsBytes, s, grp);
+    return hipGetLastError();
+}
 
 hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s)
 {
     if (a.M <= 0 || a.N <= 0 || a.K <= 0) return hipErrorInvalidValue;
-    // 64 x 64 tiles unless they would leave compute units without a workgroup
-    const long long tiles64 = (long long)((a.N + BN - 1) / BN) * ((a.M + 63) / 64);
-    const int bm = (tiles64 <= 128 && a.M > 32) ? 32 : 64;  // one workgroup per compute unit at a time (its LDS)
-    dim3 grid((a.N + BN - 1) / BN, (a.M + bm - 1) / bm);
-    constexpr size_t lds_bytes = sizeof(float) * 2 * NST * SLAB;  // 104 448 B: above the 64 KiB default
-    const bool a_fast = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((a.a_kmajor ? a.M : a.K) % 4) == 0;
-    const bool b_fast = (a.ldb % 4) == 0 && ((uintptr_t)a.B % 16) == 0 && ((a.b_kmajor ? a.N : a.K) % 4) == 0;
+    const Variant v = variant_of(a);
     typedef void (*kernel_t)(GemmF32Args);
 #define GF32_ROW(F, BMV)                                                                       \
     {{gemm_f32_kernel<F, false, false, BMV>, gemm_f32_kernel<F, false, true, BMV>},            \
@@ -258,11 +339,11 @@ hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s)
     if (!raised) {
         for (int i = 0; i < 16; ++i) {
             hipError_t e = hipFuncSetAttribute((const void*)table[i >> 3][(i >> 2) & 1][(i >> 1) & 1][i & 1],
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
             if (e != hipSuccess) return e;
         }
         raised = true;
     }
-    hipLaunchKernelGGL(table[bm == 32][a_fast && b_fast][a.a_kmajor ? 1 : 0][a.b_kmajor ? 1 : 0], grid, dim3(NTHR), lds_bytes, s, a);
+    hipLaunchKernelGGL(table[v.bm == 32][v.fast][v.akm ? 1 : 0][v.bkm ? 1 : 0], v.grid, dim3(NTHR), kLdsBytes, s, a);
     return hipGetLastError();
 }

@@ -280,6 +280,11 @@ struct GemmF32Args {
     float* bias_w; float* bias_v;
 };
 hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s);
+// up to GHIP_GEMM_F32_GROUP_MAX independent products in one launch where they run the same instantiation
+// (tile height, operand orientations, alignment class), else one launch each
+#define GHIP_GEMM_F32_GROUP_MAX 8
+struct GemmF32Group { GemmF32Args p[GHIP_GEMM_F32_GROUP_MAX]; int first[GHIP_GEMM_F32_GROUP_MAX + 1]; int gx[GHIP_GEMM_F32_GROUP_MAX]; int count; };
+hipError_t ghip_gemm_f32_group(const GemmF32Args* a, int count, hipStream_t s);
 
 // ---------------------------------------------------------------- narrow fp32 output layer (narrow_out.hip)
 // The products of a layer with at most 16 outputs as streams over its input activations H [B][ni]
