@@ -19,9 +19,12 @@
 // transposes: [k][row] for a K-major operand, [row][k] otherwise, both with pitch 68 (16-byte
 // stores).  A lane of the 32x32x2 instruction supplies one row and one of the two k of an MFMA; here
 // lane half lk takes k = 16*lk + i of its wavefront's half slab for MFMA i, so a [row][k] operand is
-// fetched with four 16-byte reads per slab (a [k][row] operand with sixteen 4-byte reads).  Three LDS
-// slabs (slab kt feeds the matrix cores, slab kt+1 waits, slab kt+2 is being written) and two
-// register sets holding the slabs after those on their way from memory.
+// fetched with four 16-byte reads per slab (a [k][row] operand with sixteen 4-byte reads).  Two LDS
+// slabs per operand (slab kt feeds the matrix cores while slab kt+1 is written into the buffer slab kt-1
+// has left) and two register sets holding the slabs after those on their way from memory: 68 KB of LDS,
+// so that two workgroups share a compute unit and one's first loads, reduction and epilogue run under
+// the other's K loop (with a third slab resting in LDS a workgroup had the unit to itself: the
+// weight gradients of cfg3's step took 49 us instead of 37).
 
 #include <cstring>
 
@@ -31,7 +34,7 @@ namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int BN = 64, BK = 64, LDT = 64 + 4, NST = 3, NTHR = 512;
+constexpr int BN = 64, BK = 64, LDT = 64 + 4, NST = 2, NTHR = 512;
 
 template <int UNITS>
 struct Frag { float4 v[UNITS]; unsigned char ok[UNITS]; };  // ok: bit j = component j of the unit lies inside the operand
@@ -127,33 +130,29 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmF32Args& g, const int bx
     float rs = 0.0f;  // this lane's share of the sum over K of its A row (the bias gradient)
 
     const int nk = (g.K + BK - 1) / BK;
-    // Slabs 0 and 1 go straight to LDS; from then on slab kt+2 is staged at the end of iteration kt from
+    // Slab 0 goes straight to LDS; from then on slab kt+1 is staged at the end of iteration kt from
     // registers filled one iteration earlier, so a global load has a whole iteration to arrive
     // (two register sets, alternating: the loop body is written out for even and odd kt).  More sets
     // in flight bring nothing: an iteration is bounded by its LDS traffic and barriers, not by memory.
-    Frag<UA> fa0 = fetch<FAST, UA>(g.A, g.lda, AKM, bm, 0, g.M, g.K, t);
-    Frag<UB> fb0 = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, 0, g.N, g.K, t);
-    Frag<UA> fa1 = fetch<FAST, UA>(g.A, g.lda, AKM, bm, BK, g.M, g.K, t);      // past K: zeros
-    Frag<UB> fb1 = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, BK, g.N, g.K, t);
+    Frag<UA> fa0, fa1;
+    Frag<UB> fb0, fb1;
     {
-        // slab 2 (staged at the end of iteration 0) sets out before the first two are waited for
-        const Frag<UA> a2 = fetch<FAST, UA>(g.A, g.lda, AKM, bm, 2 * BK, g.M, g.K, t);
-        const Frag<UB> b2 = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, 2 * BK, g.N, g.K, t);
-        stage(As, fa0, AKM, t);
-        stage(Bs, fb0, BKM, t);
-        stage(As + SLAB, fa1, AKM, t);
-        stage(Bs + SLAB, fb1, BKM, t);
-        fa0 = a2;
-        fb0 = b2;
+        const Frag<UA> a0 = fetch<FAST, UA>(g.A, g.lda, AKM, bm, 0, g.M, g.K, t);
+        const Frag<UB> b0 = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, 0, g.N, g.K, t);
+        // slab 1 (staged at the end of iteration 0) sets out before slab 0 is waited for
+        fa0 = fetch<FAST, UA>(g.A, g.lda, AKM, bm, BK, g.M, g.K, t);      // past K: zeros
+        fb0 = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, BK, g.N, g.K, t);
+        stage(As, a0, AKM, t);
+        stage(Bs, b0, BKM, t);
     }
     __syncthreads();
 
     const int lr = lane & 31, lk = lane >> 5;
     auto iteration = [&](int kt, Frag<UA>& sa_, Frag<UB>& sb_, Frag<UA>& na_, Frag<UB>& nb_) {
-        const int cur = kt % NST, nxt = (kt + 2) % NST;
-        // slab kt+3 sets out now, into the register set that was staged one iteration ago
-        na_ = fetch<FAST, UA>(g.A, g.lda, AKM, bm, (kt + 3) * BK, g.M, g.K, t);
-        nb_ = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, (kt + 3) * BK, g.N, g.K, t);
+        const int cur = kt % NST, nxt = (kt + 1) % NST;
+        // slab kt+2 sets out now, into the register set that was staged one iteration ago
+        na_ = fetch<FAST, UA>(g.A, g.lda, AKM, bm, (kt + 2) * BK, g.M, g.K, t);
+        nb_ = fetch<FAST, UB>(g.B, g.ldb, BKM, bn, (kt + 2) * BK, g.N, g.K, t);
         // lane half lk supplies k = kh + (KW/2)*lk + i to MFMA i (any pairing works as long as A and B
         // agree): KW/2 consecutive k per lane, which a [row][k] operand delivers as 16-byte reads
         const float* pa = As + cur * SLAB + (kh + (KW / 2) * lk) * ska + (wm + lr) * sra;
@@ -168,7 +167,7 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmF32Args& g, const int bx
 #pragma unroll
             for (int i = 0; i < KW / 2; ++i) rs += av[i];
         }
-        // slab kt+2 (requested during iteration kt-1) into the buffer slab kt-1 has left
+        // slab kt+1 (requested during iteration kt-1) into the buffer slab kt-1 has left
         stage(As + nxt * SLAB, sa_, AKM, t);
         stage(Bs + nxt * SLAB, sb_, BKM, t);
         // the wavefronts meet over LDS only (__syncthreads() would also drain the global loads just requested)
@@ -264,7 +263,7 @@ Variant variant_of(const GemmF32Args& a)
     Variant v;
     // 64 x 64 tiles unless they would leave compute units without a workgroup
     const long long tiles64 = (long long)((a.N + BN - 1) / BN) * ((a.M + 63) / 64);
-    v.bm = (tiles64 <= 128 && a.M > 32) ? 32 : 64;  // one workgroup per compute unit at a time (its LDS)
+    v.bm = (tiles64 <= 128 && a.M > 32) ? 32 : 64;  // (up to 256: the grouped weight gradients 47 us instead of 37)
     v.grid = dim3((a.N + BN - 1) / BN, (a.M + v.bm - 1) / v.bm);
     const bool a_fast = (a.lda % 4) == 0 && ((uintptr_t)a.A % 16) == 0 && ((a.a_kmajor ? a.M : a.K) % 4) == 0;
     const bool b_fast = (a.ldb % 4) == 0 && ((uintptr_t)a.B % 16) == 0 && ((a.b_kmajor ? a.N : a.K) % 4) == 0;
@@ -273,7 +272,7 @@ Variant variant_of(const GemmF32Args& a)
     v.bkm = a.b_kmajor != 0;
     return v;
 }
-constexpr size_t kLdsBytes = sizeof(float) * 2 * NST * SLAB;  // 104 448 B: above the 64 KiB default
+constexpr size_t kLdsBytes = sizeof(float) * 2 * NST * SLAB;  // 69 632 B: above the 64 KiB default, two per compute unit
 
 }  // namespace
 
