@@ -156,6 +156,7 @@ def run_canonical(w, args):
         flops = train_flops_per_sample(sizes)
     else:
         net.quantize_fp8(want=False)
+        net.set_fp8_activation_scaling(pg.FP8_ACT_PER_TOKEN if getattr(args, "fp8_act", "block32") == "per_token" else pg.FP8_ACT_BLOCK32)
         fn = lambda s: net.forward_resident((s % nb) * B, B)  # noqa: E731
         flops = infer_flops_per_sample(sizes)
     for s in range(args.warmup):
@@ -364,6 +365,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true",
                     help="cfg4: skip the untimed extras (fp32 loss check, 200-step sustained rate, cfg5 inference leg, vendor GEMM rates, the other configurations)")
+    ap.add_argument("--fp8-act", default="block32", choices=["block32", "per_token"],
+                    help="cfg5: activations re-quantised with an E8M0 scale per token and 32 units in the products' epilogues (default), or with one fp32 scale per token by a kernel of its own")
     ap.add_argument("--subnets", type=int, default=1,
                     help="exact workloads: this many networks (MetaNetwork subnets) side by side in one launch; value is their sum")
     args = ap.parse_args()

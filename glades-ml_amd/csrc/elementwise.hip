@@ -504,6 +504,27 @@ quant_rows_bf16x8_kernel(const uint16_t* __restrict__ src, int cols, uint8_t* __
     for (int c = threadIdx.x + kQuantKeep * 256; c < nchunk; c += 256) qr[c] = conv(x[c]);
 }
 
+// Block-scaled e4m3 quantisation of bf16 rows: a lane per 8 values, four lanes per 32-element block, sixteen per
+// stage dword (see ghip_quant_rows_mx)
+__global__ void __launch_bounds__(256)
+quant_rows_mx_kernel(const uint16_t* __restrict__ src, long long chunks, int chunks_per_row, uint8_t* __restrict__ q,
+                     unsigned int* __restrict__ scale, int ld_scale)
+{
+    const long long c = (long long)blockIdx.x * 256 + threadIdx.x;   // chunks_per_row is a multiple of 16: a wavefront never straddles rows' dwords
+    if (c >= chunks) return;
+    const uint4 v = reinterpret_cast<const uint4*>(src)[c];
+    unsigned int m = ghip_bf16x8_amax15(v.x, v.y, v.z, v.w);
+    unsigned int o = (unsigned int)__shfl_xor((int)m, 1, 64); m = m > o ? m : o;
+    o = (unsigned int)__shfl_xor((int)m, 2, 64); m = m > o ? m : o;
+    const int eb = ghip_mx_scale_byte(m);
+    reinterpret_cast<uint2*>(q)[c] = ghip_mx_quant8(v.x, v.y, v.z, v.w, eb);
+    unsigned int sd = (unsigned int)eb | ((unsigned int)__shfl_down(eb, 4, 64) << 8);
+    sd |= (unsigned int)__shfl_down((int)sd, 8, 64) << 16;
+    const long long row = c / chunks_per_row;
+    const int cc = (int)(c % chunks_per_row);
+    if ((threadIdx.x & 15) == 0) scale[(long long)(cc >> 4) * ld_scale + row] = sd;
+}
+
 inline int grid_for(long long n, int cap = 65535 * 4)
 {
     long long b = (n + 255) / 256;
@@ -589,6 +610,14 @@ hipError_t ghip_bf16_transpose(const uint16_t* src, uint16_t* dstT, int rows, in
         return hipGetLastError();
     }
     hipLaunchKernelGGL(convert_transpose_kernel<uint16_t>, grid, dim3(256), 0, s, src, rows, cols, (uint16_t*)nullptr, dstT, rows, cols);
+    return hipGetLastError();
+}
+
+hipError_t ghip_quant_rows_mx(const uint16_t* src, int rows, int cols, uint8_t* q, unsigned int* scale, int ld_scale, hipStream_t s)
+{
+    if (rows <= 0 || cols <= 0 || (cols % 128) || ld_scale < rows || ((uintptr_t)src % 16) || ((uintptr_t)q % 8)) return hipErrorInvalidValue;
+    const long long chunks = (long long)rows * (cols / 8);
+    hipLaunchKernelGGL(quant_rows_mx_kernel, dim3((unsigned int)((chunks + 255) / 256)), dim3(256), 0, s, src, chunks, cols / 8, q, scale, ld_scale);
     return hipGetLastError();
 }
 

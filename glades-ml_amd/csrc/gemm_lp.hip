@@ -72,6 +72,11 @@ __device__ __forceinline__ float lp_act_der(float y, const GemmLpArgs::ActForm& 
 // bf16: 16 bytes per lane per block (K = 16); e4m3: 32 bytes per lane per block (K = 64).
 template <bool FP8, int MI, int NI> struct Frags { v4i a[MI][FP8 ? 2 : 1], b[NI][FP8 ? 2 : 1]; };
 
+// e4m3: the 64 bytes of K of one MFMA are four 16-byte chunks, and the instruction takes chunks lh and 2 + lh
+// from the lane pair (row, lh = 0 / 1): its first 32-element scale block is the FIRST 16 bytes of both lanes,
+// its second block the second 16 bytes (established with a probe that doubles one lane's scale byte), and the
+// block scale of lane (row, lh) applies to block lh.  Reading the chunks in that order makes the blocks runs
+// of 32 consecutive K, as the producers of the scales define them.
 template <bool FP8, int MI, int NI>
 __device__ __forceinline__ void load_frags(Frags<FP8, MI, NI>& f, const unsigned char* sa, const unsigned char* sb,
                                            int ks, int wm, int wn, int l31, int lh)
@@ -81,12 +86,12 @@ __device__ __forceinline__ void load_frags(Frags<FP8, MI, NI>& f, const unsigned
     for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
         for (int h = 0; h < H; ++h)
-            f.a[mi][h] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, (ks * 2 + lh) * H + h));
+            f.a[mi][h] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, FP8 ? ks * 4 + h * 2 + lh : ks * 2 + lh));
 #pragma unroll
     for (int ni = 0; ni < NI; ++ni)
 #pragma unroll
         for (int h = 0; h < H; ++h)
-            f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, (ks * 2 + lh) * H + h));
+            f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, FP8 ? ks * 4 + h * 2 + lh : ks * 2 + lh));
 }
 
 typedef __attribute__((address_space(3))) unsigned char* lptr_t;
@@ -108,6 +113,14 @@ __device__ __forceinline__ void lds_direct_16s(const unsigned char* sbase, unsig
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(voff), "s"(sbase), "s"(lds_slab) : "memory", "m0");
 }
 
+// One dword per lane from a wavefront-uniform base plus a per-lane byte offset plus OFF, into a register the
+// compiler takes for written at once: like the operand loads it is waited for by the explicit counts alone.
+template <int OFF>
+__device__ __forceinline__ void load_dword_s(unsigned int& dst, const void* sbase, unsigned int voff)
+{
+    asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
+}
+
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 template <int V> struct IC { static constexpr int value = V; };
 
@@ -116,8 +129,9 @@ template <int V> struct IC { static constexpr int value = V; };
 // (i + 1) * STEP MFMAs of the span have, STEP = SPAN / (NDMA + 1).  A wavefront that issues all its
 // loads back to back stalls on the address unit (16 clocks per load, shared by the 8 wavefronts),
 // and the matrix pipe of its SIMD idles with it.
-template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, typename Dma>
-__device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma)
+// OPSEL: the byte of sa[mi] that holds this sub-step's E8M0 scale of the lane's block of A (e4m3 only; 0x7f = 1)
+template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, int OPSEL = 0, typename Dma>
+__device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma, const unsigned int (&sa)[MI])
 {
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -131,7 +145,7 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, 
                                    f.a[mi][1][0], f.a[mi][1][1], f.a[mi][1][2], f.a[mi][1][3]};
                 const v8i bv = v8i{f.b[ni][0][0], f.b[ni][0][1], f.b[ni][0][2], f.b[ni][0][3],
                                    f.b[ni][1][0], f.b[ni][1][1], f.b[ni][1][2], f.b[ni][1][3]};
-                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[mi][ni], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+                acc[mi][ni] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(av, bv, acc[mi][ni], 0, 0, OPSEL, (int)sa[mi], 0, 0x7f7f7f7f);
             }
             if constexpr (NDMA > 0) {
                 const int m = BEFORE + mi * NI + ni;
@@ -150,8 +164,19 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, 
         }
 }
 
+// LDS of one workgroup: a ring of five operand half-stages during the K loop, then the staging area of the epilogue.
+template <int MI, int NI>
+constexpr int lp_lds_bytes()
+{
+    constexpr int TM = 64 * MI, TN = 128 * NI;
+    return cmax(5 * cmax(TM, TN) * SKB, cmax(TM * (2 * TN + 16), TN * (2 * TM + 16)));
+}
+
+// One tile of one product, by the whole workgroup.  `id` numbers the product's tiles so that consecutive
+// numbers are neighbours in the output (the caller hands each XCD a contiguous range of them); smem is the
+// workgroup's LDS block of lp_lds_bytes<MI, NI>() bytes, 1 KiB aligned.
 template <bool FP8, int EPI, int MI, int NI>
-__global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
+__device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsigned char* smem)
 {
     constexpr int TM = 64 * MI, TN = 128 * NI;       // tile
     constexpr int WM = 32 * MI, WN = 32 * NI;        // per wavefront
@@ -160,19 +185,13 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     constexpr int NSLOT = 5;
     constexpr int PITCH = 2 * TN + 16;               // staged bf16 output row [TM][TN]: +16 rotates banks, keeps alignment
     constexpr int PITCH_T = 2 * TM + 16;             // staged transposed row [TN][TM]
-    constexpr int LDS_BYTES = cmax(NSLOT * SLOT, cmax(TM * PITCH, TN * PITCH_T));
-    // One LDS block: a ring of five operand stages during the K loop, then the staging area of the epilogue.
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    static_assert(lp_lds_bytes<MI, NI>() == cmax(NSLOT * SLOT, cmax(TM * PITCH, TN * PITCH_T)), "the ring and the staging area fit");
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6;
     const int l31 = lane & 31, lh = lane >> 5;
 
-    // ---- XCD-aware tile order: ids with equal (id % 8) run on one XCD; give each XCD a
-    //      contiguous range of tile numbers, and walk tiles in column groups of 8 rows
+    // ---- walk the tiles in column groups of 8 rows
     const int tiles_m = g.M / TM, tiles_n = g.N / TN;
-    const int nb = tiles_m * tiles_n;
-    int id = blockIdx.x;
-    if ((nb & 7) == 0) id = (id & 7) * (nb >> 3) + (id >> 3);
     constexpr int GROUP = 8;
     const int per_group = GROUP * tiles_n;
     const int gidx = id / per_group;
@@ -210,8 +229,33 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     // as soon as the barrier that ends stage j-1 has freed its slot, A(j+2) while stage j is consumed,
     // so A has two stages of lead and B one, and the wait that ends stage j leaves the A loads in flight.
     constexpr int PWA = TM / 64, PWB = TN / 64;
-    static_assert(PWA % 2 == 0 && PWB % 2 == 0 && PWA < 8, "slab parity and the vmcnt immediate assume this");
     const int ws = __builtin_amdgcn_readfirstlane(w);
+    static_assert(PWA % 2 == 0 && PWB % 2 == 0 && PWA < 8, "slab parity and the vmcnt immediate assume this");
+    // e4m3 with block-scaled activations: the E8M0 scales of A, one byte per row and 32 elements of K, lie
+    // stage-major, [K / 128][ld_scale] dwords (a dword = the four blocks of one row in one stage).  Each lane
+    // fetches the dwords of its MI rows straight into registers, two stages ahead together with the first X
+    // load; five register sets, one per ring position, so that no value ever moves between registers while
+    // its load may still be in flight.
+    constexpr bool kMX = FP8 && (EPI == LP_FP8_ACT_MX || EPI == LP_FP8_F32_MX);
+    unsigned int sc[NSLOT][MI];
+    const unsigned int* const scw = kMX ? g.a_scale + bm + (ws >> 2) * WM : nullptr;
+    const unsigned int scv = (unsigned int)l31 * 4u;
+    auto load_scales = [&](auto setc, int st) {
+        constexpr int S = decltype(setc)::value;
+        const unsigned int* const base = scw + (long long)(st < nk ? st : nk - 1) * g.ld_scale;
+        load_dword_s<0>(sc[S][0], base, scv);
+        if constexpr (MI > 1) load_dword_s<128>(sc[S][1], base, scv);
+        if constexpr (MI > 2) load_dword_s<256>(sc[S][2], base, scv);
+        if constexpr (MI > 3) load_dword_s<384>(sc[S][3], base, scv);
+        static_assert(MI <= 4, "one load per 32-row block");
+    };
+    if constexpr (kMX) { load_scales(IC<0>{}, 0); load_scales(IC<1>{}, 1); }
+    else {
+#pragma unroll
+        for (int i = 0; i < NSLOT; ++i)
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) sc[i][mi] = 0x7f7f7f7fu;
+    }
     const unsigned int smem_u = (unsigned int)(uintptr_t)((lptr_t)smem);
     unsigned int voffA[2], voffB[2];
 #pragma unroll
@@ -292,7 +336,8 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         const unsigned char* src = base + ((long long)(bm + within / PF_LPR) * g.N + bn) * PF_ES + (within % PF_LPR) * 128;
         if (lane < PF_LANES) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
     };
-    constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0);  // loads a stage's closing wait leaves in flight
+    constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0) + (kMX ? MI : 0);  // loads a stage's closing wait leaves in flight
+    static_assert(VM_STAGE <= 15, "the count fits the low four bits of the wait's immediate");
     // The Y half-stage, asked for one stage before the wait for it, is the load that arrives late, and
     // most of all where the operands come from HBM rather than the memory-side cache (the weight
     // gradient's are a forward pass old).  So its loads go out as early as their slot allows, back to
@@ -307,9 +352,15 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         const unsigned char* const NB = smem + ((2 * P + 2 + OB) % NSLOT) * SLOT;
         auto dma = [&](int d) {
             if (kTouch && d == 0) touch(j);
+            if constexpr (kMX) { if (d == 0) load_scales(IC<(P + 2) % NSLOT>{}, j + 2); }
             dmaX((2 * P + 4) % NSLOT, j + 2, d);
         };
         auto none = [](int) {};
+        // this stage's scale dwords landed before the wait that closed the stage before; lane (row, lh) scales
+        // blocks lh (first sub-step) and 2 + lh (second): bytes 0 and 2 once the dword is shifted by 8 lh bits
+        unsigned int sa[MI];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) sa[mi] = kMX ? sc[P][mi] >> (8 * lh) : 0x7f7f7f7fu;
         auto next_y = [&]() {  // the next stage's Y loads: their slot is free once this stage's closing barrier is passed
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -318,9 +369,9 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         };
         if constexpr (!kDouble) {
             constexpr int SPAN = 2 * G;
-            mma_group<FP8, MI, NI, SPAN, PWA, 0>(acc, f0, dma);
+            mma_group<FP8, MI, NI, SPAN, PWA, 0, 0>(acc, f0, dma, sa);
             load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
-            mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, f0, dma);
+            mma_group<FP8, MI, NI, SPAN, PWA, G, 2>(acc, f0, dma, sa);
             __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
             next_y();
@@ -341,10 +392,10 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                     load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (ks == 0) mma_group<FP8, MI, NI, SPAN, PWA, 0>(acc, cur, dma);
-                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, cur, dma);
-                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, PWA, 2 * G>(acc, cur, dma);
-                else mma_group<FP8, MI, NI, 1, 0, 0>(acc, cur, none);
+                if (ks == 0) mma_group<FP8, MI, NI, SPAN, PWA, 0, 0>(acc, cur, dma, sa);
+                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, cur, dma, sa);
+                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, PWA, 2 * G>(acc, cur, dma, sa);
+                else mma_group<FP8, MI, NI, 1, 0, 0, FP8 ? 2 : 0>(acc, cur, none, sa);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -400,8 +451,9 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         __builtin_amdgcn_s_barrier();
     }
 
-    constexpr bool kBf16Out = (EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT);
-    constexpr bool kFwd = (EPI == LP_FWD_ACT || EPI == LP_FWD_F32), kF8 = (EPI == LP_FP8_ACT || EPI == LP_FP8_F32);
+    constexpr bool kActMX = (EPI == LP_FP8_ACT_MX);   // e4m3 codes + block scales out, through the same bf16 staging
+    constexpr bool kBf16Out = (EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT || kActMX);
+    constexpr bool kFwd = (EPI == LP_FWD_ACT || EPI == LP_FWD_F32), kF8 = (EPI == LP_FP8_ACT || EPI == LP_FP8_F32 || kMX);
     uint2 pk[MI][NI][4];  // bf16 results, 4 consecutive rows packed per entry
     float cbias[NI], cscale[NI];
 #pragma unroll
@@ -421,7 +473,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             for (int q = 0; q < 4; ++q) {
                 const int row0 = bm + wm + mi * 32 + 8 * q + 4 * lh;
                 float rs[4] = {1.0f, 1.0f, 1.0f, 1.0f};
-                if constexpr (kF8) {
+                if constexpr (kF8 && !kMX) {
                     const float4 r4 = *reinterpret_cast<const float4*>(g.row_scale + row0);
                     rs[0] = r4.x; rs[1] = r4.y; rs[2] = r4.z; rs[3] = r4.w;
                 }
@@ -435,6 +487,8 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                         const float v = acc[mi][ni][q * 4 + r];
                         if constexpr (kFwd) {
                             o[r] = lp_squash<PLAIN>(v + cbias[ni], g.ap);
+                        } else if constexpr (kMX) {
+                            o[r] = lp_squash<PLAIN>(__fmul_rn(v, cscale[ni]), g.ap);   // the rows' scales went in block by block
                         } else if constexpr (kF8) {
                             o[r] = lp_squash<PLAIN>(__fmul_rn(v, __fmul_rn(rs[r], cscale[ni])), g.ap);
                         } else if constexpr (EPI == LP_WGRAD_SGD) {
@@ -448,13 +502,13 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
                         } else {
                             o[r] = v;
                         }
-                        if constexpr (EPI == LP_FWD_F32 || EPI == LP_FP8_F32) ((float*)g.out)[idx] = o[r];
+                        if constexpr (EPI == LP_FWD_F32 || EPI == LP_FP8_F32 || EPI == LP_FP8_F32_MX) ((float*)g.out)[idx] = o[r];
                     }
-                    if constexpr (EPI == LP_FWD_ACT || EPI == LP_FP8_ACT) {
+                    if constexpr (EPI == LP_FWD_ACT || EPI == LP_FP8_ACT || kActMX) {
                         // units past the layer's width are padding: they stay zero whatever the activation makes of 0
                         if (pad_tile && col >= g.n_valid) { o[0] = 0.0f; o[1] = 0.0f; o[2] = 0.0f; o[3] = 0.0f; }
                     }
-                    if constexpr (EPI == LP_FP8_ACT) {
+                    if constexpr (EPI == LP_FP8_ACT || kActMX) {
                         // single output: straight into the row-major staging area
                         const unsigned int p01 = ghip_f32x2_to_bf16x2(o[0], o[1]), p23 = ghip_f32x2_to_bf16x2(o[2], o[3]);
                         unsigned char* d0 = smem + (wm + mi * 32 + 8 * q + 4 * lh) * PITCH + (wn + ni * 32 + l31) * 2;
@@ -523,7 +577,7 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             __builtin_amdgcn_s_barrier();
         }
         // row-major copy: LDS[m][n]
-        if constexpr (EPI != LP_FP8_ACT)
+        if constexpr (EPI != LP_FP8_ACT && !kActMX)
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -540,6 +594,30 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
         __builtin_amdgcn_s_waitcnt(0xC07F);
         __builtin_amdgcn_s_barrier();
         constexpr int LPR = TN / 8, RPI = 64 / LPR, NIT = (TM / 8) / RPI;
+        if constexpr (kActMX) {
+            // The next layer's A operand, made here: every run of 32 outputs of a row (four lanes' 8 values) gets its
+            // power-of-two scale (ghip_mx_scale_byte) and is stored as e4m3 codes of the bf16-rounded values over
+            // that scale; the scale's E8M0 byte goes where the consuming product's lanes fetch it (a_scale's layout)
+            unsigned char* dq = (unsigned char*)g.out + (long long)bm * N + bn;
+#pragma unroll
+            for (int i = 0; i < NIT; ++i) {
+                const int ml = w * (TM / 8) + i * RPI + lane / LPR;
+                const int lc = lane % LPR;
+                const v4i val = *reinterpret_cast<const v4i*>(smem + ml * PITCH + (lc << 4));
+                const unsigned int u0 = (unsigned int)val[0], u1 = (unsigned int)val[1], u2 = (unsigned int)val[2], u3 = (unsigned int)val[3];
+                unsigned int m = ghip_bf16x8_amax15(u0, u1, u2, u3);
+                unsigned int o1 = (unsigned int)__shfl_xor((int)m, 1, 64); m = m > o1 ? m : o1;
+                o1 = (unsigned int)__shfl_xor((int)m, 2, 64); m = m > o1 ? m : o1;
+                const int eb = ghip_mx_scale_byte(m);
+                *reinterpret_cast<uint2*>(dq + (long long)ml * N + (lc << 3)) = ghip_mx_quant8(u0, u1, u2, u3, eb);
+                // the four blocks of a 128-wide run of outputs = the next product's stage: bytes of lanes 0, 4, 8, 12 of
+                // every 16 make one dword
+                unsigned int sd = (unsigned int)eb | ((unsigned int)__shfl_down(eb, 4, 64) << 8);
+                sd |= (unsigned int)__shfl_down((int)sd, 8, 64) << 16;
+                if ((lane & 15) == 0) g.out_scale[(long long)((bn >> 7) + (lc >> 4)) * g.ld_out_scale + bm + ml] = sd;
+            }
+            return;
+        }
         unsigned char* dst = (unsigned char*)g.out + ((long long)bm * N + bn) * 2;
         unsigned int am[NIT];
 #pragma unroll
@@ -589,6 +667,20 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
             if (t < TN) g.colsum[(long long)tm * N + bn + t] = red[t] + red[TN + t];
         }
     }
+}
+
+// XCD-aware tile order of a launch over one product: workgroups whose ids are congruent mod 8 run on one
+// XCD (and share its L2); each XCD gets a contiguous range of tile numbers.
+__device__ __forceinline__ int xcd_tile_id(int block, int nb)
+{
+    return (nb & 7) == 0 ? (block & 7) * (nb >> 3) + (block >> 3) : block;
+}
+
+template <bool FP8, int EPI, int MI, int NI>
+__global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[lp_lds_bytes<MI, NI>()];
+    gemm_lp_tile<FP8, EPI, MI, NI>(g, xcd_tile_id(blockIdx.x, (g.M / (64 * MI)) * (g.N / (128 * NI))), smem);
 }
 
 // 256 x 256 tiles when they give every CU at least one workgroup, else 128 x 128.
@@ -650,17 +742,22 @@ bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8)
     return M > 0 && N > 0 && K > 0 && (M % 256) == 0 && (N % 256) == 0 && (K % kq) == 0;
 }
 
-hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
+// what the kernels assume of a product's shapes, pitches and addresses
+static bool operands_ok(const GemmLpArgs& a_)
 {
-    if (!ghip_gemm_lp_shape_ok(a_.M, a_.N, a_.K, a_.fp8)) return hipErrorInvalidValue;
+    if (!ghip_gemm_lp_shape_ok(a_.M, a_.N, a_.K, a_.fp8)) return false;
     // the LDS-direct loads move 16 bytes per lane: operand rows start on 16-byte boundaries, pitches cover K
     const int es = a_.fp8 ? 1 : 2;
     // (a K-blocked operand's pitch is one stage's 128 bytes and its stages lie kstride bytes apart)
     const bool pitchA_ok = a_.kstrideA ? ((long long)a_.lda * es == 128 && a_.kstrideA % 128 == 0) : (!a_.lda || a_.lda >= a_.K);
     const bool pitchB_ok = a_.kstrideB ? ((long long)a_.ldb * es == 128 && a_.kstrideB % 128 == 0) : (!a_.ldb || a_.ldb >= a_.K);
-    if (!pitchA_ok || !pitchB_ok || (a_.lda && ((long long)a_.lda * es) % 16) || (a_.ldb && ((long long)a_.ldb * es) % 16) ||
-        (((uintptr_t)a_.A | (uintptr_t)a_.B) % 16))
-        return hipErrorInvalidValue;
+    return pitchA_ok && pitchB_ok && !(a_.lda && ((long long)a_.lda * es) % 16) && !(a_.ldb && ((long long)a_.ldb * es) % 16) &&
+           (((uintptr_t)a_.A | (uintptr_t)a_.B) % 16) == 0;
+}
+
+hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
+{
+    if (!operands_ok(a_)) return hipErrorInvalidValue;
     GemmLpArgs a = a_;
     resolve_act(a);
     if (!a.fp8) {
@@ -671,9 +768,15 @@ hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
         case LP_WGRAD_SGD: return launch<false, LP_WGRAD_SGD>(a, s);
         }
     } else {
+        const bool mx = a.epilogue == LP_FP8_ACT_MX || a.epilogue == LP_FP8_F32_MX;
+        // block-scaled activations: a dword of scales per row and stage, at least M rows to a stage
+        if (mx && (!a.a_scale || a.ld_scale < a.M || ((uintptr_t)a.a_scale % 4))) return hipErrorInvalidValue;
+        if (a.epilogue == LP_FP8_ACT_MX && (!a.out_scale || a.ld_out_scale < a.M || ((uintptr_t)a.out % 8))) return hipErrorInvalidValue;
         switch (a.epilogue) {
         case LP_FP8_ACT: return launch<true, LP_FP8_ACT>(a, s);
         case LP_FP8_F32: return launch<true, LP_FP8_F32>(a, s);
+        case LP_FP8_ACT_MX: return launch<true, LP_FP8_ACT_MX>(a, s);
+        case LP_FP8_F32_MX: return launch<true, LP_FP8_F32_MX>(a, s);
         }
     }
     return hipErrorInvalidValue;

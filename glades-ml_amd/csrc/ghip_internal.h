@@ -200,6 +200,43 @@ __device__ __forceinline__ uint8_t ghip_f32_to_e4m3(float x)
     return (uint8_t)(sign | code);
 }
 
+// Block-scaled e4m3 ("MX": an E8M0 power-of-two scale per 32 consecutive elements of a row).  The scale of a
+// block is the power of two that brings its largest magnitude into (224, 448], the top binade of e4m3, so
+// nothing saturates and the largest element keeps all three mantissa bits: with that magnitude
+// 2^(E-127) (1 + M/128) in bf16 (bits amax15 = E << 7 | M) the E8M0 byte is E - 8, one more if 1 + M/128 > 1.75
+// (256 (1 + M/128) would pass 448), never below 0 (magnitudes under 2^-119 then land under 256).
+__device__ __forceinline__ int ghip_mx_scale_byte(unsigned int amax15)
+{
+    const int eb = (int)(amax15 >> 7) - 8 + ((amax15 & 0x7fu) > 96u ? 1 : 0);
+    return eb < 0 ? 0 : eb;
+}
+// codes of 8 bf16 values (two per dword) over the scale 2^(eb - 127): the hardware's round-to-nearest-even conversion
+__device__ __forceinline__ uint2 ghip_mx_quant8(unsigned int u0, unsigned int u1, unsigned int u2, unsigned int u3, int eb)
+{
+    const float inv = __uint_as_float((unsigned int)(254 - eb) << 23);   // 2^(127 - eb), exact
+    uint2 q;
+    int p = __builtin_amdgcn_cvt_pk_fp8_f32(__uint_as_float(u0 << 16) * inv, __uint_as_float(u0 & 0xffff0000u) * inv, 0, false);
+    p = __builtin_amdgcn_cvt_pk_fp8_f32(__uint_as_float(u1 << 16) * inv, __uint_as_float(u1 & 0xffff0000u) * inv, p, true);
+    q.x = (unsigned int)p;
+    p = __builtin_amdgcn_cvt_pk_fp8_f32(__uint_as_float(u2 << 16) * inv, __uint_as_float(u2 & 0xffff0000u) * inv, 0, false);
+    p = __builtin_amdgcn_cvt_pk_fp8_f32(__uint_as_float(u3 << 16) * inv, __uint_as_float(u3 & 0xffff0000u) * inv, p, true);
+    q.y = (unsigned int)p;
+    return q;
+}
+// largest 15-bit magnitude among 8 bf16 values (bf16 magnitudes order like their bit patterns)
+__device__ __forceinline__ unsigned int ghip_bf16x8_amax15(unsigned int u0, unsigned int u1, unsigned int u2, unsigned int u3)
+{
+    unsigned int m = 0;
+    const unsigned int w[4] = {u0, u1, u2, u3};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const unsigned int lo = w[d] & 0x7fffu, hi = (w[d] >> 16) & 0x7fffu;
+        m = m > lo ? m : lo;
+        m = m > hi ? m : hi;
+    }
+    return m;
+}
+
 // ---------------------------------------------------------------- exact mode (exact_kernel.hip)
 
 // What differs between the networks of one launch: parameters, state and results.
@@ -339,7 +376,12 @@ enum LpEpilogue {
     LP_WGRAD_SGD = 3,   // acc = batch-summed gradient tile [M=n_out][N=n_in]: fused update of
                         // fp32 master + momentum, writes bf16 W [M][N] and W^T [N][M]
     LP_FP8_ACT = 4,     // fp8 inference: v = squash(acc * rs[m] * cs[n]); bf16 out + row amax
-    LP_FP8_F32 = 5      // fp8 inference last layer: fp32 out = squash(acc * rs[m] * cs[n])
+    LP_FP8_F32 = 5,     // fp8 inference last layer: fp32 out = squash(acc * rs[m] * cs[n])
+    // The same two with block-scaled activations (the MX form CDNA4's scaled MFMA takes): A comes with an E8M0
+    // scale per row and 32 elements of K (a_scale) instead of one fp32 scale per row, and LP_FP8_ACT_MX leaves
+    // its result as the next layer's A operand, e4m3 codes [M][N] + scales (out_scale), quantised in the epilogue.
+    LP_FP8_ACT_MX = 6,  // v = squash(acc * cs[n]) -> bf16 rounding -> codes + block scales
+    LP_FP8_F32_MX = 7   // fp32 out = squash(acc * cs[n])
 };
 struct GemmLpArgs {
     const void* A; const void* B;    // [M][K], [N][K], K contiguous; bf16 or e4m3
@@ -373,6 +415,10 @@ struct GemmLpArgs {
     float* master; float* mom; float lr, momf, wd1, wd2, gscale;
     // fp8
     const float* row_scale; const float* col_scale; unsigned int* row_amax_bits;
+    // block-scaled e4m3 activations: E8M0 bytes, stage-major: dword [k / 128][row] holds the scales of the four
+    // 32-element blocks k..k+127 of that row; ld = dwords from one stage's rows to the next's (>= rows)
+    const unsigned int* a_scale; int ld_scale;
+    unsigned int* out_scale; int ld_out_scale;
 };
 hipError_t ghip_gemm_lp(const GemmLpArgs& a, hipStream_t s);
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8);
@@ -408,3 +454,6 @@ hipError_t ghip_bias_update_step(BiasStepArgs& a, hipStream_t s);   // fills fir
 hipError_t ghip_quant_rows_e4m3(const void* src, int src_is_bf16, int rows, int cols, uint8_t* q,
                                 float* scale, unsigned int* amax_bits, int consume_amax, hipStream_t s);
 hipError_t ghip_fill_u32(unsigned int* p, long long n, unsigned int v, hipStream_t s);
+// Block-scaled e4m3 quantisation of bf16 rows (cols a multiple of 128, rows 16-byte aligned): codes [rows][cols]
+// and the E8M0 scales stage-major, dword [c / 128][row] = the four blocks c..c+127 of that row (GemmLpArgs::a_scale)
+hipError_t ghip_quant_rows_mx(const uint16_t* src, int rows, int cols, uint8_t* q, unsigned int* scale, int ld_scale, hipStream_t s);

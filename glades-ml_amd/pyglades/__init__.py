@@ -17,6 +17,7 @@ REGRESSION, CLASSIFICATION, KL = range(3)
 MODE_EXACT, MODE_CANONICAL = 0, 1
 F32, BF16, FP8_INFER = 0, 1, 2
 BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
+FP8_ACT_PER_TOKEN, FP8_ACT_BLOCK32 = 0, 1
 
 EXPORTS = [
     "ghip_init", "ghip_gmath_eval", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
@@ -25,7 +26,7 @@ EXPORTS = [
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
     "ghip_net_run_epoch_canonical", "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_forward_noalloc", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
-    "ghip_net_quantize_fp8", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
+    "ghip_net_quantize_fp8", "ghip_net_set_fp8_activation_scaling", "ghip_quantize_rows_e4m3_block32", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
     "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
 ]
 
@@ -104,6 +105,8 @@ def load():
             "ghip_net_confusion_get": (i, [vp, vp, i64]),
             "ghip_net_class_metrics": (i, [vp, i, C.POINTER(ClassMetrics)]),
             "ghip_net_quantize_fp8": (i, [vp, vp, vp]),
+            "ghip_net_set_fp8_activation_scaling": (i, [vp, i]),
+            "ghip_quantize_rows_e4m3_block32": (i, [vp, i64, i, vp, vp]),
             "ghip_net_sync": (i, [vp]),
             "ghip_net_profile": (i, [vp, i]),
             "ghip_net_profile_count": (i, [vp]),
@@ -148,6 +151,15 @@ def make_spec(sizes, acts, lr=0.01, mom=0.0, wd1=0.0, wd2=0.0, act_params=0.0, b
 
 def _ptr(a):
     return None if a is None else C.c_void_p(a.ctypes.data)
+
+
+def quantize_rows_e4m3_block32(x):
+    """The block-scaled e4m3 quantiser on its own: (codes [rows][cols], E8M0 bytes [rows][ceil(cols / 32)])."""
+    x = np.ascontiguousarray(x, np.float32)
+    codes = np.empty(x.shape, np.uint8)
+    scales = np.empty((x.shape[0], (x.shape[1] + 31) // 32), np.uint8)
+    _check(load().ghip_quantize_rows_e4m3_block32(_ptr(x), x.shape[0], x.shape[1], _ptr(codes), _ptr(scales)))
+    return codes, scales
 
 
 def gmath_eval(fn, kind, a, b=None, param=0.0):
@@ -324,6 +336,9 @@ class Net:
         cp = (C.c_void_p * self.nl)(*[c.ctypes.data for c in codes])
         _check(self.lib.ghip_net_quantize_fp8(self.h, C.cast(sp, C.c_void_p), C.cast(cp, C.c_void_p)))
         return codes, scales
+
+    def set_fp8_activation_scaling(self, mode):
+        _check(self.lib.ghip_net_set_fp8_activation_scaling(self.h, mode))
 
     def sync(self):
         _check(self.lib.ghip_net_sync(self.h))

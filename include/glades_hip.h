@@ -259,6 +259,23 @@ int ghip_net_class_metrics(ghip_net* net, int epoch, ghip_class_metrics* host_ou
  * reference is fp32 only); checked against its fp32 forward on the dequantised weights. */
 int ghip_net_quantize_fp8(ghip_net* net, float* const* host_scales, uint8_t* const* host_codes);
 
+/* GHIP_FP8_INFER: how the activations are re-quantised to e4m3 between layers.  No reference counterpart.
+ *   GHIP_FP8_ACT_BLOCK32 (default): every token (row) gets a power-of-two (E8M0) scale per 32 consecutive
+ *     units, the block format gfx950's scaled MFMA takes as it is; the producing product's epilogue writes
+ *     the codes and scales, so nothing runs between two layers' products.  Scale of a block = the power of
+ *     two that brings its largest magnitude into (224, 448].
+ *   GHIP_FP8_ACT_PER_TOKEN: one fp32 scale per token (row amax / 448) for the whole row; the product writes
+ *     bf16 activations and row maxima, a second kernel re-quantises the rows.
+ * Both quantise the bf16-rounded activations. */
+#define GHIP_FP8_ACT_PER_TOKEN 0
+#define GHIP_FP8_ACT_BLOCK32   1
+int ghip_net_set_fp8_activation_scaling(ghip_net* net, int mode);
+
+/* The GHIP_FP8_ACT_BLOCK32 quantiser on its own (what the products' epilogues apply between layers): host_x
+ * [rows][cols] fp32 is rounded to bf16 and quantised on the device; host_codes [rows][cols] receives the
+ * e4m3 codes, host_scales [rows][ceil(cols / 32)] the E8M0 bytes (value 2^(byte - 127)). */
+int ghip_quantize_rows_e4m3_block32(const float* host_x, int64_t rows, int cols, uint8_t* host_codes, uint8_t* host_scales);
+
 /* Blocks until everything queued on the handle's stream has finished. */
 int ghip_net_sync(ghip_net* net);
 

@@ -825,6 +825,71 @@ void go_e4m3_quant_rows(const float* x, int64_t rows, int64_t cols, uint8_t* q, 
     }
 }
 
+/* Block-scaled e4m3 ("MX"): one E8M0 power-of-two scale per row and 32 consecutive columns.  No reference
+ * counterpart (the reference is fp32); the rule is this build's: the scale is the power of two that brings
+ * the block's largest magnitude amax into (224, 448] -- byte = E - 8 for amax = 2^(E-127) m, m in [1, 2), one more
+ * if 256 m would pass 448 (m > 1.75), never below 0 -- and the codes are e4m3(x / scale), round to nearest even.
+ * scale bytes: [rows][ceil(cols / 32)]. */
+void go_e4m3_quant_rows_block32(const float* x, int64_t rows, int64_t cols, uint8_t* q, uint8_t* scale)
+{
+    const int64_t nblk = (cols + 31) / 32;
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+    for (int64_t r = 0; r < rows; ++r)
+        for (int64_t b = 0; b < nblk; ++b) {
+            const int64_t c0 = b * 32, c1 = c0 + 32 < cols ? c0 + 32 : cols;
+            float amax = 0.0f;
+            for (int64_t c = c0; c < c1; ++c) { float a = fabsf(x[r * cols + c]); if (a > amax) amax = a; }
+            const uint32_t u = f2u(amax);
+            int eb = (int)(u >> 23) - 8 + ((u & 0x7fffffu) > 0x600000u ? 1 : 0); /* mantissa field above .75 */
+            if (eb < 0) eb = 0;
+            scale[r * nblk + b] = (uint8_t)eb;
+            const float sc = ldexpf(1.0f, eb - 127);
+            for (int64_t c = c0; c < c1; ++c) q[r * cols + c] = go_e4m3_from_f32(x[r * cols + c] / sc);
+        }
+}
+
+/* go_fp8_forward with block-scaled activations: between layers the bf16-rounded activations are quantised by
+ * go_e4m3_quant_rows_block32; a product is sum over blocks of 2^(byte-127) * (sum over the block of code values
+ * times weight code values), times the output channel's weight scale. */
+void go_fp8_forward_block32(const go_spec* s, const uint8_t* const* Wq, const float* const* wscale,
+                            const float* X, int64_t B, float* out)
+{
+    static float lut[256];
+    for (int i = 0; i < 256; ++i) lut[i] = go_e4m3_to_f32((uint8_t)i);
+    int maxw = 0;
+    for (int l = 0; l <= s->n_layers; ++l) if (s->sizes[l] > maxw) maxw = s->sizes[l];
+    float* cur = (float*)malloc(sizeof(float) * B * maxw);
+    float* nxt = (float*)malloc(sizeof(float) * B * maxw);
+    uint8_t* q = (uint8_t*)malloc((size_t)B * maxw);
+    uint8_t* xs = (uint8_t*)malloc((size_t)B * ((maxw + 31) / 32));
+    memcpy(cur, X, sizeof(float) * B * s->sizes[0]);
+    for (int l = 0; l < s->n_layers; ++l) {
+        const int ni = s->sizes[l], no = s->sizes[l + 1], nblk = (ni + 31) / 32;
+        go_e4m3_quant_rows_block32(cur, B, ni, q, xs);
+        float* wf = (float*)malloc(sizeof(float) * (size_t)ni * no);
+        for (size_t k = 0; k < (size_t)ni * no; ++k) wf[k] = lut[Wq[l][k]];
+#pragma omp parallel for num_threads(g_threads) schedule(static)
+        for (int64_t b = 0; b < B; ++b) {
+            float* xf = (float*)malloc(sizeof(float) * ni);
+            for (int i = 0; i < ni; ++i) xf[i] = lut[q[b * ni + i]] * ldexpf(1.0f, (int)xs[b * nblk + i / 32] - 127);
+            for (int o = 0; o < no; ++o) {
+                const float* w = wf + (size_t)o * ni;
+                float acc = 0.0f;
+                for (int i = 0; i < ni; ++i) { float pr = w[i] * xf[i]; acc += pr; }
+                float v = acc * wscale[l][o];
+                v = go_squash(v, s->act[l], s->act_param[l]);
+                if (l + 1 < s->n_layers) v = go_bf16_to_f32(go_bf16_from_f32(v));
+                nxt[b * no + o] = v;
+            }
+            free(xf);
+        }
+        free(wf);
+        float* t = cur; cur = nxt; nxt = t;
+    }
+    memcpy(out, cur, sizeof(float) * B * s->sizes[s->n_layers]);
+    free(cur); free(nxt); free(q); free(xs);
+}
+
 void go_fp8_forward(const go_spec* s, const uint8_t* const* Wq, const float* const* wscale,
                     const float* X, int64_t B, float* out)
 {

@@ -166,6 +166,14 @@ void  go_e4m3_quant_rows(const float* x, int64_t rows, int64_t cols, uint8_t* q,
 void  go_fp8_forward(const go_spec* spec, const uint8_t* const* Wq, const float* const* wscale,
                      const float* X, int64_t B, float* out);
 
+/* the same with block-scaled activations: an E8M0 byte per row and 32 consecutive columns, [rows][ceil(cols/32)],
+   value 2^(byte-127) = the power of two that brings the block's largest magnitude into (224, 448]; no reference
+   counterpart.  Pinned by tests/test_oracle_formats.py against torch's float8_e4m3fn casts and the rule's
+   defining inequalities. */
+void  go_e4m3_quant_rows_block32(const float* x, int64_t rows, int64_t cols, uint8_t* q, uint8_t* scale);
+void  go_fp8_forward_block32(const go_spec* spec, const uint8_t* const* Wq, const float* const* wscale,
+                             const float* X, int64_t B, float* out);
+
 #ifdef __cplusplus
 }
 #endif

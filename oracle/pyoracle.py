@@ -101,6 +101,8 @@ def lib():
             "go_e4m3_to_f32": (C.c_float, [C.c_uint8]),
             "go_e4m3_quant_rows": (None, [f32p, C.c_int64, C.c_int64, u8p, f32p]),
             "go_fp8_forward": (None, [C.POINTER(Spec), C.POINTER(vp), C.POINTER(vp), f32p, C.c_int64, f32p]),
+            "go_e4m3_quant_rows_block32": (None, [f32p, C.c_int64, C.c_int64, u8p, u8p]),
+            "go_fp8_forward_block32": (None, [C.POINTER(Spec), C.POINTER(vp), C.POINTER(vp), f32p, C.c_int64, f32p]),
         }
         for name, (res, args) in sig.items():
             fn = getattr(L, name)
@@ -274,7 +276,16 @@ def e4m3_table():
     return np.array([lib().go_e4m3_to_f32(i) for i in range(256)], np.float32)
 
 
-def fp8_forward(spec, Wq, wscale, X):
+def e4m3_quant_rows_block32(x):
+    """Block-scaled quantiser: (codes [rows][cols], E8M0 bytes [rows][ceil(cols / 32)])."""
+    x = np.ascontiguousarray(x, np.float32)
+    q = np.empty(x.shape, np.uint8)
+    s = np.empty((x.shape[0], (x.shape[1] + 31) // 32), np.uint8)
+    lib().go_e4m3_quant_rows_block32(x, x.shape[0], x.shape[1], q, s)
+    return q, s
+
+
+def fp8_forward(spec, Wq, wscale, X, block32=False):
     nl = spec.n_layers
     X = np.ascontiguousarray(X, np.float32)
     Wq = [np.ascontiguousarray(w, np.uint8) for w in Wq]
@@ -282,7 +293,7 @@ def fp8_forward(spec, Wq, wscale, X):
     wp = (C.c_void_p * nl)(*[w.ctypes.data for w in Wq])
     sp = (C.c_void_p * nl)(*[s.ctypes.data for s in wscale])
     out = np.empty((X.shape[0], spec.sizes[nl]), np.float32)
-    lib().go_fp8_forward(C.byref(spec), wp, sp, X, X.shape[0], out)
+    (lib().go_fp8_forward_block32 if block32 else lib().go_fp8_forward)(C.byref(spec), wp, sp, X, X.shape[0], out)
     return out
 
 

@@ -108,22 +108,48 @@ def test_fp8_quantiser_bit_exact_and_forward():
         q, s = po.e4m3_quant_rows(Ws[l])
         assert np.array_equal(codes[l], q), l          # byte work: bit exact
         assert np.array_equal(scales[l].view(np.uint32), s.view(np.uint32)), l
-    out = g.forward(X)
     spec = po.make_spec(sizes, acts)
-    emu = po.fp8_forward(spec, codes, scales, X)
-    # same quantised pipeline, only the fp32 accumulation order differs (plus re-quantisation
-    # flips it can cause): 2e-2 relative RMS, typically ~1e-3
-    err = np.sqrt(np.mean((out - emu) ** 2)) / np.sqrt(np.mean(emu ** 2))
-    assert err < 2e-2, err
     ca = po.CanonNet(spec)
     for l in range(3):
         ca.set_params(l, po.e4m3_table()[codes[l]] * scales[l][:, None])
     ref = ca.forward(X)
-    err = np.sqrt(np.mean((out - ref) ** 2)) / np.sqrt(np.mean(ref ** 2))
-    assert err < 5e-2, err
-    # random weights, 256 near-flat classes: printed, not a tolerance (see the trained networks below)
-    print("e4m3 top-1 agreement on random weights, all rows", (out.argmax(1) == ref.argmax(1)).mean(), flush=True)
+    # both ways of re-quantising the activations between layers: a power-of-two scale per token and 32 units
+    # (made in the products' epilogues), one fp32 scale per token (a kernel of its own)
+    for mode in (pg.FP8_ACT_BLOCK32, pg.FP8_ACT_PER_TOKEN):
+        g.set_fp8_activation_scaling(mode)
+        out = g.forward(X)
+        emu = po.fp8_forward(spec, codes, scales, X, block32=(mode == pg.FP8_ACT_BLOCK32))
+        # same quantised pipeline, only the fp32 accumulation order differs (plus re-quantisation
+        # flips it can cause): 2e-2 relative RMS, typically ~1e-3
+        err = np.sqrt(np.mean((out - emu) ** 2)) / np.sqrt(np.mean(emu ** 2))
+        print("activation scaling", mode, "vs restated pipeline", err, flush=True)
+        assert err < 2e-2, (mode, err)
+        err = np.sqrt(np.mean((out - ref) ** 2)) / np.sqrt(np.mean(ref ** 2))
+        print("activation scaling", mode, "vs fp32 forward on the dequantised weights", err, flush=True)
+        assert err < 5e-2, (mode, err)
+        # random weights, 256 near-flat classes: printed, not a tolerance (see the trained networks below)
+        print("e4m3 top-1 agreement on random weights, all rows", (out.argmax(1) == ref.argmax(1)).mean(), flush=True)
     g.close()
+
+
+def test_block32_quantiser_bit_exact():
+    """The block-scaled activation quantiser on its own (the device function the products' epilogues apply):
+    codes and E8M0 bytes bit for bit against the restatement, on blocks of very different magnitudes, an
+    all-zero block, a ragged last block and the rule's edge (largest magnitude exactly 448 2^k, and one
+    bf16 step above)."""
+    import pyglades as pg
+    rng = np.random.default_rng(77)
+    rows, cols = 129, 32 * 11 + 5
+    mag = 10.0 ** rng.uniform(-8, 8, (rows, (cols + 31) // 32))
+    x = po.bf16_round((rng.standard_normal((rows, cols)) * np.repeat(mag, 32, axis=1)[:, :cols]).astype(np.float32))
+    x[3, 32:64] = 0.0
+    x[4, :] = 0.0
+    x[5, 0:32] = 0.0; x[5, 7] = 448.0 * 2.0 ** -5
+    x[6, 0:32] = 0.0; x[6, 7] = -450.0 * 2.0 ** -5
+    codes, scales = pg.quantize_rows_e4m3_block32(x)
+    rq, rs = po.e4m3_quant_rows_block32(x)
+    assert np.array_equal(scales, rs)
+    assert np.array_equal(codes, rq)
 
 
 def test_lowprec_state_rules():
@@ -224,10 +250,12 @@ def test_low_precision_random_shapes(seed):
         c, sc = po.e4m3_quant_rows(Ws[l])
         assert np.array_equal(codes[l], c) and np.array_equal(scales[l].view(np.uint32), sc.view(np.uint32)), l
     Xq = po.bf16_round(X[:B])
-    out = q.forward(Xq)
-    emu = po.fp8_forward(po.make_spec(sizes, facts, act_params=1.0), codes, scales, Xq)
-    err = np.sqrt(np.mean((out - emu) ** 2)) / max(np.sqrt(np.mean(emu ** 2)), 1e-30)
-    assert err < 2e-2, err
+    for mode in (pg.FP8_ACT_BLOCK32, pg.FP8_ACT_PER_TOKEN):
+        q.set_fp8_activation_scaling(mode)
+        out = q.forward(Xq)
+        emu = po.fp8_forward(po.make_spec(sizes, facts, act_params=1.0), codes, scales, Xq, block32=(mode == pg.FP8_ACT_BLOCK32))
+        err = np.sqrt(np.mean((out - emu) ** 2)) / max(np.sqrt(np.mean(emu ** 2)), 1e-30)
+        assert err < 2e-2, (mode, err)
     q.close()
 
 
@@ -323,13 +351,15 @@ def test_fp8_forward_off_the_tile_grid():
         q, s = po.e4m3_quant_rows(Ws[l])
         assert np.array_equal(codes[l], q), l
         assert np.array_equal(scales[l].view(np.uint32), s.view(np.uint32)), l
-    out = g.forward(X)
-    assert out.shape == (B, sizes[-1])
     spec = po.make_spec(sizes, acts, act_params=1.0)
-    emu = po.fp8_forward(spec, codes, scales, X)
-    err = np.sqrt(np.mean((out - emu) ** 2)) / np.sqrt(np.mean(emu ** 2))
-    print("off-grid e4m3 vs restated pipeline", err, flush=True)
-    assert err < 2e-2, err
+    for mode in (pg.FP8_ACT_PER_TOKEN, pg.FP8_ACT_BLOCK32):
+        g.set_fp8_activation_scaling(mode)
+        out = g.forward(X)
+        assert out.shape == (B, sizes[-1])
+        emu = po.fp8_forward(spec, codes, scales, X, block32=(mode == pg.FP8_ACT_BLOCK32))
+        err = np.sqrt(np.mean((out - emu) ** 2)) / np.sqrt(np.mean(emu ** 2))
+        print("off-grid e4m3 vs restated pipeline, activation scaling", mode, err, flush=True)
+        assert err < 2e-2, (mode, err)
     # the same rows as a table on the device, and its metrics pass
     Y = np.eye(sizes[-1], dtype=np.float32)[emu.argmax(1)]
     g.set_dataset(X, Y)
@@ -541,15 +571,17 @@ def test_lowprec_inference_top1_on_a_trained_network():
     for l in range(3):
         q.set_params(l, Wt[l][0], Wt[l][1])
     codes, scales = q.quantize_fp8()
-    got8 = q.forward(Xt)
-    q.close()
     for l in range(3):
         ref.set_params(l, po.e4m3_table()[codes[l]] * scales[l][:, None], Wt[l][1])
     want8 = ref.forward(Xt)
-    agree8 = (got8.argmax(1) == want8.argmax(1)).mean()
-    print("e4m3 forward: top-1 agreement %.4f over all rows, logits rel RMS %.2e" % (agree8, rel_rms(got8, want8)), flush=True)
-    assert agree8 >= 0.995
-    assert rel_rms(got8, want8) <= 5e-2      # three quantisation points
+    for mode in (pg.FP8_ACT_BLOCK32, pg.FP8_ACT_PER_TOKEN):
+        q.set_fp8_activation_scaling(mode)
+        got8 = q.forward(Xt)
+        agree8 = (got8.argmax(1) == want8.argmax(1)).mean()
+        print("e4m3 forward, activation scaling %d: top-1 agreement %.4f over all rows, logits rel RMS %.2e" % (mode, agree8, rel_rms(got8, want8)), flush=True)
+        assert agree8 >= 0.995
+        assert rel_rms(got8, want8) <= 5e-2      # three quantisation points
+    q.close()
 
 
 def test_bf16_training_top1_on_separable_classes():
@@ -626,6 +658,7 @@ def test_cfg5_full_size_e4m3_against_fp32():
         codes, scales = q.quantize_fp8()
         for l in range(4):
             r.set_params(l, tab[codes[l]] * scales[l][:, None], bs[l])
+        q.set_fp8_activation_scaling(pg.FP8_ACT_BLOCK32)
         return q.forward(X), r.forward(X)
 
     got, want = both([w for w, _ in Wt], [b_ for _, b_ in Wt], Xt)
@@ -635,6 +668,12 @@ def test_cfg5_full_size_e4m3_against_fp32():
     assert (want.argmax(1) == cls).mean() >= 0.995
     assert agree >= 0.995
     assert err <= 6e-2
+    # the same network with one fp32 scale per token: the same bars
+    q.set_fp8_activation_scaling(pg.FP8_ACT_PER_TOKEN)
+    got_t = q.forward(Xt)
+    agree_t, err_t = (got_t.argmax(1) == want.argmax(1)).mean(), rel_rms(got_t, want)
+    print("trained network, one scale per token: top-1 agreement %.5f, logits rel RMS %.3e" % (agree_t, err_t), flush=True)
+    assert agree_t >= 0.995 and err_t <= 6e-2
     del Wt
     rng = np.random.default_rng(31)
     Wr = [rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(1.0 / sizes[l])) for l in range(4)]
