@@ -65,7 +65,7 @@ def measured_traffic(workload, kernel):
 WORKLOADS = {
     "cfg4": dict(desc="bf16 train MLP 4096-4096-4096-4096-4096-1024 ReLU softmax-CE, batch 8192, SGD momentum 0.9, fp32 master",
                  sizes=[4096, 4096, 4096, 4096, 4096, 1024], batch=8192, rows=262144, dtype="bf16", kind="train"),
-    "cfg5": dict(desc="e4m3 inference MLP 8192-8192-8192-8192-1024 ReLU, batch 16384, per-channel weight / per-row activation scales",
+    "cfg5": dict(desc="e4m3 inference MLP 8192-8192-8192-8192-1024 ReLU, batch 16384, fp32 scale per weight output channel, activations re-quantised per token between layers",
                  sizes=[8192, 8192, 8192, 8192, 1024], batch=16384, rows=16384, dtype="fp8", kind="infer"),
     "cfg3": dict(desc="fp32 train MLP 784-1024-1024-10 ReLU softmax-CE, batch 512, SGD lr .05 momentum .9 L2 1e-4",
                  sizes=[784, 1024, 1024, 10], batch=512, rows=60000, dtype="f32", kind="train"),
@@ -73,6 +73,11 @@ WORKLOADS = {
                  sizes=[32, 64, 64, 1], batch=256, rows=10000, dtype="f32", kind="exact"),
     "cfg1": dict(desc="exact mode MLP 4-16-3 sigmoid BCE, 150 rows, mb 150, lr .01 momentum .9",
                  sizes=[4, 16, 3], batch=150, rows=150, dtype="f32", kind="exact"),
+    # the two narrow configurations in canonical (batched) mode; cfg1 here is BASELINE.json's configs[0] as written
+    "cfg1_canonical": dict(desc="canonical mode MLP 4-16-3 sigmoid / softmax cross-entropy, 150 rows, full batch, lr .1 momentum .9, Xavier-uniform",
+                           sizes=[4, 16, 3], batch=150, rows=150, dtype="f32", kind="narrow"),
+    "cfg2_canonical": dict(desc="canonical mode MLP 32-64-64-1 tanh/tanh/linear MSE, 10000 rows, mb 256, lr .01 momentum .9",
+                           sizes=[32, 64, 64, 1], batch=256, rows=10000, dtype="f32", kind="narrow"),
 }
 
 
@@ -307,13 +312,79 @@ def run_exact(w, args):
     return value, el, roof, extra
 
 
+def narrow_tables(w, pg_or_po):
+    """Synthetic tables, activations and weights of the two narrow configurations."""
+    m = pg_or_po
+    sizes, N = w["sizes"], w["rows"]
+    rng = np.random.default_rng(1234)
+    if w["name"].startswith("cfg2"):
+        t = np.arange(N + 32, dtype=np.float64)
+        f, ph = rng.random(3) * 0.05 + 0.01, rng.random(3) * 6.28
+        sig = sum(np.sin(2 * np.pi * f[k] * t + ph[k]) for k in range(3)) + rng.standard_normal(N + 32) * 0.05
+        X = np.stack([sig[i:i + 32] for i in range(N)]).astype(np.float32)
+        Y = sig[32:32 + N, None].astype(np.float32)
+        acts, params, cost, hyper = [m.TANH, m.TANH, m.LINEAR], [0, 0, 1.0], m.REGRESSION, dict(lr=0.01, mom=0.9)
+    else:
+        c = rng.random((3, 4)) * 8
+        lab = np.repeat(np.arange(3), 50)
+        X = (c[lab] + rng.standard_normal((150, 4)) * 0.5).astype(np.float32)
+        Y = np.eye(3, dtype=np.float32)[lab]
+        acts, params, cost, hyper = [m.SIGMOID, m.SOFTMAX], [0, 0], m.CLASSIFICATION, dict(lr=0.1, mom=0.9)
+    nl = len(sizes) - 1
+    Ws = [rng.uniform(-1, 1, (sizes[l + 1], sizes[l])).astype(np.float32) * np.float32(np.sqrt(6.0 / (sizes[l] + sizes[l + 1]))) for l in range(nl)]
+    return X, Y, acts, params, cost, hyper, Ws
+
+
+def run_narrow(w, args):
+    """Canonical mode on a narrow network: `steps` epochs through ghip_net_run_epochs_canonical, with the
+    library's own choice of kernels (value) and with each of the two paths forced (detail)."""
+    import pyglades as pg
+    sizes, N, B = w["sizes"], w["rows"], w["batch"]
+    X, Y, acts, params, cost, hyper, Ws = narrow_tables(w, pg)
+    nl = len(sizes) - 1
+    res = {}
+    for path, code in (("auto", pg.CANON_PATH_AUTO), ("one_workgroup", pg.CANON_PATH_ONE_WORKGROUP), ("launches", pg.CANON_PATH_LAUNCHES)):
+        net = pg.Net(pg.make_spec(sizes, acts, act_params=params, cost=cost, mode=pg.MODE_CANONICAL, dtype=pg.F32, batch=B, **hyper))
+        for l in range(nl):
+            net.set_params(l, Ws[l])
+        net.set_canonical_path(code)
+        net.set_dataset(X, Y)
+        for _ in range(max(1, args.warmup)):
+            net.run_epochs_canonical(B, 1)
+        net.sync()
+        t0 = time.perf_counter()
+        ms = net.run_epochs_canonical(B, args.steps)
+        net.sync()
+        el = time.perf_counter() - t0
+        prof = kernel_profile(net, lambda s_: net.run_epochs_canonical(B, args.steps), 1)
+        net.close()
+        res[path] = dict(el=el, loss=ms[-1][0], prof=prof)
+    el = res["auto"]["el"]
+    value = args.steps * N / el
+    prof = res["auto"]["prof"]
+    dom = max(prof, key=lambda k: prof[k][0])
+    kernel_ms = sum(v[0] for v in prof.values())
+    bytes_per_sample = 4 * (sizes[0] + sizes[-1])
+    ach = args.steps * N * bytes_per_sample / (kernel_ms * 1e-3) / 1e9
+    roof = dict(bound="hbm", kernel=dom, achieved=round(ach, 4), peak=HBM_PEAK, unit="GB/s", frac=round(ach / HBM_PEAK, 8), traffic=None,
+                avg_launch_ms=round(prof[dom][0] / prof[dom][1], 4),
+                note="latency- and issue-bound: table traffic is 4 (inputs + outputs) bytes per row against a few thousand multiply-adds")
+    extra = dict(final_loss=res["auto"]["loss"], flop_per_sample=train_flops_per_sample(sizes),
+                 paths={k: dict(ms_per_epoch=round(v["el"] / args.steps * 1e3, 4), value=round(args.steps * N / v["el"], 1),
+                                launches_per_call=int(sum(c for _, c in v["prof"].values()))) for k, v in res.items()})
+    return value, el, roof, extra
+
+
 def cpu_baseline(w, budget_s=20.0):
-    """The CPU restatement (oracle/, kind "port") timed on this host's cores on a bounded sample."""
+    """The CPU restatement (oracle/, kind "port") timed on this host's cores on a bounded sample.  `cores` = the
+    threads used, `nproc` = the cores this process may run on; exact mode runs on one thread as the reference does,
+    canonical mode on one thread AND on all cores (value = all cores, `one_thread` beside it)."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import pyoracle as po
     sizes = w["sizes"]
     nl = len(sizes) - 1
-    cores = min(16, os.cpu_count() or 1)
+    nproc = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(16, nproc)
     rng = np.random.default_rng(7)
     if w["kind"] == "exact":
         acts = [po.TANH, po.TANH, po.LINEAR] if w["name"] == "cfg2" else [po.SIGMOID, po.SIGMOID]
@@ -331,29 +402,52 @@ def cpu_baseline(w, budget_s=20.0):
                 net.epoch(X, Y, want_preds=False)
                 ep += 1
         el = time.perf_counter() - t0
-        return dict(value=round(ep * N / el, 1), unit="samples/s", cores=1, kind="port",
+        return dict(value=round(ep * N / el, 1), unit="samples/s", cores=1, nproc=nproc, kind="port",
                     sample=f"{ep} epochs of {N} rows, exact mode, 1 thread (the reference is single-threaded)")
-    po.lib().go_set_threads(cores)
+    if w["kind"] == "narrow":
+        X, Y, acts, params, cost, hyper, Ws = narrow_tables(w, po)
+        N, B = w["rows"], w["batch"]
+        out = {}
+        for threads in (1, cores):
+            po.lib().go_set_threads(threads)
+            net = po.CanonNet(po.make_spec(sizes, acts, act_params=params, cost=cost, **hyper))
+            for l in range(nl):
+                net.set_params(l, Ws[l])
+            ep, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < min(budget_s, 3.0):
+                for r0 in range(0, N, B):
+                    net.step(X[r0:r0 + B], Y[r0:r0 + B])
+                ep += 1
+            out[threads] = (ep * N / (time.perf_counter() - t0), ep)
+        best = max(out, key=lambda k: out[k][0])
+        return dict(value=round(out[best][0], 1), unit="samples/s", cores=best, nproc=nproc, kind="port",
+                    one_thread=round(out[1][0], 1), all_cores=round(out[cores][0], 1),
+                    sample=f"{out[best][1]} epochs of {N} rows in batches of {B}, canonical mode, fp32; 1 thread and {cores} OpenMP threads timed, the faster reported")
     acts = [po.RELU] * (nl - 1) + ([po.SOFTMAX] if w["kind"] == "train" else [po.RELU])
-    net = po.CanonNet(po.make_spec(sizes, acts, lr=0.01, mom=0.9, cost=po.CLASSIFICATION))
-    for l in range(nl):
-        net.set_params(l, (rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l]))))
     rows = {"cfg4": 256, "cfg5": 256, "cfg3": 512}.get(w["name"], 256)
     X = rng.standard_normal((rows, sizes[0]), dtype=np.float32)
     Y = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], rows)]
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        if w["kind"] == "train":
-            net.step(X, Y)
-        else:
-            net.forward(X)
-        reps += 1
-        if time.perf_counter() - t0 > budget_s / 2 or reps >= 50:
-            break
-    el = time.perf_counter() - t0
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l]))) for l in range(nl)]
+    rates = {}
+    for threads, share in ((cores, 0.8), (1, 0.2)):
+        po.lib().go_set_threads(threads)
+        net = po.CanonNet(po.make_spec(sizes, acts, lr=0.01, mom=0.9, cost=po.CLASSIFICATION))
+        for l in range(nl):
+            net.set_params(l, Ws[l])
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            if w["kind"] == "train":
+                net.step(X, Y)
+            else:
+                net.forward(X)
+            reps += 1
+            if time.perf_counter() - t0 > budget_s * share / 2 or reps >= 50:
+                break
+        rates[threads] = (reps * rows / (time.perf_counter() - t0), reps)
+        del net
     what = "fwd+bwd+update steps" if w["kind"] == "train" else "fp32 forwards"
-    return dict(value=round(reps * rows / el, 1), unit="samples/s", cores=cores, kind="port",
-                sample=f"{reps} {what} of {rows} rows (1/{w['batch'] // rows} of a batch), fp32, {cores} OpenMP threads")
+    return dict(value=round(rates[cores][0], 1), unit="samples/s", cores=cores, nproc=nproc, kind="port", one_thread=round(rates[1][0], 1),
+                sample=f"{rates[cores][1]} {what} of {rows} rows (1/{w['batch'] // rows} of a batch), fp32, {cores} OpenMP threads ({rates[1][1]} on 1 thread for one_thread)")
 
 
 def main():
@@ -390,9 +484,9 @@ def main():
         return
     w = dict(WORKLOADS[args.workload], name=args.workload)
     if args.steps is None:
-        args.steps = {"cfg4": 40, "cfg5": 40, "cfg3": 200, "cfg2": 5, "cfg1": 200}[args.workload]
+        args.steps = {"cfg4": 40, "cfg5": 40, "cfg3": 200, "cfg2": 5, "cfg1": 200, "cfg1_canonical": 500, "cfg2_canonical": 10}[args.workload]
     if args.warmup is None:
-        args.warmup = {"cfg4": 5, "cfg5": 5, "cfg3": 20, "cfg2": 1, "cfg1": 5}[args.workload]
+        args.warmup = {"cfg4": 5, "cfg5": 5, "cfg3": 20, "cfg2": 1, "cfg1": 5, "cfg1_canonical": 1, "cfg2_canonical": 1}[args.workload]
     import torch
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -400,6 +494,9 @@ def main():
     args.extras = args.workload == "cfg4" and not args.no_extras
     if w["kind"] == "exact":
         value, el, roof, extra = run_exact(w, args)
+        unit_rows = w["rows"]
+    elif w["kind"] == "narrow":
+        value, el, roof, extra = run_narrow(w, args)
         unit_rows = w["rows"]
     else:
         value, el, roof, extra = run_canonical(w, args)
@@ -413,8 +510,16 @@ def main():
             v5, el5, roof5, extra5 = run_canonical(w5, a5)
             extra["infer"] = dict(metric="infer samples/sec", value=round(v5, 1), unit="samples/s", steps=a5.steps, warmup=a5.warmup,
                                   ms_per_step=round(el5 / a5.steps * 1e3, 4), dtype="fp8", workload="cfg5: " + w5["desc"],
+                                  activation_scaling="per token, an E8M0 scale per 32 units, written by the producing product's epilogue",
                                   flop_per_sample=infer_flops_per_sample(w5["sizes"]), roofline=roof5,
                                   step_frac_of_peak=extra5["step_frac_of_peak"], kernel_ms_per_step=extra5["kernel_ms_per_step"])
+            if not args.no_cpu_baseline:
+                extra["infer"]["cpu_baseline"] = cpu_baseline(w5, budget_s=8.0)
+            # the same pass with one fp32 scale per token, re-quantised by a kernel of its own
+            a5.fp8_act = "per_token"
+            v5t, el5t, roof5t, extra5t = run_canonical(w5, a5)
+            extra["infer"]["per_token_fp32_scale"] = dict(value=round(v5t, 1), ms_per_step=round(el5t / a5.steps * 1e3, 4),
+                                                          step_frac_of_peak=extra5t["step_frac_of_peak"], kernel_ms_per_step=extra5t["kernel_ms_per_step"])
         except Exception as e:  # noqa: BLE001
             extra["infer"] = dict(error=repr(e))
         try:
@@ -422,16 +527,25 @@ def main():
         except Exception as e:  # noqa: BLE001
             extra["vendor_gemm"] = dict(error=repr(e))
         others = {}
-        for name, subnets in (("cfg3", 1), ("cfg1", 1), ("cfg2", 1), ("cfg1", 1024), ("cfg1", 4096)):
+        for name, subnets in (("cfg3", 1), ("cfg1", 1), ("cfg2", 1), ("cfg1", 1024), ("cfg1", 4096), ("cfg1_canonical", 1), ("cfg2_canonical", 1)):
             key = name if subnets == 1 else f"{name}_x{subnets}"
             try:
                 wo = dict(WORKLOADS[name], name=name)
-                ao = argparse.Namespace(steps={"cfg3": 200, "cfg2": 5, "cfg1": 200}[name], warmup={"cfg3": 20, "cfg2": 1, "cfg1": 5}[name],
+                ao = argparse.Namespace(steps={"cfg3": 200, "cfg2": 5, "cfg1": 200, "cfg1_canonical": 500, "cfg2_canonical": 10}[name],
+                                        warmup={"cfg3": 20, "cfg2": 1, "cfg1": 5, "cfg1_canonical": 1, "cfg2_canonical": 1}[name],
                                         extras=False, subnets=subnets)
-                vo, elo, roofo, _ = run_exact(wo, ao) if wo["kind"] == "exact" else run_canonical(wo, ao)
+                run = {"exact": run_exact, "narrow": run_narrow}.get(wo["kind"], run_canonical)
+                vo, elo, roofo, extrao = run(wo, ao)
                 others[key] = dict(value=round(vo, 1), unit="samples/s", steps=ao.steps, ms_per_step=round(elo / ao.steps * 1e3, 4),
                                    dtype=wo["dtype"], workload=f"{name}: {wo['desc']}" + (f", {subnets} subnets side by side" if subnets > 1 else ""),
-                                   kernel=roofo["kernel"], kernel_avg_launch_ms=roofo["avg_launch_ms"])
+                                   kernel=roofo["kernel"], kernel_avg_launch_ms=roofo["avg_launch_ms"],
+                                   roofline={k: roofo[k] for k in ("bound", "kernel", "achieved", "peak", "unit", "frac", "traffic") if k in roofo})
+                if "step_frac_of_peak" in extrao:
+                    others[key]["step_frac_of_peak"] = extrao["step_frac_of_peak"]
+                if "paths" in extrao:
+                    others[key]["paths"] = extrao["paths"]
+                if not args.no_cpu_baseline and subnets == 1:
+                    others[key]["cpu_baseline"] = cpu_baseline(wo, budget_s=6.0)
             except Exception as e:  # noqa: BLE001
                 others[key] = dict(error=repr(e))
         extra["other_configs"] = others
@@ -445,6 +559,9 @@ def main():
                    "flop_per_sample": train_flops_per_sample(w["sizes"]) if w["kind"] != "infer" else infer_flops_per_sample(w["sizes"])},
         "roofline": roof,
     }
+    if w["kind"] == "infer":
+        out["config"]["activation_scaling"] = ("one fp32 scale per token, a re-quantisation kernel between layers" if args.fp8_act == "per_token" else
+                                               "per token, an E8M0 scale per 32 units, written by the producing product's epilogue")
     out["detail"] = extra
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w)

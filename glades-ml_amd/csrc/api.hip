@@ -135,6 +135,15 @@ struct ghip_net {
     float* narrowPart = nullptr;  // fp32 canonical, output layer at most 16 wide: partial gradient sums per chunk of rows
     float* stageX = nullptr;
     int cap_batch = 0;
+    // narrow networks as one persistent workgroup (canon_narrow.hip): layout for training / for evaluation,
+    // per-epoch figures of a launch over several epochs, the number of epochs it ran
+    bool narrow_fit = false;
+    CanonNarrowArgs narrowTrain, narrowEval;
+    size_t narrowLdsTrain = 0, narrowLdsEval = 0;
+    double* narrowEpochs = nullptr;
+    int narrowEpochsCap = 0;
+    int* narrowRan = nullptr;
+    int canon_path = GHIP_CANON_PATH_AUTO;
     // metrics of a batch: three banks of 4 doubles.  A metrics launch adds into bank accBank^1 and
     // clears the bank the launch after it will use, so no separate clearing launch is needed; bank 2
     // takes the sums of launches whose metrics nobody reads.
@@ -364,6 +373,11 @@ int setup_canon(ghip_net* n)
             TRY(dalloc(&n->wscale[l], (size_t)ps[l + 1]));
         }
     }
+    if (s.dtype == GHIP_F32) {
+        n->narrow_fit = ghip_canon_narrow_plan(s.sizes, s.n_layers, 1, &n->narrowTrain, &n->narrowLdsTrain) &&
+                        ghip_canon_narrow_plan(s.sizes, s.n_layers, 0, &n->narrowEval, &n->narrowLdsEval);
+        if (n->narrow_fit) TRY(dalloc(&n->narrowRan, 1));
+    }
     TRY(dalloc(&n->dAcc, 16));  // two alternating banks per step, one for softmax-only launches, one per pass over the table
     HIP_TRY(hipMemsetAsync(n->dAcc, 0, 16 * sizeof(double), n->stream));
     return 0;
@@ -519,8 +533,49 @@ int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
     return 0;
 }
 
+// ---- narrow canonical networks: one persistent workgroup ----
+// Whether a pass in batches of `batch` goes to the one-workgroup kernel.  It runs on one CU, whose fp32 rate bounds
+// it; the GEMM launches cost a fixed ~8 us each (7 to a step) and then use the whole chip.  Measured cross-over:
+// about 2.5 10^5 multiply-adds per forward pass of a batch
+// (13 us + 0.14 us per thousand of them against 50 us of launches).
+bool use_narrow(const ghip_net* n, int batch)
+{
+    if (!n->narrow_fit || n->canon_path == GHIP_CANON_PATH_LAUNCHES) return false;
+    if (n->canon_path == GHIP_CANON_PATH_ONE_WORKGROUP) return true;
+    long long macs = 0;
+    for (int l = 0; l < n->spec.n_layers; ++l) macs += (long long)n->spec.sizes[l] * n->spec.sizes[l + 1];
+    return macs * batch <= 250000;
+}
+
+// n_epochs passes over rows [row0, row0 + rows) in batches of `batch`; per epoch 4 doubles at `metrics` (device)
+int run_narrow(ghip_net* n, int64_t row0, int64_t rows, int batch, int n_epochs, int train, float stop_accuracy, int reset_cm,
+               double* metrics, double* clear4 = nullptr)
+{
+    const ghip_net_spec& s = n->spec;
+    const int L = s.n_layers;
+    CanonNarrowArgs a = train ? n->narrowTrain : n->narrowEval;
+    for (int l = 0; l < L; ++l) {
+        a.act[l] = s.act[l]; a.act_param[l] = s.act_param[l];
+        a.lr[l] = s.lr[l]; a.mom[l] = s.mom[l]; a.wd1[l] = s.wd1[l]; a.wd2[l] = s.wd2[l];
+        a.W[l] = n->W[l]; a.b[l] = n->b[l]; a.vW[l] = n->vW[l]; a.vb[l] = n->vb[l];
+    }
+    a.cost = s.cost;
+    a.X = n->dX + row0 * s.sizes[0]; a.Y = n->dY + row0 * s.sizes[L];
+    a.n_rows = rows; a.batch = batch; a.n_epochs = n_epochs; a.train = train ? 1 : 0; a.stop_accuracy = stop_accuracy;
+    a.cm = n->cm; a.reset_cm = reset_cm;
+    a.metrics = metrics; a.epochs_run = n->narrowRan; a.clear4 = clear4;
+    LAUNCH(n, train ? "canon_narrow_train" : "canon_narrow_eval",
+           ghip_canon_narrow_run(a, train ? n->narrowLdsTrain : n->narrowLdsEval, n->stream));
+    return 0;
+}
+
 int step_f32(ghip_net* n, int64_t row0, int B)
 {
+    if (use_narrow(n, B)) {
+        // the kernel writes the batch's sums where the next reader expects them; the bank after it starts at zero
+        const DeltaArgs da = delta_args(n, nullptr, nullptr, nullptr, nullptr, B);
+        return run_narrow(n, row0, B, B, 1, 1, 0.0f, 0, da.acc, da.acc_clear);
+    }
     const ghip_net_spec& s = n->spec;
     const int L = s.n_layers;
     const float* X = n->dX + row0 * s.sizes[0];
@@ -854,7 +909,7 @@ int ghip_net_destroy(ghip_net* n)
         dfree(n->W[l]); dfree(n->b[l]); dfree(n->vW[l]); dfree(n->vb[l]);
         dfree(n->Wh[l]); dfree(n->WhT[l]); dfree(n->Wq[l]); dfree(n->wscale[l]);
     }
-    dfree(n->dAcc);
+    dfree(n->dAcc); dfree(n->narrowEpochs); dfree(n->narrowRan);
     if (n->stream) (void)hipStreamDestroy(n->stream);
     delete n;
     return 0;
@@ -1306,6 +1361,18 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
     if (batch > N) batch = (int)N;
     TRY(reserve_batch(n, batch));
     if (s.dtype == GHIP_BF16) TRY(refresh_shadows(n));
+    if (s.dtype == GHIP_F32 && use_narrow(n, batch)) {
+        // the whole pass is one launch
+        TRY(run_narrow(n, 0, N, batch, 1, train, 0.0f, 0, n->dAcc + 12));
+        n->last_batch = (int)(N % batch ? N % batch : batch);
+        double acc[4];
+        HIP_TRY(hipMemcpyAsync(acc, n->dAcc + 12, sizeof(acc), hipMemcpyDeviceToHost, n->stream));
+        HIP_TRY(hipStreamSynchronize(n->stream));
+        host_metrics->loss = (float)(acc[0] / (double)N);
+        host_metrics->accuracy = (float)(acc[1] / ((double)N * s.sizes[L]));
+        host_metrics->correct = (int64_t)(acc[2] + 0.5);
+        return 0;
+    }
     LAUNCH(n, "fill_pass_metrics", ghip_fill_f64(n->dAcc + 12, 4, 0.0, n->stream));
     n->passAcc = true;
     int rc = 0;
@@ -1330,6 +1397,62 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
     host_metrics->loss = (float)(acc[0] / (double)N);
     host_metrics->accuracy = (float)(acc[1] / ((double)N * s.sizes[L]));
     host_metrics->correct = (int64_t)(acc[2] + 0.5);
+    return 0;
+}
+
+int ghip_net_run_epochs_canonical(ghip_net* n, int batch, int n_epochs, int train, float stop_accuracy,
+                                  ghip_metrics* host_metrics, int* epochs_run)
+{
+    if (!n || batch < 1 || n_epochs < 1 || !host_metrics) return fail(GHIP_EINVAL, "bad arguments");
+    HIP_TRY(hipSetDevice(g_device));
+    if (!is_canon(n)) return fail(GHIP_ESTATE, "network is not in canonical mode");
+    if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset");
+    const ghip_net_spec& s = n->spec;
+    const int64_t N = n->n_rows;
+    if (batch > N) batch = (int)N;
+    if (s.dtype == GHIP_F32 && use_narrow(n, batch)) {
+        // narrow network: the epochs are one launch, the stop condition is looked at on the device
+        if (n_epochs > n->narrowEpochsCap) {
+            (void)hipStreamSynchronize(n->stream);
+            dfree(n->narrowEpochs);
+            TRY(dalloc(&n->narrowEpochs, (size_t)4 * n_epochs));
+            n->narrowEpochsCap = n_epochs;
+        }
+        TRY(run_narrow(n, 0, N, batch, n_epochs, train, stop_accuracy, n->cm ? 1 : 0, n->narrowEpochs));
+        n->last_batch = (int)(N % batch ? N % batch : batch);
+        int ran = 0;
+        HIP_TRY(hipMemcpyAsync(&ran, n->narrowRan, sizeof(int), hipMemcpyDeviceToHost, n->stream));
+        HIP_TRY(hipStreamSynchronize(n->stream));
+        if (ran < 0 || ran > n_epochs) return fail(GHIP_EHIP, "the kernel reports %d epochs", ran);
+        std::vector<double> acc((size_t)4 * (ran > 0 ? ran : 1));
+        if (ran > 0) HIP_TRY(hipMemcpy(acc.data(), n->narrowEpochs, sizeof(double) * 4 * ran, hipMemcpyDeviceToHost));
+        for (int e = 0; e < ran; ++e) {
+            host_metrics[e].loss = (float)(acc[4 * e] / (double)N);
+            host_metrics[e].accuracy = (float)(acc[4 * e + 1] / ((double)N * s.sizes[s.n_layers]));
+            host_metrics[e].correct = (int64_t)(acc[4 * e + 2] + 0.5);
+        }
+        if (epochs_run) *epochs_run = ran;
+        return 0;
+    }
+    int ran = 0;
+    for (int e = 0; e < n_epochs; ++e) {
+        if (n->cm) TRY(ghip_net_confusion_reset(n));   // CMatrix::reset at the head of every epoch (network.cpp:183-185)
+        TRY(ghip_net_run_epoch_canonical(n, batch, train, host_metrics + e));
+        ++ran;
+        if (stop_accuracy > 0.0f && host_metrics[e].accuracy >= stop_accuracy) break;
+    }
+    if (epochs_run) *epochs_run = ran;
+    return 0;
+}
+
+int ghip_net_set_canonical_path(ghip_net* n, int path)
+{
+    if (!n || !is_canon(n)) return fail(GHIP_EINVAL, "not a canonical network");
+    if (path != GHIP_CANON_PATH_AUTO && path != GHIP_CANON_PATH_LAUNCHES && path != GHIP_CANON_PATH_ONE_WORKGROUP)
+        return fail(GHIP_EINVAL, "unknown path %d", path);
+    if (path == GHIP_CANON_PATH_ONE_WORKGROUP && !n->narrow_fit)
+        return fail(GHIP_EINVAL, "the one-workgroup kernel takes fp32 networks whose layers are at most 64 wide and fit its LDS");
+    n->canon_path = path;
     return 0;
 }
 

@@ -364,6 +364,33 @@ hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s);
 hipError_t ghip_narrow_train(const NarrowOutArgs& a, const DeltaArgs& da, hipStream_t s);
 hipError_t ghip_narrow_update(const NarrowOutArgs& a, hipStream_t s);
 
+// ---------------------------------------------------------------- narrow networks as one persistent workgroup (canon_narrow.hip)
+// Canonical fp32 training or evaluation of a network whose layers are all at most 64 wide: n_epochs passes over
+// rows [0, n_rows) of X / Y in batches of `batch` (the last one shorter), parameters and momentum read from and
+// written back to W / b / vW / vb, per epoch four doubles in `metrics` (loss sum, accuracy-term sum, rows whose
+// class agrees, 0) and the number of epochs run in *epochs_run (fewer than n_epochs if the mean accuracy term
+// reached stop_accuracy > 0).  ghip_canon_narrow_plan fills the layout fields; the caller fills the rest.
+struct CanonNarrowArgs {
+    int   n_layers;
+    int   sizes[GHIP_MAX_LAYERS + 1];
+    int   act[GHIP_MAX_LAYERS]; float act_param[GHIP_MAX_LAYERS];
+    float lr[GHIP_MAX_LAYERS], mom[GHIP_MAX_LAYERS], wd1[GHIP_MAX_LAYERS], wd2[GHIP_MAX_LAYERS];
+    int   cost;
+    const float* X; const float* Y; long long n_rows; int batch, n_epochs, train; float stop_accuracy;
+    float* W[GHIP_MAX_LAYERS]; float* b[GHIP_MAX_LAYERS]; float* vW[GHIP_MAX_LAYERS]; float* vb[GHIP_MAX_LAYERS];
+    int*  cm; int reset_cm;       // confusion counters (or NULL); cleared at the head of every epoch if reset_cm
+    double* metrics; int* epochs_run;
+    double* clear4;               // four doubles the launch sets to zero (the next metrics launch's accumulators), or NULL
+    // layout of the workgroup's LDS block, in floats
+    int rows_per_chunk, rc_shift;   // a power of two and its logarithm
+    int wave_per_weight;            // gradient sums: a wavefront per weight (small networks) or a thread per weight
+    int offW[GHIP_MAX_LAYERS], offB[GHIP_MAX_LAYERS], offVW[GHIP_MAX_LAYERS], offVB[GHIP_MAX_LAYERS], offG[GHIP_MAX_LAYERS], offGB[GHIP_MAX_LAYERS];
+    int offA[GHIP_MAX_LAYERS + 1], offD[GHIP_MAX_LAYERS + 1], pitchA[GHIP_MAX_LAYERS + 1];
+    int offY;                       // a chunk's targets, or -1 if they do not fit
+};
+bool ghip_canon_narrow_plan(const int* sizes, int n_layers, int train, CanonNarrowArgs* out, size_t* lds_bytes);
+hipError_t ghip_canon_narrow_run(const CanonNarrowArgs& a, size_t lds_bytes, hipStream_t s);
+
 hipError_t ghip_fill_f32(float* p, long long n, float v, hipStream_t s);
 hipError_t ghip_fill_f64(double* p, long long n, double v, hipStream_t s);
 

@@ -18,13 +18,14 @@ MODE_EXACT, MODE_CANONICAL = 0, 1
 F32, BF16, FP8_INFER = 0, 1, 2
 BIAS_SEQUENTIAL, BIAS_CLOSED_FORM = 0, 1
 FP8_ACT_PER_TOKEN, FP8_ACT_BLOCK32 = 0, 1
+CANON_PATH_AUTO, CANON_PATH_LAUNCHES, CANON_PATH_ONE_WORKGROUP = 0, 1, 2
 
 EXPORTS = [
     "ghip_init", "ghip_gmath_eval", "ghip_net_create", "ghip_net_destroy", "ghip_net_set_params", "ghip_net_get_params",
     "ghip_net_get_state", "ghip_net_set_state",
     "ghip_net_set_dropout_masks", "ghip_net_get_dropout_state", "ghip_net_set_dropout_state",
     "ghip_net_set_dataset", "ghip_net_set_dataset_device", "ghip_net_run_epochs_exact", "ghip_net_run_epochs_exact_multi",
-    "ghip_net_run_epoch_canonical", "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_forward_noalloc", "ghip_net_eval_resident",
+    "ghip_net_run_epoch_canonical", "ghip_net_run_epochs_canonical", "ghip_net_set_canonical_path", "ghip_net_train_step", "ghip_net_last_metrics", "ghip_net_forward", "ghip_net_forward_resident", "ghip_forward_noalloc", "ghip_net_eval_resident",
     "ghip_net_confusion_enable", "ghip_net_confusion_reset", "ghip_net_confusion_get", "ghip_net_class_metrics",
     "ghip_net_quantize_fp8", "ghip_net_set_fp8_activation_scaling", "ghip_quantize_rows_e4m3_block32", "ghip_net_sync", "ghip_net_profile", "ghip_net_profile_count",
     "ghip_net_profile_entry", "ghip_net_profile_reset", "ghip_last_error", "ghip_version",
@@ -94,6 +95,8 @@ def load():
             "ghip_net_run_epochs_exact": (i, [vp, i, i, f, vp, C.POINTER(i), vp]),
             "ghip_net_run_epochs_exact_multi": (i, [vp, i, i, i, f, vp, vp]),
             "ghip_net_run_epoch_canonical": (i, [vp, i, i, C.POINTER(Metrics)]),
+            "ghip_net_run_epochs_canonical": (i, [vp, i, i, i, f, vp, C.POINTER(i)]),
+            "ghip_net_set_canonical_path": (i, [vp, i]),
             "ghip_net_train_step": (i, [vp, i64, i, vp]),
             "ghip_net_last_metrics": (i, [vp, C.POINTER(Metrics)]),
             "ghip_net_forward": (i, [vp, vp, i, vp]),
@@ -306,6 +309,17 @@ class Net:
         m = Metrics()
         _check(self.lib.ghip_net_run_epoch_canonical(self.h, int(batch), 1 if train else 0, C.byref(m)))
         return m
+
+    def run_epochs_canonical(self, batch, n_epochs, train=True, stop_accuracy=0.0):
+        """Up to n_epochs passes (one launch for a narrow fp32 network): list of (loss, accuracy, correct) per epoch run."""
+        ms = (Metrics * n_epochs)()
+        ran = C.c_int(0)
+        _check(self.lib.ghip_net_run_epochs_canonical(self.h, int(batch), int(n_epochs), 1 if train else 0, float(stop_accuracy),
+                                                      C.cast(ms, C.c_void_p), C.byref(ran)))
+        return [(ms[e].loss, ms[e].accuracy, ms[e].correct) for e in range(ran.value)]
+
+    def set_canonical_path(self, path):
+        _check(self.lib.ghip_net_set_canonical_path(self.h, int(path)))
 
     def last_metrics(self):
         m = Metrics()

@@ -199,6 +199,27 @@ int ghip_net_run_epochs_exact_multi(ghip_net* const* nets, int count, int n_epoc
  * last ghip_net_train_step. */
 int ghip_net_run_epoch_canonical(ghip_net* net, int batch, int train, ghip_metrics* host_metrics);
 
+/* Canonical mode: up to n_epochs such passes, the epoch loop of NNetwork::run
+ * (Backend/Machine Learning/Networks/network.cpp:171-195) with the Terminator's accuracy condition
+ * (State/Terminator.cpp:63-78): host_metrics[e] receives epoch e's figures, *epochs_run how many were run;
+ * the loop ends early once an epoch's accuracy reaches stop_accuracy (> 0).  The confusion counters, if
+ * enabled, restart at the head of every epoch (network.cpp:183-185).  An fp32 network whose layers are all at
+ * most 64 wide runs the whole call as ONE launch of one persistent workgroup (parameters, momentum and a
+ * chunk of rows' activations in LDS; see ghip_net_set_canonical_path); other networks run pass by pass. */
+int ghip_net_run_epochs_canonical(ghip_net* net, int batch, int n_epochs, int train, float stop_accuracy,
+                                  ghip_metrics* host_metrics, int* epochs_run);
+
+/* Canonical fp32 networks: which kernels train and evaluate them.  No reference counterpart.
+ *   GHIP_CANON_PATH_AUTO (default): the one-workgroup kernel where it applies (every layer at most 64 wide,
+ *     state fits the LDS) and the work of a batch is small enough for one CU to beat a step's seven launches;
+ *   GHIP_CANON_PATH_LAUNCHES: always the GEMM / streaming launches;
+ *   GHIP_CANON_PATH_ONE_WORKGROUP: always the one-workgroup kernel (refused where it does not apply).
+ * Results agree to fp32 summation order either way. */
+#define GHIP_CANON_PATH_AUTO          0
+#define GHIP_CANON_PATH_LAUNCHES      1
+#define GHIP_CANON_PATH_ONE_WORKGROUP 2
+int ghip_net_set_canonical_path(ghip_net* net, int path);
+
 /* Canonical mode: one training step (forward, backward, update) on rows [row0, row0+batch) of
  * the resident table.  host_metrics may be NULL (then the call does not synchronise). */
 int ghip_net_train_step(ghip_net* net, int64_t row0, int batch, ghip_metrics* host_metrics);

@@ -8,7 +8,9 @@ import pyoracle as po
 pytestmark = pytest.mark.gpu
 
 
-def build_pair(sizes, acts, params, cost, lr, mom, wd1, wd2, seed, bias=True):
+def build_pair(sizes, acts, params, cost, lr, mom, wd1, wd2, seed, bias=True, path="launches"):
+    """path: which kernels the GPU network runs: "launches" (GEMM / streaming kernels, a step = several launches),
+    "one_workgroup" (the persistent kernel for narrow networks) or "auto" (the library's choice)."""
     import pyglades as pg
     rng = np.random.default_rng(seed)
     nl = len(sizes) - 1
@@ -20,6 +22,7 @@ def build_pair(sizes, acts, params, cost, lr, mom, wd1, wd2, seed, bias=True):
     for l in range(nl):
         o.set_params(l, Ws[l], bs[l])
         g.set_params(l, Ws[l], bs[l])
+    g.set_canonical_path({"auto": pg.CANON_PATH_AUTO, "launches": pg.CANON_PATH_LAUNCHES, "one_workgroup": pg.CANON_PATH_ONE_WORKGROUP}[path])
     return o, g, rng
 
 
@@ -52,10 +55,18 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("name,sizes,acts,params,cost,B", CASES)
-def test_training_steps_match_cpu(name, sizes, acts, params, cost, B):
-    print("case", name, flush=True)
-    o, g, rng = build_pair(sizes, acts, params, cost, 0.05, 0.9, 1e-4, 1e-3, 11)
+# the shapes whose layers are all at most 64 wide also run as one persistent workgroup
+NARROW_CASES = [c for c in CASES if max(c[1]) <= 64] + [
+    ("four_layers_widths_around_the_lane_groups", [63, 64, 1, 33, 17], [po.TANH, po.RELU, po.SIGMOID, po.SOFTMAX], [0] * 4, po.CLASSIFICATION, 97),
+    ("more_rows_than_a_chunk_and_a_ragged_last_chunk", [8, 24, 5], [po.RELU, po.SOFTMAX], [0, 0], po.CLASSIFICATION, 150),
+]
+
+
+@pytest.mark.parametrize("name,sizes,acts,params,cost,B,path",
+                         [c + ("launches",) for c in CASES] + [c + ("one_workgroup",) for c in NARROW_CASES])
+def test_training_steps_match_cpu(name, sizes, acts, params, cost, B, path):
+    print("case", name, path, flush=True)
+    o, g, rng = build_pair(sizes, acts, params, cost, 0.05, 0.9, 1e-4, 1e-3, 11, path=path)
     steps = 8
     N = B * steps
     X = rng.standard_normal((N, sizes[0])).astype(np.float32)
@@ -230,3 +241,151 @@ def test_cfg3_one_epoch_on_its_own_data():
     np.testing.assert_allclose(lg, lo, rtol=1e-4, atol=1e-4 * np.abs(lo).max())
     assert agree >= 0.995
     g.close()
+
+
+def _cfg1_as_written(seed=1234):
+    """BASELINE configs[0]: 150 rows x 4 features from 3 isotropic Gaussian clusters (sigma 0.5, centres uniform in
+    [0, 8]^4), one-hot labels, MLP 4-16-3 sigmoid / softmax, cross-entropy, Xavier-uniform weights, zero biases."""
+    rng = np.random.default_rng(seed)
+    centres = rng.random((3, 4)) * 8
+    lab = np.repeat(np.arange(3), 50)
+    X = (centres[lab] + rng.standard_normal((150, 4)) * 0.5).astype(np.float32)
+    Y = np.eye(3, dtype=np.float32)[lab]
+    sizes = [4, 16, 3]
+    Ws = [rng.uniform(-1, 1, (sizes[l + 1], sizes[l])).astype(np.float32) * np.float32(np.sqrt(6.0 / (sizes[l] + sizes[l + 1]))) for l in range(2)]
+    return sizes, [po.SIGMOID, po.SOFTMAX], X, Y, Ws
+
+
+@pytest.mark.parametrize("path", ["one_workgroup", "launches"])
+def test_cfg1_as_written_500_epochs_free_running(path):
+    """configs[0] as it is written (softmax + cross-entropy, full batch 150, lr 0.1, momentum 0.9, 500 epochs),
+    which only canonical mode can express: the GPU run and the CPU restatement each take their own 500 steps from
+    the same start, nothing is re-seeded on the way.  Every epoch's loss within 1e-4 relative, every epoch's count
+    of correct rows equal, final logits within 1e-4 of their scale with the same class on every row, final
+    parameters within 1e-4.  As one persistent workgroup the 500 epochs are ONE launch."""
+    import pyglades as pg
+    print("cfg1 as written, 500 epochs,", path, flush=True)
+    sizes, acts, X, Y, Ws = _cfg1_as_written()
+    kw = dict(lr=0.1, mom=0.9, cost=po.CLASSIFICATION)
+    o = po.CanonNet(po.make_spec(sizes, acts, **kw))
+    g = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_CANONICAL, dtype=pg.F32, **kw))
+    for l in range(2):
+        o.set_params(l, Ws[l]); g.set_params(l, Ws[l])
+    g.set_canonical_path(pg.CANON_PATH_ONE_WORKGROUP if path == "one_workgroup" else pg.CANON_PATH_LAUNCHES)
+    g.set_dataset(X, Y)
+    got = g.run_epochs_canonical(150, 500)
+    assert len(got) == 500
+    worst = 0.0
+    for e in range(500):
+        mo = o.step(X, Y)
+        worst = max(worst, abs(got[e][0] - mo.loss) / abs(mo.loss))
+        assert abs(got[e][0] - mo.loss) <= 1e-4 * abs(mo.loss), (e, got[e][0], mo.loss)
+        assert got[e][2] == mo.correct, (e, got[e][2], mo.correct)
+    print("first / last loss %.5f / %.5f, correct %d of 150, worst relative loss gap of an epoch %.2e" % (got[0][0], got[-1][0], got[-1][2], worst), flush=True)
+    assert got[-1][0] < 0.2 * got[0][0] and got[-1][2] >= 145       # it has learnt the clusters
+    lo, lg = o.forward(X), g.forward(X)
+    np.testing.assert_allclose(lg, lo, rtol=1e-4, atol=1e-4 * np.abs(lo).max())
+    assert np.array_equal(lg.argmax(1), lo.argmax(1))
+    for l in range(2):
+        np.testing.assert_allclose(g.get_params(l)[0], o.get_params(l)[0], rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(g.get_params(l)[1], o.get_params(l)[1], rtol=1e-4, atol=1e-5)
+    g.close()
+
+
+def _cfg2_table(seed=1234, N=10000):
+    """BASELINE configs[1]: windows of 32 lagged values of a sum of 3 sines (random frequency and phase) plus
+    N(0, 0.05) noise, the next value as target."""
+    rng = np.random.default_rng(seed)
+    t = np.arange(N + 32, dtype=np.float64)
+    f, ph = rng.random(3) * 0.05 + 0.01, rng.random(3) * 6.28
+    sig = sum(np.sin(2 * np.pi * f[k] * t + ph[k]) for k in range(3)) + rng.standard_normal(N + 32) * 0.05
+    X = np.stack([sig[i:i + 32] for i in range(N)]).astype(np.float32)
+    Y = sig[32:32 + N, None].astype(np.float32)
+    sizes = [32, 64, 64, 1]
+    Ws = [rng.uniform(-1, 1, (sizes[l + 1], sizes[l])).astype(np.float32) * np.float32(np.sqrt(6.0 / (sizes[l] + sizes[l + 1]))) for l in range(3)]
+    return sizes, [po.TANH, po.TANH, po.LINEAR], [0, 0, 1.0], X, Y, Ws
+
+
+@pytest.mark.parametrize("path", ["one_workgroup", "launches"])
+def test_cfg2_canonical_50_epochs_free_running(path):
+    """configs[1] in canonical mode (32-64-64-1 tanh / tanh / linear, MSE, minibatch 256, lr 0.01, momentum 0.9,
+    50 epochs of 40 steps on 10 000 windows), free-running against the CPU restatement: every epoch's loss within
+    1e-4 relative, final predictions within 1e-4 of their scale."""
+    import pyglades as pg
+    print("cfg2 canonical, 50 epochs,", path, flush=True)
+    sizes, acts, params, X, Y, Ws = _cfg2_table()
+    kw = dict(lr=0.01, mom=0.9, act_params=params, cost=po.REGRESSION)
+    o = po.CanonNet(po.make_spec(sizes, acts, **kw))
+    g = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_CANONICAL, dtype=pg.F32, **kw))
+    for l in range(3):
+        o.set_params(l, Ws[l]); g.set_params(l, Ws[l])
+    g.set_canonical_path(pg.CANON_PATH_ONE_WORKGROUP if path == "one_workgroup" else pg.CANON_PATH_LAUNCHES)
+    g.set_dataset(X, Y)
+    po.lib().go_set_threads(8)
+    N, B = X.shape[0], 256
+    got = g.run_epochs_canonical(B, 50)
+    assert len(got) == 50
+    worst = 0.0
+    for e in range(50):
+        loss = 0.0
+        for r0 in range(0, N, B):
+            n = min(B, N - r0)
+            loss += o.step(X[r0:r0 + n], Y[r0:r0 + n]).loss * n
+        loss /= N
+        worst = max(worst, abs(got[e][0] - loss) / loss)
+        assert abs(got[e][0] - loss) <= 1e-4 * loss, (e, got[e][0], loss)
+    print("first / last epoch loss %.5f / %.5f, worst relative gap of an epoch %.2e" % (got[0][0], got[-1][0], worst), flush=True)
+    assert got[-1][0] < 0.1 * got[0][0]
+    po_out, pg_out = o.forward(X[:2048]), g.forward(X[:2048])
+    np.testing.assert_allclose(pg_out, po_out, rtol=1e-4, atol=1e-4 * np.abs(po_out).max())
+    g.close()
+
+
+def test_one_workgroup_epochs_in_one_launch():
+    """The persistent kernel's epoch loop: n epochs in one launch leave bit for bit the parameters, momentum and
+    per-epoch figures of n launches of one epoch; the accuracy stop ends the launch at the epoch that reaches it;
+    an evaluation pass changes nothing and its figures are those of the launches path; the confusion counters of
+    the last epoch equal the launches path's."""
+    import pyglades as pg
+    sizes, acts = [10, 24, 12, 4], [po.RELU, po.TANH, po.SOFTMAX]
+    nets = []
+    for _ in range(3):
+        _, g, rng = build_pair(sizes, acts, [0, 0, 0], po.CLASSIFICATION, 0.05, 0.9, 1e-4, 1e-3, 31, path="one_workgroup")
+        nets.append(g)
+    a, b, c = nets
+    c.set_canonical_path(pg.CANON_PATH_LAUNCHES)
+    N, B = 333, 50
+    X = rng.standard_normal((N, sizes[0])).astype(np.float32)
+    T = rng.standard_normal((sizes[0], sizes[-1])).astype(np.float32)
+    Y = np.eye(sizes[-1], dtype=np.float32)[(X @ T).argmax(1)]
+    for g in nets:
+        g.set_dataset(X, Y)
+        g.confusion_enable(True)
+    many = a.run_epochs_canonical(B, 12)
+    single = [b.run_epochs_canonical(B, 1)[0] for _ in range(12)]
+    launches = c.run_epochs_canonical(B, 12)
+    assert many == single
+    for l in range(3):
+        assert np.array_equal(a.get_params(l)[0], b.get_params(l)[0]) and np.array_equal(a.get_params(l)[1], b.get_params(l)[1])
+        assert np.array_equal(a.get_state(l)[0], b.get_state(l)[0]) and np.array_equal(a.get_state(l)[1], b.get_state(l)[1])
+        np.testing.assert_allclose(a.get_params(l)[0], c.get_params(l)[0], rtol=1e-4, atol=2e-6)
+    for e in range(12):
+        assert abs(many[e][0] - launches[e][0]) <= 1e-4 * abs(launches[e][0]) and abs(many[e][2] - launches[e][2]) <= 1
+    assert many[-1][0] < many[0][0]
+    # confusion counters of the last epoch (they restart at every epoch's head)
+    cm_a, cm_c = a.confusion(), c.confusion()
+    assert cm_a.sum() == N and cm_c.sum() == N and np.abs(cm_a - cm_c).sum() <= 2
+    # evaluation pass: same figures both ways, parameters untouched
+    W_before = a.get_params(0)[0].copy()
+    ev_a, ev_c = a.run_epochs_canonical(B, 1, train=False)[0], c.run_epochs_canonical(B, 1, train=False)[0]
+    assert abs(ev_a[0] - ev_c[0]) <= 1e-4 * abs(ev_c[0]) and abs(ev_a[2] - ev_c[2]) <= 1
+    assert np.array_equal(a.get_params(0)[0], W_before)
+    # accuracy stop: the epoch that reaches the bar is the last one run
+    bar = many[5][1]
+    _, d, _ = build_pair(sizes, acts, [0, 0, 0], po.CLASSIFICATION, 0.05, 0.9, 1e-4, 1e-3, 31, path="one_workgroup")
+    d.set_dataset(X, Y)
+    stopped = d.run_epochs_canonical(B, 12, stop_accuracy=float(bar))
+    first = next(e for e in range(12) if many[e][1] >= bar)
+    assert len(stopped) == first + 1 and stopped == many[:first + 1]
+    for g in nets + [d]:
+        g.close()
