@@ -105,6 +105,7 @@ __global__ void __launch_bounds__(1024) canon_narrow_kernel(CanonNarrowArgs p)
             for (int c0 = 0; c0 < bcount; c0 += RC) {
                 const int rc = bcount - c0 < RC ? bcount - c0 : RC;
                 const long long row0 = r0 + c0;
+                const int in_row0 = resident ? (int)row0 : 0;   // where the chunk's inputs start in the staged rows
                 // ---- the chunk's rows (the table is read as it lies: consecutive lanes, consecutive floats)
                 if (!resident) {
                     stage_rows(row0, rc);
@@ -115,7 +116,7 @@ __global__ void __launch_bounds__(1024) canon_narrow_kernel(CanonNarrowArgs p)
                     const int ni = p.sizes[l], no = p.sizes[l + 1];
                     const float* Wl = lds + p.offW[l];
                     const float* Bl = lds + p.offB[l];
-                    const float* ar = lds + p.offA[l] + tr * p.pitchA[l];
+                    const float* ar = lds + p.offA[l] + ((l == 0 ? in_row0 : 0) + tr) * p.pitchA[l];
                     float* Aout = lds + p.offA[l + 1] + tr * p.pitchA[l + 1];
                     const bool raw = softmax && l == L - 1;   // the row function takes softmax's logits
                     const int act = p.act[l]; const float ap = p.act_param[l];
@@ -163,8 +164,8 @@ __global__ void __launch_bounds__(1024) canon_narrow_kernel(CanonNarrowArgs p)
                     for (int l = 0; l < L; ++l) {
                         const int ni = p.sizes[l], no = p.sizes[l + 1];
                         const float* Dn = lds + p.offD[l + 1];
-                        const float* Al = lds + p.offA[l];
                         const int pa = p.pitchA[l], pd = p.pitchA[l + 1];
+                        const float* Al = lds + p.offA[l] + (l == 0 ? in_row0 : 0) * pa;
                         float* G = lds + p.offG[l];
                         float* GB = lds + p.offGB[l];
                         if (p.wave_per_weight) {

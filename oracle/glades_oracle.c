@@ -493,6 +493,10 @@ void go_dropout_draw(const go_spec* s, const float* p, int64_t N, uint8_t* masks
 
 static int g_threads = 1;
 void go_set_threads(int t) { g_threads = t > 0 ? t : 1; }
+/* canonical mode only: walk every sum (a unit's inputs, a unit's outputs, a weight's batch rows) from the far end.
+   Same mathematics, another order of fp32 addition: what a second implementation may legitimately differ by. */
+static int g_reverse = 0;
+void go_set_sum_order(int reversed) { g_reverse = reversed ? 1 : 0; }
 
 struct go_canon {
     go_spec s;
@@ -588,7 +592,8 @@ static void canon_layer_forward(const float* W, const float* bias, const float* 
             float acc[TB];
             for (int t = 0; t < TB; ++t) acc[t] = 0.0f;
             const float* w = W + (size_t)o * ni;
-            for (int i = 0; i < ni; ++i) {
+            for (int i0 = 0; i0 < ni; ++i0) {
+                const int i = g_reverse ? ni - 1 - i0 : i0;
                 const float wi = w[i];
                 const float* at = At + (size_t)i * TB;
                 for (int t = 0; t < TB; ++t) { float pr = wi * at[t]; acc[t] += pr; }
@@ -698,7 +703,8 @@ static void canon_dgrad(const float* W, const float* D, float* E, int64_t B, int
     for (int64_t b = 0; b < B; ++b) {
         float* e = E + b * ni;
         for (int i = 0; i < ni; ++i) e[i] = 0.0f;
-        for (int o = 0; o < no; ++o) {
+        for (int o0 = 0; o0 < no; ++o0) {
+            const int o = g_reverse ? no - 1 - o0 : o0;
             const float dv = D[b * no + o];
             const float* w = W + (size_t)o * ni;
             for (int i = 0; i < ni; ++i) { float pr = dv * w[i]; e[i] += pr; }
@@ -716,7 +722,8 @@ static void canon_wgrad(const float* D, const float* A, float* G, float* gb, int
         float* g = G + (size_t)o * ni;
         for (int i = 0; i < ni; ++i) g[i] = 0.0f;
         float sb = 0.0f;
-        for (int64_t b = 0; b < B; ++b) {
+        for (int64_t b0 = 0; b0 < B; ++b0) {
+            const int64_t b = g_reverse ? B - 1 - b0 : b0;
             const float dv = D[b * no + o];
             const float* a = A + b * ni;
             for (int i = 0; i < ni; ++i) { float pr = dv * a[i]; g[i] += pr; }

@@ -151,6 +151,8 @@ void  go_canon_get_grads(const go_canon* n, int layer, float* gW, float* gb);
 /* mean per-sample loss of a batch without touching parameters */
 double go_canon_loss(go_canon* n, const float* X, const float* Y, int64_t B);
 void  go_set_threads(int t);
+/* canonical mode: 1 = every sum is walked from its far end (same mathematics, another order of fp32 addition) */
+void  go_set_sum_order(int reversed);
 
 /* ---- low-precision formats ---- */
 uint16_t go_bf16_from_f32(float x);           /* round-to-nearest-even, NaN kept quiet */

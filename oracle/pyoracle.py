@@ -95,6 +95,7 @@ def lib():
             "go_canon_step": (None, [vp, f32p, f32p, C.c_int64, C.POINTER(Metrics)]),
             "go_canon_loss": (C.c_double, [vp, f32p, f32p, C.c_int64]),
             "go_set_threads": (None, [C.c_int]),
+            "go_set_sum_order": (None, [C.c_int]),
             "go_bf16_from_f32": (C.c_uint16, [C.c_float]),
             "go_bf16_to_f32": (C.c_float, [C.c_uint16]),
             "go_e4m3_from_f32": (C.c_uint8, [C.c_float]),

@@ -604,16 +604,21 @@ def test_bf16_training_top1_on_separable_classes():
 
 def test_cfg4_full_size_training_bf16_against_fp32():
     """The wide benchmark network at its full size -- 4096-4096-4096-4096-4096-1024, batch 8192, both
-    tile sizes and the transposed-table operand in every step -- trained 32 steps in bf16 and, side by
-    side, in fp32 on the GPU (the fp32 path is pinned to the CPU restatement in test_gpu_canonical.py):
-    loss within 2e-2 relative at every step, and the trained networks agree on the class of >= 99.5 %
-    of 8192 held-out rows, all rows counted.  1024 separable classes (Gaussian clusters)."""
+    tile sizes and the transposed-table operand in every step -- trained its whole schedule of 200 steps in
+    bf16 and, side by side, in fp32 on the GPU (the fp32 path is pinned to the CPU restatement in
+    test_gpu_canonical.py): loss within 2e-2 relative at every step (measured: 1e-3 at worst, while the loss
+    falls from 8.0 to 0.05), and the trained networks agree on the class of >= 99.5 % of 8192 held-out rows, all
+    rows counted.  1024 separable classes (Gaussian clusters), 8 batches of 8192 rows walked 25 times, learning
+    rate 0.002 with momentum 0.9 (at 0.02 the loss is below 0.03 after 30 steps and two runs' losses, both next
+    to nothing, are several per cent of each other apart: a comparison of noise)."""
     import pyglades as pg
     print("cfg4 at full size: bf16 vs fp32 training", flush=True)
     sizes = [4096, 4096, 4096, 4096, 4096, 1024]
-    (f, b), hist, draw = _trained_pair(sizes, 8192, 4, 32, 0.02, 23, [pg.F32, pg.BF16])
+    (f, b), hist, draw = _trained_pair(sizes, 8192, 8, 200, 0.002, 23, [pg.F32, pg.BF16])
     worst = 0.0
     for s, (mf, mb) in enumerate(hist):
+        if s % 20 == 0 or s == len(hist) - 1:
+            print("step %d loss fp32 %.6f bf16 %.6f" % (s, mf.loss, mb.loss), flush=True)
         worst = max(worst, abs(mb.loss - mf.loss) / abs(mf.loss))
         assert abs(mb.loss - mf.loss) <= 2e-2 * abs(mf.loss), (s, mb.loss, mf.loss)
     assert hist[-1][0].loss < 0.2 * hist[0][0].loss                     # the schedule does train

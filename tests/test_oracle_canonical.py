@@ -121,3 +121,42 @@ def test_forward_equals_exact_mode_forward():
         ca.set_params(l, Ws[l], np.full(sizes[l + 1], sb[l], np.float32))
     _, preds = ex.epoch(X, Y, train=False)
     assert bits_equal(ca.forward(X), preds)
+
+
+def test_cfg3_schedule_two_summation_orders_part_ways():
+    """BASELINE configs[2]'s schedule (784-1024-1024-10 ReLU / softmax, batch 512, lr 0.05, momentum 0.9, L2 1e-4 on
+    its own data) is not stable enough for two correct fp32 implementations to stay within 1e-4 of each other: the
+    restatement run twice from one start, once with every sum walked from its other end (same products, same
+    formulas, another order of fp32 addition), agrees to 1e-6 over the first steps and is more than 1e-4 apart in
+    the loss of some step before step 24.  That is why the GPU test of this schedule re-seeds the GPU network from
+    the CPU run's state before every step instead of comparing two free runs after 585 steps."""
+    rng = np.random.default_rng(1234)
+    sizes, acts = [784, 1024, 1024, 10], [po.RELU, po.RELU, po.SOFTMAX]
+    B, steps = 512, 24
+    X = rng.random((60000, 784), dtype=np.float32)
+    T1 = rng.standard_normal((784, 256), dtype=np.float32) / np.float32(28.0)
+    T2 = rng.standard_normal((256, 10), dtype=np.float32) / np.float32(16.0)
+    Hc = X @ T1
+    Hc -= Hc.mean(0)
+    Y = np.eye(10, dtype=np.float32)[(np.maximum(Hc, 0) @ T2).argmax(1)]
+    X, Y = X[:B * steps], Y[:B * steps]
+    Ws = [rng.standard_normal((sizes[l + 1], sizes[l]), dtype=np.float32) * np.float32(np.sqrt(2.0 / sizes[l])) for l in range(3)]
+    kw = dict(lr=0.05, mom=0.9, wd2=1e-4, cost=po.CLASSIFICATION)
+    a, b = po.CanonNet(po.make_spec(sizes, acts, **kw)), po.CanonNet(po.make_spec(sizes, acts, **kw))
+    for l in range(3):
+        a.set_params(l, Ws[l]); b.set_params(l, Ws[l])
+    po.lib().go_set_threads(8)
+    gaps = []
+    try:
+        for s in range(steps):
+            po.lib().go_set_sum_order(0)
+            ma = a.step(X[s * B:(s + 1) * B], Y[s * B:(s + 1) * B])
+            po.lib().go_set_sum_order(1)
+            mb = b.step(X[s * B:(s + 1) * B], Y[s * B:(s + 1) * B])
+            gaps.append(abs(ma.loss - mb.loss) / ma.loss)
+    finally:
+        po.lib().go_set_sum_order(0)
+        po.lib().go_set_threads(1)
+    print("relative loss gap per step:", " ".join("%.1e" % g for g in gaps))
+    assert max(gaps[:4]) < 1e-6        # the same run to begin with
+    assert max(gaps[10:]) > 1e-4       # and two different ones a dozen steps later
