@@ -1547,6 +1547,10 @@ int ghip_forward_noalloc(const ghip_net_spec* spec, const float* const* dev_W, c
     const int L = spec->n_layers;
     for (int l = 0; l < L; ++l)
         if (!dev_W[l] || !dev_bias[l]) return fail(GHIP_EINVAL, "layer %d: weights or biases are NULL", l);
+    // the kernels' 16-byte accesses: a pointer off that grid would quietly take the slow variants
+    bool aligned = (((uintptr_t)dev_X | (uintptr_t)dev_out) % 16) == 0;
+    for (int l = 0; l < L; ++l) aligned = aligned && (((uintptr_t)dev_W[l] | (uintptr_t)dev_bias[l]) % 16) == 0;
+    if (!aligned) return fail(GHIP_EINVAL, "ghip_forward_noalloc takes 16-byte aligned device pointers");
     for (int l = 1; l < L; ++l)
         if ((int64_t)batch * spec->sizes[l] > (int64_t)GHIP_NOALLOC_MAX_ACTIVATIONS)
             return fail(GHIP_EINVAL, "batch %d x hidden layer %d of %d units = %lld activations: the fixed scratch of this entry point "

@@ -30,6 +30,8 @@
 
 #include "ghip_internal.h"
 
+#include <mutex>
+
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -312,15 +314,15 @@ hipError_t ghip_gemm_f32_group(const GemmF32Args* a, int count, hipStream_t s)
      {gemm_f32_group_kernel<F, true, false, BMV>, gemm_f32_group_kernel<F, true, true, BMV>}}
     static const kernel_t table[2][2][2][2] = {{GF32_ROW(false, 64), GF32_ROW(true, 64)}, {GF32_ROW(false, 32), GF32_ROW(true, 32)}};
 #undef GF32_ROW
-    static bool raised = false;
-    if (!raised) {
-        for (int i = 0; i < 16; ++i) {
-            hipError_t e = hipFuncSetAttribute((const void*)table[i >> 3][(i >> 2) & 1][(i >> 1) & 1][i & 1],
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
-            if (e != hipSuccess) return e;
-        }
-        raised = true;
-    }
+    // once per process, whichever thread comes first (handles on several host threads launch side by side)
+    static std::once_flag once;
+    static hipError_t raised = hipSuccess;
+    std::call_once(once, [] {
+        for (int i = 0; i < 16 && raised == hipSuccess; ++i)
+            raised = hipFuncSetAttribute((const void*)table[i >> 3][(i >> 2) & 1][(i >> 1) & 1][i & 1],
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    });
+    if (raised != hipSuccess) return raised;
     hipLaunchKernelGGL(table[v0.bm == 32][v0.fast][v0.akm ? 1 : 0][v0.bkm ? 1 : 0], dim3(blocks), dim3(NTHR), kLdsBytes, s, grp);
     return hipGetLastError();
 }
@@ -335,15 +337,15 @@ hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s)
      {gemm_f32_kernel<F, true, false, BMV>, gemm_f32_kernel<F, true, true, BMV>}}
     static const kernel_t table[2][2][2][2] = {{GF32_ROW(false, 64), GF32_ROW(true, 64)}, {GF32_ROW(false, 32), GF32_ROW(true, 32)}};
 #undef GF32_ROW
-    static bool raised = false;
-    if (!raised) {
-        for (int i = 0; i < 16; ++i) {
-            hipError_t e = hipFuncSetAttribute((const void*)table[i >> 3][(i >> 2) & 1][(i >> 1) & 1][i & 1],
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
-            if (e != hipSuccess) return e;
-        }
-        raised = true;
-    }
+    // once per process, whichever thread comes first (handles on several host threads launch side by side)
+    static std::once_flag once;
+    static hipError_t raised = hipSuccess;
+    std::call_once(once, [] {
+        for (int i = 0; i < 16 && raised == hipSuccess; ++i)
+            raised = hipFuncSetAttribute((const void*)table[i >> 3][(i >> 2) & 1][(i >> 1) & 1][i & 1],
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsBytes);
+    });
+    if (raised != hipSuccess) return raised;
     hipLaunchKernelGGL(table[v.bm == 32][v.fast][v.akm ? 1 : 0][v.bkm ? 1 : 0], v.grid, dim3(NTHR), kLdsBytes, s, a);
     return hipGetLastError();
 }

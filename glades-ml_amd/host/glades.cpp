@@ -437,7 +437,7 @@ NNetwork::NNetwork()
     : di(NULL), skeleton(NULL), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
       dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
-      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false), prepaidDrawEpochs(0)
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false), prepaidDrawEpochs(0), randFidelity(true)
 {
 }
 
@@ -445,7 +445,7 @@ NNetwork::NNetwork(NNInfo* newNNInfo)
     : di(NULL), skeleton(newNNInfo), dev(NULL), running(false), netType(TYPE_DFF), epochs(0), mode(MODE_EXACT),
       dtype(DTYPE_F32), biasMode(0), verbose(true), overallTotalError(0.0f), overallTotalAccuracy(0.0f), overallClassAccuracy(0.0f), overallClassPrecision(0.0f),
       overallClassRecall(0.0f), overallClassSpecificity(0.0f), overallClassF1(0.0f), overallCorrect(0),
-      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false), prepaidDrawEpochs(0)
+      minibatchSize(1), id(g_next_id++), nRows(0), nFeat(0), nOut(0), dropoutOn(false), prepaidDrawEpochs(0), randFidelity(true)
 {
 }
 
@@ -726,7 +726,7 @@ size_t NNetwork::dropoutDrawsPerEpoch() const
 
 void NNetwork::skipDropoutDraws(int64_t n)
 {
-    if (dropoutOn || n <= 0) return;  // with dropout the flags themselves are drawn (drawDropout)
+    if (dropoutOn || n <= 0 || !randFidelity) return;  // with dropout the flags themselves are drawn (drawDropout)
     const int64_t paid = prepaidDrawEpochs < n ? prepaidDrawEpochs : n;
     prepaidDrawEpochs -= paid;
     const size_t per = dropoutDrawsPerEpoch();
@@ -736,7 +736,7 @@ void NNetwork::skipDropoutDraws(int64_t n)
 
 void NNetwork::prepayDropoutDraws(int64_t n)
 {
-    if (dropoutOn || n <= 0) return;
+    if (dropoutOn || n <= 0 || !randFidelity) return;
     const size_t per = dropoutDrawsPerEpoch();
     for (int64_t e = 0; e < n; ++e)
         for (size_t k = 0; k < per; ++k) (void)rand();
@@ -789,8 +789,19 @@ bool NNetwork::build()
     // reference's order (so libc's rand() moves as it does there) and injected layers replace their draw
     std::vector<std::vector<float> > sampled;
     bool allInjected = true;
-    for (int l = 0; l <= H; ++l)
-        allInjected = allInjected && (size_t)l < initW.size() && initW[l].size() == (size_t)s.sizes[l] * s.sizes[l + 1];
+    for (int l = 0; l <= H; ++l) {
+        const size_t want = (size_t)s.sizes[l] * s.sizes[l + 1];
+        const size_t have = (size_t)l < initW.size() ? initW[l].size() : 0;
+        // a layer either has no injected weights (it is sampled: samplesOnBuild() tells the same story before
+        // the sizes are known) or has all of them
+        if (have != 0 && have != want) {
+            char msg[160];
+            snprintf(msg, sizeof(msg), "weight layer %d was given %zu weights, it has %zu", l, have, want);
+            lastError = msg;
+            return false;
+        }
+        allInjected = allInjected && have == want;
+    }
     if (!allInjected && !sampleInitialWeights(skeleton, (int)nFeat, (int)nOut, sampled, &lastError)) return false;
     if (ghip_net_create(&s, &dev) != 0) { lastError = ghip_last_error(); dev = NULL; return false; }
     for (int l = 0; l <= H; ++l) {
@@ -1245,8 +1256,15 @@ void NNetwork::run(DataInput* newDataInput, int runType)
                 drawDropout();
                 if (ghip_net_set_dropout_masks(dev, dropFlags.data(), 1) != 0) { lastError = ghip_last_error(); break; }
             }
-            if (ghip_net_run_epochs_exact(dev, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran,
-                                          want_preds ? preds.data() : NULL) != 0) {
+            // the darts of a run without dropout: on a second thread while the device runs, where every epoch of the
+            // chunk is certain to run (the accuracy condition is the only one looked at inside a launch)
+            std::thread payer;
+            if (!dropoutOn && randFidelity && terminator.getAccuracy() <= 0.0f && prepaidDrawEpochs == 0)
+                payer = std::thread([this, chunk] { prepayDropoutDraws(chunk); });
+            const int rc = ghip_net_run_epochs_exact(dev, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran,
+                                                     want_preds ? preds.data() : NULL);
+            if (payer.joinable()) payer.join();
+            if (rc != 0) {
                 lastError = ghip_last_error();
                 break;
             }
@@ -1255,17 +1273,21 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             for (int e = 0; e < ran; ++e) learningCurve.push_back(ms[e].accuracy);
             afterEpochs(&ms[ran - 1], ran, runType);
         } else {
-            if (confusionMatrix.size() > 0) ghip_net_confusion_reset(dev);  // network.cpp:183-185
-            // canonical mode: batches [k*mb, (k+1)*mb), the last one averaged over its true size
+            // canonical mode: batches [k*mb, (k+1)*mb), the last one averaged over its true size; the confusion
+            // counters restart at the head of every epoch (network.cpp:183-185).  Several epochs per call where the
+            // stop conditions allow it: a narrow network then runs them as one launch, any other pass by pass with
+            // every step of a pass enqueued back to back and the metrics added up on the device.
             const int mb = minibatchSize > 0 ? minibatchSize : (int)nRows;
-            // every step of the pass is enqueued back to back; the device adds up the metrics
-            ghip_metrics last;
-            if (ghip_net_run_epoch_canonical(dev, mb, runType == RUN_TRAIN ? 1 : 0, &last) != 0) {
+            const int chunk = epochChunk(terminator, epochs, runType);
+            std::vector<ghip_metrics> ms(chunk);
+            int ran = 0;
+            if (ghip_net_run_epochs_canonical(dev, mb, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran) != 0) {
                 lastError = ghip_last_error();
                 break;
             }
-            learningCurve.push_back(last.accuracy);
-            afterEpochs(&last, 1, runType);
+            if (ran <= 0) break;
+            for (int e = 0; e < ran; ++e) learningCurve.push_back(ms[e].accuracy);
+            afterEpochs(&ms[ran - 1], ran, runType);
         }
         if (terminator.triggered(time(NULL), epochs, overallTotalAccuracy)) break;
         if (runType == RUN_TEST) break;

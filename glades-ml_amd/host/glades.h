@@ -368,6 +368,7 @@ class NNetwork
     // where no dart can drop anything (layer.cpp:102-134): a run without dropout still moves libc's
     // rand() by that many draws per epoch, which the next network's weight sampler then starts from
     int64_t prepaidDrawEpochs;                       // epochs whose draws have been taken ahead of the run
+    bool randFidelity;                               // take those draws at all (setRandStreamFidelity)
     size_t dropoutDrawsPerEpoch() const;
     void skipDropoutDraws(int64_t epochs);           // exact mode, no flags: take the draws and throw them away
     void prepayDropoutDraws(int64_t epochs);
@@ -429,6 +430,13 @@ public:
     const CMatrix& getConfusionMatrix() const { return confusionMatrix; }
     void setMode(int newMode, int newDtype = DTYPE_F32) { mode = newMode; dtype = newDtype; }
     void setSequentialBias(bool faithful) { biasMode = faithful ? 0 : 1; }
+    // A run without dropout still moves libc's rand() by one draw per node and row and epoch, as the reference's
+    // does (layer.cpp:102-134), so that whatever draws from rand() next (another network's weight sampler, the
+    // caller) finds the stream where the reference leaves it.  That is tens of millions of libc calls per epoch
+    // for a table of cfg2's size; they are made on a second host thread while the device runs the epochs where
+    // the number of epochs is known ahead (no accuracy condition), after the launch otherwise.  A caller who
+    // never reads rand() again may turn them off.
+    void setRandStreamFidelity(bool faithful) { randFidelity = faithful; }
     void setVerbose(bool v) { verbose = v; }  // the per-epoch progress line and the [NN] banners
     // layer = weight layer 0..numHiddenLayers(); W is [n_out][n_in] row-major
     bool setWeights(unsigned int layer, const std::vector<float>& W);

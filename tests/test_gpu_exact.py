@@ -319,3 +319,103 @@ def test_many_networks_in_one_launch_equal_their_solo_runs():
         pg.run_epochs_exact_multi([group[0], group[0]], 1)
     for n in solo + group + fresh:
         n.close()
+
+
+# Which kernel a launch runs follows from the network and the launch (ghip_launch_exact): one case per
+# instantiation, named for it, each bit for bit against the CPU restatement.
+#   exact_wave_kernel<layers 2|3, wavefronts per SIMD 2|4>: two or three weight layers, no layer wider than 64, no
+#       dropout state; the 4-per-SIMD build when one launch carries more than 2048 networks
+#   exact_kernel<state in LDS, dropout, layers 2|3|any, at most 64|1024 threads>: everything else
+INSTANTIATIONS = [
+    # name,                                sizes,              mb, dropout, networks in the launch
+    ("wave_2_layers",                      [5, 7, 3],           3, False, 1),
+    ("wave_3_layers",                      [6, 9, 5, 2],        1, False, 1),
+    ("wave_2_layers_crowded",              [3, 4, 2],           2, False, 2060),
+    ("wave_3_layers_crowded",              [3, 4, 3, 2],        4, False, 2060),
+    ("general_2_layers_64_threads_drop",   [6, 8, 2],           3, True, 1),
+    ("general_3_layers_64_threads_drop",   [5, 7, 6, 4],        2, True, 1),
+    ("general_2_layers_wide",              [70, 100, 3],        4, False, 1),
+    ("general_3_layers_wide",              [20, 80, 66, 2],     1, False, 1),
+    ("general_3_layers_wide_drop",         [20, 80, 66, 2],     3, True, 1),
+    ("general_1_layer",                    [9, 4],              2, False, 1),
+    ("general_4_layers",                   [8, 7, 6, 5, 3],     3, False, 1),
+    ("general_4_layers_drop",              [8, 7, 6, 5, 3],     1, True, 1),
+]
+
+
+@pytest.mark.parametrize("name,sizes,mb,drop,count", INSTANTIATIONS, ids=[c[0] for c in INSTANTIATIONS])
+def test_each_kernel_instantiation(name, sizes, mb, drop, count):
+    import pyglades as pg
+    print("instantiation", name, flush=True)
+    rng = np.random.default_rng(sum(map(ord, name)))
+    nl, N, E = len(sizes) - 1, 11, 3
+    acts = [po.TANH, po.SIGMOID, po.RELU, po.LEAKY][:nl - 1] + [po.SIGMOID]
+    kw = dict(lr=0.01, mom=0.5, wd1=1e-3, wd2=1e-3, act_params=[0.0, 0.0, 0.0, 0.05][:nl - 1] + [0.0], batch=mb, cost=po.CLASSIFICATION)
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (0.6 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(nl)]
+    bs = [float(np.float32(rng.normal(0, 0.1))) for _ in range(nl)]
+    X = rng.random((N, sizes[0])).astype(np.float32)
+    Y = (rng.random((N, sizes[-1])) * 0.98 + 0.01).astype(np.float32)
+    masks = None
+    if drop:   # a third of the nodes of every input and hidden layer, never a whole layer of a row
+        masks = (rng.random((E, N, sum(sizes[:-1]))) < 0.33).astype(np.uint8)
+        off = 0
+        for l in range(nl):
+            masks[:, :, off] = 0
+            off += sizes[l]
+    o = po.ExactNet(po.make_spec(sizes, acts, **kw))
+    for l in range(nl):
+        o.set_weights(l, Ws[l]); o.set_bias(l, bs[l])
+    om = [o.epoch(X, Y, masks=None if masks is None else masks[e]) for e in range(E)]
+    nets = []
+    for _ in range(min(count, 3) if count > 1 else 1):   # of a crowded launch the first three are compared ...
+        n = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_EXACT, **kw))
+        for l in range(nl):
+            n.set_params(l, Ws[l], bs[l])
+        n.set_dataset(X, Y)
+        nets.append(n)
+    if count > 1:
+        fill = []
+        for _ in range(count - len(nets)):                # ... the others only fill the launch
+            n = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_EXACT, **kw))
+            for l in range(nl):
+                n.set_params(l, Ws[l], bs[l])
+            n.set_dataset(X, Y)
+            fill.append(n)
+        got = pg.run_epochs_exact_multi(nets + fill, E)
+        ms_all = got[:len(nets)]
+        preds = None
+    else:
+        fill = []
+        if drop:
+            nets[0].set_dropout_masks(masks)
+        ms, preds = nets[0].run_epochs_exact(E, want_preds=True)
+        ms_all = [ms]
+    for ms in ms_all:
+        assert bits_equal([m[0] for m in ms], [m.loss for m, _ in om])
+        assert bits_equal([m[1] for m in ms], [m.accuracy for m, _ in om])
+        assert [m[2] for m in ms] == [m.correct for m, _ in om]
+    if preds is not None:
+        assert bits_equal(preds, om[-1][1])
+    for n in nets:
+        for l in range(nl):
+            W, b = n.get_params(l)
+            assert bits_equal(W, o.get_weights(l)), l
+            assert bits_equal(np.float32(b), o.get_bias(l)), l
+            if not drop:
+                sa, sb = n.get_state(l)
+                wa, wb = o.get_window(l)
+                assert bits_equal(sa, wa) and bits_equal(sb, wb), l
+    # the accuracy stop inside the launch: the first epoch at or above the bar is the last one run
+    # (wide layers overflow the reference's doubling accumulator to NaN within an epoch, bit for bit here too: no bar to reach)
+    if count == 1 and not drop and np.isfinite([m[1] for m in ms_all[0]]).all():
+        acc = [m[1] for m in ms_all[0]]
+        n2 = pg.Net(pg.make_spec(sizes, acts, mode=pg.MODE_EXACT, **kw))
+        for l in range(nl):
+            n2.set_params(l, Ws[l], bs[l])
+        n2.set_dataset(X, Y)
+        bar = float(acc[1])
+        stopped, _ = n2.run_epochs_exact(E, stop_accuracy=bar)
+        assert len(stopped) == next(e for e in range(E) if acc[e] >= bar) + 1
+        n2.close()
+    for n in nets + fill:
+        n.close()

@@ -24,7 +24,17 @@ def hip():
         _hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
         _hip.hipFree.argtypes = [C.c_void_p]
         _hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        _hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+        _hip.hipStreamCreate.argtypes = [C.POINTER(C.c_void_p)]
+        _hip.hipStreamSynchronize.argtypes = [C.c_void_p]
+        _hip.hipStreamDestroy.argtypes = [C.c_void_p]
     return _hip
+
+
+def free_device_bytes():
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip().hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
 
 
 class DeviceArray:
@@ -120,3 +130,40 @@ def test_noalloc_forward_refuses_what_its_scratch_cannot_hold():
     rc = lib.ghip_forward_noalloc(C.byref(exact), p2, p2, t.ptr, 4, t.ptr, None)
     assert rc == -1
     t.free()
+
+
+def test_noalloc_forward_allocates_nothing_and_takes_a_stream():
+    """What the entry point is for: between two readings of the device's free memory, with the caller's buffers
+    already in place and one warm-up call behind (the first call on a device resolves the scratch array's
+    address and may load code), calls on a stream of the caller's change the free memory by nothing; the result
+    on that stream is the null stream's bit for bit; a pointer off the 16-byte grid is refused."""
+    lib = pg.load()
+    pg._check(lib.ghip_init(0))
+    rng = np.random.default_rng(12)
+    sizes, acts = [64, 256, 128, 10], [pg.RELU, pg.TANH, pg.SOFTMAX]
+    spec, Ws, bs, X = _case(rng, sizes, acts, 300)
+    dW = [DeviceArray(w) for w in Ws]
+    db = [DeviceArray(b) for b in bs]
+    dX = DeviceArray(X)
+    out0 = DeviceArray(shape=(300, 10), fill=np.nan)
+    out1 = DeviceArray(shape=(300, 10), fill=np.nan)
+    pw = (C.c_void_p * 3)(*[t.ptr.value for t in dW])
+    pb = (C.c_void_p * 3)(*[t.ptr.value for t in db])
+    stream = C.c_void_p()
+    assert hip().hipStreamCreate(C.byref(stream)) == 0
+    pg._check(lib.ghip_forward_noalloc(C.byref(spec), pw, pb, dX.ptr, 300, out0.ptr, None))      # warm-up, null stream
+    pg._check(lib.ghip_forward_noalloc(C.byref(spec), pw, pb, dX.ptr, 300, out1.ptr, stream))   # warm-up of the stream
+    assert hip().hipStreamSynchronize(stream) == 0 and hip().hipDeviceSynchronize() == 0
+    before = free_device_bytes()
+    for _ in range(5):
+        pg._check(lib.ghip_forward_noalloc(C.byref(spec), pw, pb, dX.ptr, 300, out1.ptr, stream))
+    assert hip().hipStreamSynchronize(stream) == 0
+    after = free_device_bytes()
+    assert after == before, (before, after)
+    assert out1.numpy().tobytes() == out0.numpy().tobytes()
+    # a pointer off the 16-byte grid
+    rc = lib.ghip_forward_noalloc(C.byref(spec), pw, pb, C.c_void_p(dX.ptr.value + 4), 299, out1.ptr, stream)
+    assert rc == -1 and b"aligned" in lib.ghip_last_error()
+    assert hip().hipStreamDestroy(stream) == 0
+    for t in dW + db + [dX, out0, out1]:
+        t.free()
