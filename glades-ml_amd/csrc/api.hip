@@ -158,6 +158,7 @@ struct ghip_net {
     uint16_t* D[GHIP_MAX_LAYERS + 1] = {};
     uint16_t* DT[GHIP_MAX_LAYERS + 1] = {};
     float* csum[GHIP_MAX_LAYERS + 1] = {};  // per-tile-row column sums of D[l] (bias gradient partials)
+    unsigned int* Hmask[GHIP_MAX_LAYERS + 1] = {};  // signs of H[l] where its activation's derivative is a step (ReLU, leaky): a bit per element
     float* logits = nullptr;
     bool shadow_dirty = true;
     // fp8
@@ -388,7 +389,7 @@ void free_batch_buffers(ghip_net* n)
     for (int l = 0; l <= GHIP_MAX_LAYERS; ++l) {
         dfree(n->act[l]); dfree(n->dlt[l]);
         if (l > 0) dfree(n->H[l]);
-        dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]); dfree(n->csum[l]);
+        dfree(n->HT[l]); dfree(n->D[l]); dfree(n->DT[l]); dfree(n->csum[l]); dfree(n->Hmask[l]);
     }
     dfree(n->stageX); dfree(n->logits); dfree(n->narrowPart); dfree(n->narrowMetrics);
     dfree(n->Aq[0]); dfree(n->Aq[1]); dfree(n->ascale[0]); dfree(n->ascale[1]);
@@ -435,6 +436,7 @@ int reserve_batch(ghip_net* n, int batch)
             if (l < L) {
                 TRY(dalloc_zero(n, &n->H[l], (size_t)B * ps[l]));
                 TRY(dalloc_zero(n, &n->HT[l], (size_t)B * ps[l]));
+                if ((s.act[l - 1] == GHIP_RELU || s.act[l - 1] == GHIP_LEAKY)) TRY(dalloc_zero(n, &n->Hmask[l], (size_t)B * ps[l] / 32));
             }
             // the output deltas are written for the units and rows the batch has; the rest of D[L] stays zero
             TRY(dalloc_zero(n, &n->D[l], (size_t)B * ps[l]));
@@ -657,6 +659,7 @@ int forward_bf16(ghip_net* n, const uint16_t* X, int batch, bool for_training = 
         g.act = out_act(s, l, &g.act_param);
         if (l < L - 1) {
             g.epilogue = LP_FWD_ACT; g.out = n->H[l + 1]; g.outT = for_training ? n->HT[l + 1] : nullptr; g.outT_blocked = 1;
+            g.mask_out = for_training ? n->Hmask[l + 1] : nullptr;
             g.n_valid = ps[l + 1] != s.sizes[l + 1] ? s.sizes[l + 1] : 0;
             LAUNCH(n, "gemm_bf16_forward", ghip_gemm_lp(g, n->stream));
         } else {
@@ -698,6 +701,7 @@ int step_bf16(ghip_net* n, int64_t row0, int batch)
             g.A = n->D[l + 1]; g.B = n->WhT[l]; g.M = B; g.N = ni; g.K = no;
             g.ldb = 64; g.kstrideB = (long long)ni * 128;   // W^T is kept K-blocked: [n_out / 64][n_in][64]
             g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.outT_blocked = 1; g.aux = n->H[l]; g.colsum = n->csum[l];
+            g.mask_in = n->Hmask[l];   // where the activation below is a ReLU: its signs as the forward product left them
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1];
             LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));
         }

@@ -189,6 +189,8 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
 
     const int t = threadIdx.x, lane = t & 63, w = t >> 6;
     const int l31 = lane & 31, lh = lane >> 5;
+    constexpr bool kDgrad = (EPI == LP_DGRAD || EPI == LP_DGRAD_MASK);   // back-propagation: derivative from the activations / from their signs
+    constexpr bool kMask = (EPI == LP_DGRAD_MASK);
 
     // ---- walk the tiles in column groups of 8 rows
     const int tiles_m = g.M / TM, tiles_n = g.N / TN;
@@ -313,7 +315,8 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     // epilogue asks for them.  The touch goes out between the B and the A loads of the fill, so the
     // wait that ends a stage (which only needs B) leaves it in flight like the A loads; its result
     // is never used.
-    constexpr bool kTouch = (EPI == LP_WGRAD_SGD || EPI == LP_DGRAD);
+    constexpr bool kTouch = (EPI == LP_WGRAD_SGD || kDgrad);
+    constexpr int MASK_WORDS = MI * NI * 16 / 32;   // a lane's accumulators, one bit each
     constexpr int PF_ES = (EPI == LP_WGRAD_SGD) ? 4 : 2;         // bytes per element of the touched arrays
     constexpr int PF_ARRAYS = (EPI == LP_WGRAD_SGD) ? 2 : 1;
     constexpr int PF_LPR = TN * PF_ES / 128;                     // lines per tile row
@@ -331,9 +334,11 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
         i = i < 0 ? 0 : (i >= PF_N ? PF_N - 1 : i);  // outside the window: repeat a touched line
         const int line = (i * 8 + ws) * PF_LANES + (lane & (PF_LANES - 1));
         const int within = line % PF_PER;
-        const unsigned char* base = (EPI == LP_DGRAD) ? (const unsigned char*)g.aux
+        const unsigned char* base = kDgrad ? (const unsigned char*)g.aux
                                   : (line < PF_PER) ? (const unsigned char*)g.master : (const unsigned char*)g.mom;
         const unsigned char* src = base + ((long long)(bm + within / PF_LPR) * g.N + bn) * PF_ES + (within % PF_LPR) * 128;
+        if constexpr (kMask)   // derivative from the sign bits the forward product left: its lines instead
+            src = (const unsigned char*)g.mask_in + (long long)(tm * tiles_n + tn) * (NT * MASK_WORDS * 4) + (line % (NT * MASK_WORDS * 4 / 128)) * 128;
         if (lane < PF_LANES) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
     };
     constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0) + (kMX ? MI : 0);  // loads a stage's closing wait leaves in flight
@@ -422,6 +427,25 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     const int M = g.M, N = g.N;
     __builtin_amdgcn_s_barrier();  // every wavefront is done with the ring
 
+    if constexpr (kMask) {
+        // The activation below is a step in its derivative (ReLU, leaky ReLU): f' takes one of two values by the sign of
+        // the activation, and the forward product that stored the activations left those signs, a bit per element in
+        // the order of the accumulators of the workgroup that computed them -- which is this workgroup's order: same
+        // rows, same units, same tile.  16 bytes per lane instead of a 128 KB tile through LDS.
+        const unsigned int* mw = g.mask_in + ((long long)(tm * tiles_n + tn) * NT + t) * MASK_WORDS;
+        unsigned int bits[MASK_WORDS];
+#pragma unroll
+        for (int k = 0; k < MASK_WORDS; ++k) bits[k] = mw[k];
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int b = (mi * NI + ni) * 16 + i;
+                    acc[mi][ni][i] *= ((bits[b >> 5] >> (b & 31)) & 1u) ? g.ap.dhi : g.ap.dlo;
+                }
+    }
     if constexpr (EPI == LP_DGRAD) {
         // activation tile [TM][TN] bf16 -> LDS (row pitch 2*TN bytes) with LDS-direct loads
         constexpr int LPR = TN / 8;         // lanes per tile row (16 bytes each)
@@ -452,7 +476,7 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     }
 
     constexpr bool kActMX = (EPI == LP_FP8_ACT_MX);   // e4m3 codes + block scales out, through the same bf16 staging
-    constexpr bool kBf16Out = (EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT || kActMX);
+    constexpr bool kBf16Out = (EPI == LP_FWD_ACT || kDgrad || EPI == LP_WGRAD_SGD || EPI == LP_FP8_ACT || kActMX);
     constexpr bool kFwd = (EPI == LP_FWD_ACT || EPI == LP_FWD_F32), kF8 = (EPI == LP_FP8_ACT || EPI == LP_FP8_F32 || kMX);
     uint2 pk[MI][NI][4];  // bf16 results, 4 consecutive rows packed per entry
     float cbias[NI], cscale[NI];
@@ -526,10 +550,33 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     };
     if ((kFwd || kF8) && !g.ap.plain) finish(IC<0>{});
     else finish(IC<1>{});
+    if constexpr (EPI == LP_FWD_ACT) {
+        if (g.mask_out) {   // the signs of the stored activations, for the back-propagation product of this tile (see there)
+            unsigned int bits[MASK_WORDS];
+#pragma unroll
+            for (int k = 0; k < MASK_WORDS; ++k) bits[k] = 0u;
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint2 v = pk[mi][ni][q];
+                        // a bf16 is positive where its 16 bits, read as a signed integer, are
+                        const unsigned int four = ((short)(v.x & 0xffffu) > 0 ? 1u : 0u) | ((short)(v.x >> 16) > 0 ? 2u : 0u) |
+                                                  ((short)(v.y & 0xffffu) > 0 ? 4u : 0u) | ((short)(v.y >> 16) > 0 ? 8u : 0u);
+                        const int b = (mi * NI + ni) * 16 + q * 4;
+                        bits[b >> 5] |= four << (b & 31);
+                    }
+            unsigned int* mw = g.mask_out + ((long long)(tm * tiles_n + tn) * NT + t) * MASK_WORDS;
+#pragma unroll
+            for (int k = 0; k < MASK_WORDS; ++k) mw[k] = bits[k];
+        }
+    }
     // back-propagation also leaves the column sums of the deltas it stores (the bias gradient of
     // the layer below), per tile row so that the caller adds them in a fixed order
     float csum[NI];
-    if constexpr (EPI == LP_DGRAD) {
+    if constexpr (kDgrad) {
 #pragma unroll
         for (int ni = 0; ni < NI; ++ni) {
             float s = 0.0f;
@@ -546,7 +593,7 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     }
     if constexpr (kBf16Out) {
         // transposed copy first: LDS_T[n][m], a lane's 4 consecutive rows are 8 contiguous bytes
-        if ((EPI == LP_FWD_ACT || EPI == LP_DGRAD || EPI == LP_WGRAD_SGD) && g.outT) {
+        if ((EPI == LP_FWD_ACT || kDgrad || EPI == LP_WGRAD_SGD) && g.outT) {
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
@@ -654,7 +701,7 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
                 for (int i = 0; i < NIT; ++i) atomicMax(&g.row_amax_bits[bm + w * (TM / 8) + i * RPI + lane / LPR], am[i] << 16);
         }
     }
-    if constexpr (EPI == LP_DGRAD) {
+    if constexpr (kDgrad) {
         if (g.colsum) {
             float* red = reinterpret_cast<float*>(smem);  // [2][TN]: one row per wavefront row
             __builtin_amdgcn_s_waitcnt(0xC07F);
@@ -764,7 +811,9 @@ hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
         switch (a.epilogue) {
         case LP_FWD_ACT: return launch<false, LP_FWD_ACT>(a, s);
         case LP_FWD_F32: return launch<false, LP_FWD_F32>(a, s);
-        case LP_DGRAD: return launch<false, LP_DGRAD>(a, s);
+        case LP_DGRAD:
+            if (a.mask_in && a.ap.step) return launch<false, LP_DGRAD_MASK>(a, s);
+            return launch<false, LP_DGRAD>(a, s);
         case LP_WGRAD_SGD: return launch<false, LP_WGRAD_SGD>(a, s);
         }
     } else {

@@ -408,7 +408,8 @@ enum LpEpilogue {
     // scale per row and 32 elements of K (a_scale) instead of one fp32 scale per row, and LP_FP8_ACT_MX leaves
     // its result as the next layer's A operand, e4m3 codes [M][N] + scales (out_scale), quantised in the epilogue.
     LP_FP8_ACT_MX = 6,  // v = squash(acc * cs[n]) -> bf16 rounding -> codes + block scales
-    LP_FP8_F32_MX = 7   // fp32 out = squash(acc * cs[n])
+    LP_FP8_F32_MX = 7,  // fp32 out = squash(acc * cs[n])
+    LP_DGRAD_MASK = 8   // LP_DGRAD for a step derivative, from the sign bits in mask_in (chosen by ghip_gemm_lp; callers ask for LP_DGRAD)
 };
 struct GemmLpArgs {
     const void* A; const void* B;    // [M][K], [N][K], K contiguous; bf16 or e4m3
@@ -427,6 +428,10 @@ struct GemmLpArgs {
     void* out; void* outT;            // see LpEpilogue; outT may be NULL
     const float* bias;                // [N] or NULL
     const uint16_t* aux;              // LP_DGRAD: activations bf16 [M][N]
+    // LP_FWD_ACT may leave, and LP_DGRAD take instead of aux, the signs of the stored activations (1 = positive), a bit
+    // per element in the order of the computing workgroup's accumulators: M * N / 8 bytes.  For activations whose
+    // derivative is a step (ReLU, leaky ReLU); both products then have to run the same tiling of [M][N].
+    unsigned int* mask_out; const unsigned int* mask_in;
     float* colsum;                    // LP_DGRAD: if set, [M / tile_m][N] column sums of the stored deltas per tile row
     int act; float act_param;   // resolved into `ap` by ghip_gemm_lp
     struct ActForm {
