@@ -33,6 +33,8 @@
 
 #include "ghip_internal.h"
 
+#include <string.h>
+
 namespace {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -307,41 +309,8 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     constexpr int KS = FP8 ? 2 : 4;
     constexpr int G = MI * NI;
     constexpr bool kDouble = !(FP8 && G > 2);
-    // Tiles whose epilogue reads more memory get it moving while the K loop leaves HBM idle:
-    // weight-gradient tiles end with a read-modify-write of the fp32 master weights and momentum
-    // (2 x TN x 4 bytes per tile row, bound by HBM), back-propagation tiles read the bf16
-    // activations (TN x 2 bytes per row).  Every stage of the last PF_N each wavefront touches one
-    // dword of 8 of those 128-byte lines, which are then in the memory-side cache (or L2) when the
-    // epilogue asks for them.  The touch goes out between the B and the A loads of the fill, so the
-    // wait that ends a stage (which only needs B) leaves it in flight like the A loads; its result
-    // is never used.
-    constexpr bool kTouch = (EPI == LP_WGRAD_SGD || kDgrad);
     constexpr int MASK_WORDS = MI * NI * 16 / 32;   // a lane's accumulators, one bit each
-    constexpr int PF_ES = (EPI == LP_WGRAD_SGD) ? 4 : 2;         // bytes per element of the touched arrays
-    constexpr int PF_ARRAYS = (EPI == LP_WGRAD_SGD) ? 2 : 1;
-    constexpr int PF_LPR = TN * PF_ES / 128;                     // lines per tile row
-    constexpr int PF_PER = TM * PF_LPR;                          // lines per array
-    // lines a wavefront touches per stage: every line is a request of its own to the address unit that
-    // the operand loads also go through, so wider touches over fewer stages cost more than they save
-    // (16 lanes: the training step 1.6 % slower, 32: 4 %, 64: 26 %)
-    constexpr int PF_LANES = 8;
-    constexpr int PF_N = cmax(PF_ARRAYS * PF_PER / (8 * PF_LANES), 1);    // stages needed: 8 * PF_LANES lines per stage and workgroup
-    constexpr int PF_LEAD = 2;
-    int pfreg = 0;
-    const int pf_j0 = nk - PF_N - PF_LEAD > 0 ? nk - PF_N - PF_LEAD : 0;
-    auto touch = [&](int j) {
-        int i = j - pf_j0;
-        i = i < 0 ? 0 : (i >= PF_N ? PF_N - 1 : i);  // outside the window: repeat a touched line
-        const int line = (i * 8 + ws) * PF_LANES + (lane & (PF_LANES - 1));
-        const int within = line % PF_PER;
-        const unsigned char* base = kDgrad ? (const unsigned char*)g.aux
-                                  : (line < PF_PER) ? (const unsigned char*)g.master : (const unsigned char*)g.mom;
-        const unsigned char* src = base + ((long long)(bm + within / PF_LPR) * g.N + bn) * PF_ES + (within % PF_LPR) * 128;
-        if constexpr (kMask)   // derivative from the sign bits the forward product left: its lines instead
-            src = (const unsigned char*)g.mask_in + (long long)(tm * tiles_n + tn) * (NT * MASK_WORDS * 4) + (line % (NT * MASK_WORDS * 4 / 128)) * 128;
-        if (lane < PF_LANES) asm volatile("global_load_dword %0, %1, off" : "+v"(pfreg) : "v"(src) : "memory");
-    };
-    constexpr int VM_STAGE = PWA + (kTouch ? 1 : 0) + (kMX ? MI : 0);  // loads a stage's closing wait leaves in flight
+    constexpr int VM_STAGE = PWA + (kMX ? MI : 0);  // loads a stage's closing wait leaves in flight
     static_assert(VM_STAGE <= 15, "the count fits the low four bits of the wait's immediate");
     // The Y half-stage, asked for one stage before the wait for it, is the load that arrives late, and
     // most of all where the operands come from HBM rather than the memory-side cache (the weight
@@ -356,7 +325,6 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
         const unsigned char* const NA = smem + ((2 * P + 2 + OA) % NSLOT) * SLOT;
         const unsigned char* const NB = smem + ((2 * P + 2 + OB) % NSLOT) * SLOT;
         auto dma = [&](int d) {
-            if (kTouch && d == 0) touch(j);
             if constexpr (kMX) { if (d == 0) load_scales(IC<(P + 2) % NSLOT>{}, j + 2); }
             dmaX((2 * P + 4) % NSLOT, j + 2, d);
         };
@@ -417,7 +385,6 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     }
     // nothing may still be writing this workgroup's LDS when its wavefronts retire
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    asm volatile("" : : "v"(pfreg));  // the touches' destination stays reserved up to here
 
     // ---- epilogue.  Accumulator layout of a 32x32 tile: lane -> column lane%32,
     //      register i -> row 8*(i/4) + 4*(lane/32) + i%4  (4 consecutive rows per register quad).
@@ -493,6 +460,27 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
         constexpr bool PLAIN = decltype(plain_c)::value;
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
+            // weight gradient: the master weights and momentum of a whole 32-row block are asked for together,
+            // ahead of the arithmetic and of any store (element by element, each load pair would wait out a round
+            // trip to memory before the next one could leave: 128 round trips per lane were the update's time)
+            float mw[4][NI][4], mv[4][NI][4];
+            if constexpr (EPI == LP_WGRAD_SGD) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            mw[q][ni][r] = g.master[(long long)(bm + wm + mi * 32 + 8 * q + 4 * lh + r) * N + bn + wn + ni * 32 + l31];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            mv[q][ni][r] = g.mom[(long long)(bm + wm + mi * 32 + 8 * q + 4 * lh + r) * N + bn + wn + ni * 32 + l31];
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
                 const int row0 = bm + wm + mi * 32 + 8 * q + 4 * lh;
@@ -516,10 +504,10 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
                         } else if constexpr (kF8) {
                             o[r] = lp_squash<PLAIN>(__fmul_rn(v, __fmul_rn(rs[r], cscale[ni])), g.ap);
                         } else if constexpr (EPI == LP_WGRAD_SGD) {
-                            const float wv = g.master[idx];
+                            const float wv = mw[q][ni][r];
                             const float sg = (wv > 0.0f) ? 1.0f : ((wv < 0.0f) ? -1.0f : 0.0f);
                             const float gr = v * g.gscale + g.wd1 * sg + g.wd2 * wv;
-                            const float d = g.lr * gr + g.momf * g.mom[idx];
+                            const float d = g.lr * gr + g.momf * mv[q][ni][r];
                             g.mom[idx] = d;
                             o[r] = wv - d;
                             g.master[idx] = o[r];
@@ -730,6 +718,23 @@ __global__ void __launch_bounds__(NT) gemm_lp_kernel(GemmLpArgs g)
     gemm_lp_tile<FP8, EPI, MI, NI>(g, xcd_tile_id(blockIdx.x, (g.M / (64 * MI)) * (g.N / (128 * NI))), smem);
 }
 
+// The 256 x 256-tile weight gradients of a training step as ONE launch: they are independent of one another once the
+// back-propagation chain is through.  A workgroup looks up its product and tile in a schedule the host lays out
+// (ghip_gemm_lp_wgrad_plan).  Without a launch boundary after every layer a CU that has finished a tile's update goes
+// on with the next layer's tile while its neighbours still write theirs: measured 2 to 4 % less than a launch per
+// layer.  (Also measured, and not kept: starting half of the CUs, or half of the XCDs, late, so that the two halves
+// never update at the same time.  It recovers about half of the delay it costs and no more.)
+struct GemmLpGroupArgs {
+    GemmLpArgs p[GHIP_GEMM_LP_GROUP_MAX];
+    const unsigned int* sched;   // per workgroup: bits 24..30 = product, bits 0..23 = tile number
+};
+__global__ void __launch_bounds__(NT) gemm_lp_wgrad_group_kernel(GemmLpGroupArgs grp)
+{
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[lp_lds_bytes<4, 2>()];
+    const unsigned int e = grp.sched[blockIdx.x];
+    gemm_lp_tile<false, LP_WGRAD_SGD, 4, 2>(grp.p[(e >> 24) & 0x7f], (int)(e & 0xffffffu), smem);
+}
+
 // 256 x 256 tiles when they give every CU at least one workgroup, else 128 x 128.
 constexpr int kCUs = 256;
 inline bool use_small_tile(int M, int N) { return (long long)(M / 256) * (N / 256) < kCUs; }
@@ -800,6 +805,56 @@ static bool operands_ok(const GemmLpArgs& a_)
     const bool pitchB_ok = a_.kstrideB ? ((long long)a_.ldb * es == 128 && a_.kstrideB % 128 == 0) : (!a_.ldb || a_.ldb >= a_.K);
     return pitchA_ok && pitchB_ok && !(a_.lda && ((long long)a_.lda * es) % 16) && !(a_.ldb && ((long long)a_.ldb * es) % 16) &&
            (((uintptr_t)a_.A | (uintptr_t)a_.B) % 16) == 0;
+}
+
+// Schedule of a grouped weight-gradient launch over `count` products of M[i] x N[i] outputs, all of them 256 x 256-tile
+// products (ghip_gemm_lp_tile_m): one entry per workgroup.  Workgroup b runs on XCD b % 8, and a CU takes one
+// workgroup at a time (the kernel asks for all of its LDS), so entries b, b + 8, b + 16, ... are what one XCD's CUs
+// work through in order: every XCD gets a contiguous eighth of each product's tiles (its CUs then share operand
+// rows in its L2), the products in the caller's order.  Returns the number of workgroups, -1 if it does not apply.
+int ghip_gemm_lp_wgrad_plan(const int* M, const int* N, int count, unsigned int* sched, int cap)
+{
+    if (count < 1 || count > GHIP_GEMM_LP_GROUP_MAX) return -1;
+    int total = 0;
+    bool by_xcd = true;
+    for (int i = 0; i < count; ++i) {
+        if (use_small_tile(M[i], N[i])) return -1;
+        const int nb = (M[i] / 256) * (N[i] / 256);
+        if (nb > 0xffffff) return -1;
+        by_xcd = by_xcd && (nb % 8) == 0;
+        total += nb;
+    }
+    if (total > cap) return -1;
+    int k = 0;
+    if (!by_xcd) {
+        for (int i = 0; i < count; ++i)
+            for (int t = 0; t < (M[i] / 256) * (N[i] / 256); ++t) sched[k++] = ((unsigned int)i << 24) | (unsigned int)t;
+        return total;
+    }
+    for (int i = 0; i < count; ++i) {
+        const int per = (M[i] / 256) * (N[i] / 256) / 8;
+        for (int t = 0; t < per; ++t)
+            for (int x = 0; x < 8; ++x) sched[k++] = ((unsigned int)i << 24) | (unsigned int)(x * per + t);
+    }
+    return total;
+}
+
+hipError_t ghip_gemm_lp_wgrad_group(const GemmLpArgs* a, int count, const unsigned int* dev_sched, int blocks, hipStream_t s)
+{
+    if (count < 1 || count > GHIP_GEMM_LP_GROUP_MAX || !dev_sched || blocks < 1) return hipErrorInvalidValue;
+    GemmLpGroupArgs grp;
+    memset(&grp, 0, sizeof(grp));
+    int total = 0;
+    for (int i = 0; i < count; ++i) {
+        if (a[i].fp8 || a[i].epilogue != LP_WGRAD_SGD || !operands_ok(a[i]) || use_small_tile(a[i].M, a[i].N)) return hipErrorInvalidValue;
+        grp.p[i] = a[i];
+        resolve_act(grp.p[i]);
+        total += (a[i].M / 256) * (a[i].N / 256);
+    }
+    if (total != blocks) return hipErrorInvalidValue;   // the schedule was laid out for other products
+    grp.sched = dev_sched;
+    hipLaunchKernelGGL(gemm_lp_wgrad_group_kernel, dim3(blocks), dim3(NT), 0, s, grp);
+    return hipGetLastError();
 }
 
 hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)

@@ -453,6 +453,13 @@ struct GemmLpArgs {
     unsigned int* out_scale; int ld_out_scale;
 };
 hipError_t ghip_gemm_lp(const GemmLpArgs& a, hipStream_t s);
+// The 256 x 256-tile weight gradients (LP_WGRAD_SGD, bf16) of up to GHIP_GEMM_LP_GROUP_MAX layers as one launch.
+// ghip_gemm_lp_wgrad_plan lays out the launch's schedule for products of M[i] x N[i] outputs into `sched` (host
+// memory, `cap` entries) and returns the number of workgroups, or -1 if a product takes the smaller tile; the
+// launch takes that schedule in device memory.
+#define GHIP_GEMM_LP_GROUP_MAX 8
+int ghip_gemm_lp_wgrad_plan(const int* M, const int* N, int count, unsigned int* sched, int cap);
+hipError_t ghip_gemm_lp_wgrad_group(const GemmLpArgs* a, int count, const unsigned int* dev_sched, int blocks, hipStream_t s);
 bool ghip_gemm_lp_shape_ok(int M, int N, int K, int fp8);
 int ghip_gemm_lp_tile_m(int M, int N);  // rows per tile the launcher picks for this product
 
