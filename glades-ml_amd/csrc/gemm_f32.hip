@@ -218,6 +218,23 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmF32Args& g, const int bx
     const int col = bn + wn + lr;
     if (col < g.N) {
         const float bias = (g.epilogue == EPI_BIAS_ACT && g.bias) ? g.bias[col] : 0.0f;
+        // what the epilogue reads (activations for the derivative; weights and momentum for the update) is asked for in
+        // one go, ahead of the first store: element by element, every load would wait out a round trip of its own
+        float in0[16], in1[16];
+        if (g.epilogue == EPI_SGD || g.epilogue == EPI_MUL_DER) {
+            const float* s0 = g.epilogue == EPI_SGD ? g.C : g.aux;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = bm + wm + 8 * (i >> 2) + 4 * lk + (i & 3);
+                in0[i] = row < g.M ? s0[(long long)row * g.ldc + col] : 0.0f;
+            }
+            if (g.epilogue == EPI_SGD)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int row = bm + wm + 8 * (i >> 2) + 4 * lk + (i & 3);
+                    in1[i] = row < g.M ? g.V[(long long)row * g.ldc + col] : 0.0f;
+                }
+        }
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int row = bm + wm + 8 * (i >> 2) + 4 * lk + (i & 3);
@@ -225,12 +242,12 @@ __device__ __forceinline__ void gemm_f32_tile(const GemmF32Args& g, const int bx
                 float v = acc[i];
                 const long long idx = (long long)row * g.ldc + col;
                 if (g.epilogue == EPI_BIAS_ACT) v = ghip_squash<false>(v + bias, g.act, g.act_param);
-                else if (g.epilogue == EPI_MUL_DER) v = v * ghip_act_der_canon(g.aux[idx], g.act, g.act_param);
+                else if (g.epilogue == EPI_MUL_DER) v = v * ghip_act_der_canon(in0[i], g.act, g.act_param);
                 else if (g.epilogue == EPI_SGD) {
-                    const float wgt = g.C[idx];
+                    const float wgt = in0[i];
                     const float sg = (wgt > 0.0f) ? 1.0f : ((wgt < 0.0f) ? -1.0f : 0.0f);
                     const float grad = v * g.alpha + g.wd1 * sg + g.wd2 * wgt;
-                    const float d = g.lr * grad + g.mom * g.V[idx];
+                    const float d = g.lr * grad + g.mom * in1[i];
                     g.V[idx] = d;
                     v = wgt - d;
                 } else v = v * g.alpha;
