@@ -238,7 +238,8 @@ int ghip_net_forward_resident(ghip_net* net, int64_t row0, int batch, float* dev
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It takes no handle and calls
  * no allocating routine: parameters, inputs and outputs are the caller's device memory (dev_W[l]:
  * sizes[l+1] x sizes[l] row-major, dev_bias[l]: sizes[l+1], dev_X: batch x sizes[0], dev_out: batch x
- * sizes[n_layers], all fp32, 16-byte aligned), and the hidden layers' activations live in a fixed
+ * sizes[n_layers], all fp32, 16-byte aligned: other pointers are refused with GHIP_EINVAL), and the
+ * hidden layers' activations live in a fixed
  * array in the library's device image (2 x GHIP_NOALLOC_MAX_ACTIVATIONS floats + 256 bytes = 32 MiB
  * per GPU, held until the process ends).  batch x sizes[l] of every hidden layer l must not exceed
  * GHIP_NOALLOC_MAX_ACTIVATIONS; larger requests are refused with GHIP_EINVAL.  spec: mode
