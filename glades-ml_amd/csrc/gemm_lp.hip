@@ -96,6 +96,26 @@ __device__ __forceinline__ void load_frags(Frags<FP8, MI, NI>& f, const unsigned
             f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, FP8 ? ks * 4 + h * 2 + lh : ks * 2 + lh));
 }
 
+// the same in two parts: row block mi of A, and all of B
+template <bool FP8, int MI, int NI>
+__device__ __forceinline__ void load_frag_a(Frags<FP8, MI, NI>& f, const unsigned char* sa, int ks, int mi, int wm, int l31, int lh)
+{
+    constexpr int H = FP8 ? 2 : 1;
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+        f.a[mi][h] = *reinterpret_cast<const v4i*>(sa + swz(wm + mi * 32 + l31, FP8 ? ks * 4 + h * 2 + lh : ks * 2 + lh));
+}
+template <bool FP8, int MI, int NI>
+__device__ __forceinline__ void load_frags_b(Frags<FP8, MI, NI>& f, const unsigned char* sb, int ks, int wn, int l31, int lh)
+{
+    constexpr int H = FP8 ? 2 : 1;
+#pragma unroll
+    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+            f.b[ni][h] = *reinterpret_cast<const v4i*>(sb + swz(wn + ni * 32 + l31, FP8 ? ks * 4 + h * 2 + lh : ks * 2 + lh));
+}
+
 typedef __attribute__((address_space(3))) unsigned char* lptr_t;
 
 // LDS-direct load of one 1 KiB slab: lane i's 16 bytes land at lds_slab + 16*i.
@@ -123,6 +143,12 @@ __device__ __forceinline__ void load_dword_s(unsigned int& dst, const void* sbas
     asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(dst) : "v"(voff), "s"(sbase), "n"(OFF) : "memory");
 }
 
+// 16 bytes per lane the same way: an operand half-stage on its way to LDS through registers (see the main loop)
+__device__ __forceinline__ void load_x4_s(v4i& dst, const void* sbase, unsigned int voff)
+{
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(dst) : "v"(voff), "s"(sbase) : "memory");
+}
+
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 template <int V> struct IC { static constexpr int value = V; };
 
@@ -132,8 +158,10 @@ template <int V> struct IC { static constexpr int value = V; };
 // loads back to back stalls on the address unit (16 clocks per load, shared by the 8 wavefronts),
 // and the matrix pipe of its SIMD idles with it.
 // OPSEL: the byte of sa[mi] that holds this sub-step's E8M0 scale of the lane's block of A (e4m3 only; 0x7f = 1)
-template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, int OPSEL = 0, typename Dma>
-__device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma, const unsigned int (&sa)[MI])
+// row(mi) runs once the MFMAs that read row block mi of A have been issued (the rolling fragment loads: the block's
+// registers are free for the next sub-step's block from there on).
+template <bool FP8, int MI, int NI, int SPAN, int NDMA, int BEFORE, int OPSEL = 0, typename Dma, typename Row>
+__device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, MI, NI>& f, Dma&& dma, const unsigned int (&sa)[MI], Row&& row)
 {
 #pragma unroll
     for (int mi = 0; mi < MI; ++mi)
@@ -163,6 +191,7 @@ __device__ __forceinline__ void mma_group(v16f (&acc)[MI][NI], const Frags<FP8, 
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
+            if (ni == NI - 1) row(mi);
         }
 }
 
@@ -286,13 +315,41 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     auto dmaX = [&](int slot, int st, int jj) { if constexpr (kSwap) dmaB(slot, st, jj); else dmaA(slot, st, jj); };
     auto dmaY = [&](int slot, int st, int jj) { if constexpr (kSwap) dmaA(slot, st, jj); else dmaB(slot, st, jj); };
     constexpr int OA = kSwap ? 1 : 0, OB = kSwap ? 0 : 1;  // places of A and B within a stage's pair of slots
+    // The bf16 128-row tiles (two workgroups to a CU, the global->LDS path their bound) take Y's half-stages through
+    // registers.  Straight into LDS, a half-stage can only be asked for once its slot is free, one stage ahead of its
+    // use.  A register set per stage parity holds Y(j+2) from the start of stage j until the middle of stage j+1, when
+    // it is written to the slot that stage j's barrier freed: a stage and a half in flight for 2 x PWB x 4 registers
+    // (the narrow layer's weight gradient runs 16 % faster).  The 256 x 256 tiles lose 3 to 7 % that way, with the loads
+    // in one go behind the barrier or spread between the MFMAs alike, and keep the direct path: each operand's loads
+    // alone cost their loop 3 %, both together 35 % -- its bound is what the path delivers, not how early it is asked.
+    constexpr int RY = (!FP8 && MI * NI < 8) ? PWB : 0;   // slabs of Y per wavefront that go through registers
+    constexpr bool kRegY = RY > 0;
+    v4i yreg[2][RY > 0 ? RY : 1];
+    auto ldY = [&](auto setc, int st, int jj) {
+        constexpr int S = decltype(setc)::value;
+        if constexpr (kSwap) {
+            const long long kb = (long long)(st < nk ? st : nk - 1) * ksA;
+            load_x4_s(yreg[S][jj], gAw + (long long)(jj * 8) * lda + kb, voffA[jj & 1]);
+        } else {
+            const long long kb = (long long)(st < nk ? st : nk - 1) * ksB;
+            load_x4_s(yreg[S][jj], gBw + (long long)(jj * 8) * ldb + kb, voffB[jj & 1]);
+        }
+    };
+    auto wrY = [&](auto setc, int slot) {   // lane i's 16 bytes to where the direct load puts them: slab + 16 i
+        constexpr int S = decltype(setc)::value;
+#pragma unroll
+        for (int jj = 0; jj < RY; ++jj)
+            *reinterpret_cast<v4i*>(smem + slot * SLOT + (ws * PWB + jj) * 1024 + lane * 16) = yreg[S][jj];
+    };
 #pragma unroll
     for (int jj = 0; jj < PWA; ++jj) dmaX(0, 0, jj);
 #pragma unroll
     for (int jj = 0; jj < PWB; ++jj) dmaY(1, 0, jj);
 #pragma unroll
+    for (int jj = 0; jj < RY; ++jj) ldY(IC<1>{}, 1, jj);
+#pragma unroll
     for (int jj = 0; jj < PWA; ++jj) dmaX(2, 1, jj);
-    __builtin_amdgcn_s_waitcnt(0x0F70 | PWA);  // vmcnt(PWA): A0 and B0 have landed
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (PWA + RY));  // A0 and B0 have landed
     __builtin_amdgcn_s_barrier();
 
     typedef Frags<FP8, MI, NI> F;
@@ -300,30 +357,42 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
     load_frags<FP8, MI, NI>(f0, smem + OA * SLOT, smem + OB * SLOT, 0, wm, wn, l31, lh);
 
     // One stage (P = j mod 5 fixes the slots at compile time).  Sub-steps are software pipelined:
-    // each one first states that its own fragments (requested one MFMA group earlier) have landed,
-    // then requests the next sub-step's fragments, then issues its MFMAs with the fill's loads
-    // between them.  The last sub-step waits for B(j+1), meets the other wavefronts (bare
-    // s_barrier: the explicit counts are exactly what has to be visible) and requests the first
-    // fragments of stage j+1.  The 256 x 256 e4m3 tile has no registers left for a second fragment
-    // set and runs its two sub-steps in sequence.
+    // each one requests the next sub-step's B fragments, then issues its MFMAs with the fill's loads
+    // between them and, behind the MFMAs that read a row block of A, the request for the next
+    // sub-step's block (the compiler places the waits for these LDS reads).  The last sub-step waits
+    // for B(j+1), meets the other wavefronts (bare s_barrier: the explicit counts are exactly what has
+    // to be visible) and requests the first fragments of stage j+1.  The 256 x 256 e4m3 tile runs its
+    // two sub-steps in sequence on one fragment set.
     constexpr int KS = FP8 ? 2 : 4;
     constexpr int G = MI * NI;
     constexpr bool kDouble = !(FP8 && G > 2);
     constexpr int MASK_WORDS = MI * NI * 16 / 32;   // a lane's accumulators, one bit each
-    constexpr int VM_STAGE = PWA + (kMX ? MI : 0);  // loads a stage's closing wait leaves in flight
-    static_assert(VM_STAGE <= 15, "the count fits the low four bits of the wait's immediate");
-    // The Y half-stage, asked for one stage before the wait for it, is the load that arrives late, and
-    // most of all where the operands come from HBM rather than the memory-side cache (the weight
-    // gradient's are a forward pass old).  So its loads go out as early as their slot allows, back to
-    // back right behind the barrier that closes the stage before (spread over the stage with X's, they
-    // cost the bf16 training step 5 % and the e4m3 products 7 %), and only X's, which have a stage more,
-    // are spread between the MFMAs.
-    auto stage = [&](auto Pc, int j) {
+    // loads a stage's closing wait leaves in flight: X(j+2), and Y(j+2) on its way to registers / the scale dwords
+    constexpr int VM_STAGE = PWA + (kMX ? MI : 0) + RY;
+    // ... and the wait in the middle of a stage for the registers of Y(j+1): X(j+1), Y(j+2) and X(j+2) were asked for later
+    constexpr int VM_MID = 2 * PWA + PWB;
+    static_assert(VM_STAGE <= 15 && VM_MID <= 15, "the counts fit the low four bits of the wait's immediate");
+    // Y's loads go out as early as their slot allows, back to back right behind the barrier that closes
+    // the stage before (spread over the stage with X's, they cost the bf16 training step 5 % and the e4m3
+    // products 7 %), and only X's, which have a stage more, are spread between the MFMAs.  What the loop
+    // waits for is the path from L2 to LDS as a whole: without any loads the 256 x 256 bf16 loop keeps the
+    // matrix pipes busy (1.07 us per stage), with either operand's loads alone it takes 3 % longer, with both
+    // 45 % (1.56 us): 64 KB per stage and CU are 15 TB/s over the chip at the matrix pipes' rate, and the
+    // path delivers 10 to 11 in this loop.
+    auto stage = [&](auto Pc, auto Qc, int j) {
         constexpr int P = decltype(Pc)::value;
-        const unsigned char* const RA = smem + ((2 * P + OA) % NSLOT) * SLOT;
-        const unsigned char* const RB = smem + ((2 * P + OB) % NSLOT) * SLOT;
-        const unsigned char* const NA = smem + ((2 * P + 2 + OA) % NSLOT) * SLOT;
-        const unsigned char* const NB = smem + ((2 * P + 2 + OB) % NSLOT) * SLOT;
+        constexpr int Q = decltype(Qc)::value;   // j mod 2: the register set that holds Y(j+2); the other one turns over in this stage
+        // The slots' offsets reach the fragment reads as scalars the compiler cannot fold: folded, every (slot, sub-step,
+        // operand) combination becomes an address register of its own, kept across the whole loop (24 of them)
+        auto slot_at = [&](auto slot_c) {
+            unsigned int off;
+            asm volatile("s_mov_b32 %0, %1" : "=s"(off) : "i"(decltype(slot_c)::value * SLOT));
+            return smem + off;
+        };
+        const unsigned char* const RA = slot_at(IC<(2 * P + OA) % NSLOT>{});
+        const unsigned char* const RB = slot_at(IC<(2 * P + OB) % NSLOT>{});
+        const unsigned char* const NA = slot_at(IC<(2 * P + 2 + OA) % NSLOT>{});
+        const unsigned char* const NB = slot_at(IC<(2 * P + 2 + OB) % NSLOT>{});
         auto dma = [&](int d) {
             if constexpr (kMX) { if (d == 0) load_scales(IC<(P + 2) % NSLOT>{}, j + 2); }
             dmaX((2 * P + 4) % NSLOT, j + 2, d);
@@ -337,14 +406,17 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
         auto next_y = [&]() {  // the next stage's Y loads: their slot is free once this stage's closing barrier is passed
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int d = 0; d < PWB; ++d) dmaY((2 * P + 5) % NSLOT, j + 2, d);
+            for (int d = RY; d < PWB; ++d) dmaY((2 * P + 5) % NSLOT, j + 2, d);   // straight into LDS: one stage ahead
+#pragma unroll
+            for (int d = 0; d < RY; ++d) ldY(IC<(Q + 1) & 1>{}, j + 3, d);        // by way of registers: two
             __builtin_amdgcn_sched_barrier(0);
         };
+        auto norow = [](int) {};
         if constexpr (!kDouble) {
             constexpr int SPAN = 2 * G;
-            mma_group<FP8, MI, NI, SPAN, PWA, 0, 0>(acc, f0, dma, sa);
+            mma_group<FP8, MI, NI, SPAN, PWA, 0, 0>(acc, f0, dma, sa, norow);
             load_frags<FP8, MI, NI>(f0, RA, RB, 1, wm, wn, l31, lh);
-            mma_group<FP8, MI, NI, SPAN, PWA, G, 2>(acc, f0, dma, sa);
+            mma_group<FP8, MI, NI, SPAN, PWA, G, 2>(acc, f0, dma, sa, norow);
             __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
             __builtin_amdgcn_s_barrier();
             next_y();
@@ -355,36 +427,84 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
             for (int ks = 0; ks < KS; ++ks) {
                 F& cur = (ks & 1) ? f1 : f0;
                 F& nxt = (ks & 1) ? f0 : f1;
+                // The next sub-step's fragments: B's at the head of this one, A's block by block behind the MFMAs that
+                // read the block before it (one set of A fragments and a block in transit instead of two sets)
+                const unsigned char* const FA = (ks + 1 < KS) ? RA : NA;
+                const int fks = (ks + 1 < KS) ? ks + 1 : 0;
+                auto row = [&](int mi) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_frag_a<FP8, MI, NI>(nxt, FA, fks, mi, wm, l31, lh);
+                    __builtin_amdgcn_sched_barrier(0);
+                };
                 if (ks + 1 < KS) {
-                    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): cur has landed
-                    load_frags<FP8, MI, NI>(nxt, RA, RB, ks + 1, wm, wn, l31, lh);
+                    load_frags_b<FP8, MI, NI>(nxt, RB, ks + 1, wn, l31, lh);
+                    if constexpr (kRegY) {
+                        if (ks == KS - 2) {   // all of X(j+2) has been asked for by now (see mma_group): the count below holds
+                            static_assert((2 * G) / ((KS - 1) * G / (PWA + 1) > 0 ? (KS - 1) * G / (PWA + 1) : 1) >= PWA, "X's loads are out after two sub-steps");
+                            __builtin_amdgcn_sched_barrier(0);
+                            __builtin_amdgcn_s_waitcnt(0x0F70 | VM_MID);  // Y(j+1) is in its registers
+                            __builtin_amdgcn_sched_barrier(0);
+                            wrY(IC<(Q + 1) & 1>{}, (2 * P + 3) % NSLOT);   // Y's place in stage j+1's pair of slots
+                        }
+                    }
                 } else {
                     __builtin_amdgcn_s_waitcnt(0x0070 | VM_STAGE);  // vmcnt(VM_STAGE) lgkmcnt(0)
                     __builtin_amdgcn_s_barrier();
                     next_y();
-                    load_frags<FP8, MI, NI>(nxt, NA, NB, 0, wm, wn, l31, lh);
+                    load_frags_b<FP8, MI, NI>(nxt, NB, 0, wn, l31, lh);
                 }
                 __builtin_amdgcn_sched_barrier(0);
-                if (ks == 0) mma_group<FP8, MI, NI, SPAN, PWA, 0, 0>(acc, cur, dma, sa);
-                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, cur, dma, sa);
-                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, PWA, 2 * G>(acc, cur, dma, sa);
-                else mma_group<FP8, MI, NI, 1, 0, 0, FP8 ? 2 : 0>(acc, cur, none, sa);
+                if (ks == 0) mma_group<FP8, MI, NI, SPAN, PWA, 0, 0>(acc, cur, dma, sa, row);
+                else if (ks == 1 && KS > 2) mma_group<FP8, MI, NI, SPAN, PWA, G>(acc, cur, dma, sa, row);
+                else if (ks == 2 && KS > 3) mma_group<FP8, MI, NI, SPAN, PWA, 2 * G>(acc, cur, dma, sa, row);
+                else mma_group<FP8, MI, NI, 1, 0, 0, FP8 ? 2 : 0>(acc, cur, none, sa, row);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
-    // what the first stage's closing wait is for (X1 went out with the ring's first fill)
+    // what the first stage's waits are for (X1 went out with the ring's first fill)
 #pragma unroll
-    for (int d = 0; d < PWB; ++d) dmaY(3, 1, d);
-    for (int j = 0;;) {
-        stage(IC<0>{}, j); if (++j == nk) break;
-        stage(IC<1>{}, j); if (++j == nk) break;
-        stage(IC<2>{}, j); if (++j == nk) break;
-        stage(IC<3>{}, j); if (++j == nk) break;
-        stage(IC<4>{}, j); if (++j == nk) break;
+    for (int d = RY; d < PWB; ++d) dmaY(3, 1, d);
+#pragma unroll
+    for (int d = 0; d < RY; ++d) ldY(IC<0>{}, 2, d);
+    if constexpr (kRegY) {
+        for (int j = 0;;) {
+            stage(IC<0>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<1>{}, IC<1>{}, j); if (++j == nk) break;
+            stage(IC<2>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<3>{}, IC<1>{}, j); if (++j == nk) break;
+            stage(IC<4>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<0>{}, IC<1>{}, j); if (++j == nk) break;
+            stage(IC<1>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<2>{}, IC<1>{}, j); if (++j == nk) break;
+            stage(IC<3>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<4>{}, IC<1>{}, j); if (++j == nk) break;
+        }
+    } else {
+        for (int j = 0;;) {
+            stage(IC<0>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<1>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<2>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<3>{}, IC<0>{}, j); if (++j == nk) break;
+            stage(IC<4>{}, IC<0>{}, j); if (++j == nk) break;
+        }
     }
-    // nothing may still be writing this workgroup's LDS when its wavefronts retire
+    // nothing may still be writing this workgroup's LDS when its wavefronts retire -- nor the registers of the loads
+    // that were asked for past the last stage: those registers stay taken until the wait is over (the compiler,
+    // which keeps no book on these loads, would hand them to the epilogue's first values otherwise)
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (kRegY) {
+#pragma unroll
+        for (int jj = 0; jj < RY; ++jj) asm volatile("" : : "v"(yreg[0][jj]), "v"(yreg[1][jj]));
+    }
+    if constexpr (kMX) {
+#pragma unroll
+        for (int i = 0; i < NSLOT; ++i)
+#pragma unroll
+            for (int mi = 0; mi < MI; ++mi) asm volatile("" : : "v"(sc[i][mi]));
+    }
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- epilogue.  Accumulator layout of a 32x32 tile: lane -> column lane%32,
     //      register i -> row 8*(i/4) + 4*(lane/32) + i%4  (4 consecutive rows per register quad).
