@@ -730,7 +730,8 @@ int step_bf16(ghip_net* n, int64_t row0, int batch)
             memset(&g, 0, sizeof(g));
             g.A = n->D[l + 1]; g.B = n->WhT[l]; g.M = B; g.N = ni; g.K = no;
             g.ldb = 64; g.kstrideB = (long long)ni * 128;   // W^T is kept K-blocked: [n_out / 64][n_in][64]
-            g.epilogue = LP_DGRAD; g.out = n->D[l]; g.outT = n->DT[l]; g.outT_blocked = 1; g.aux = n->H[l]; g.colsum = n->csum[l];
+            // (the first hidden layer's deltas have one reader, the first layer's weight gradient, which takes them transposed)
+            g.epilogue = LP_DGRAD; g.out = l > 1 ? n->D[l] : nullptr; g.outT = n->DT[l]; g.outT_blocked = 1; g.aux = n->H[l]; g.colsum = n->csum[l];
             g.mask_in = n->Hmask[l];   // where the activation below is a ReLU: its signs as the forward product left them
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1];
             LAUNCH(n, "gemm_bf16_dgrad", ghip_gemm_lp(g, n->stream));

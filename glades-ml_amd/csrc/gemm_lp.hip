@@ -731,7 +731,10 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
             __builtin_amdgcn_s_waitcnt(0xC07F);
             __builtin_amdgcn_s_barrier();
         }
-        // row-major copy: LDS[m][n]
+        // row-major copy: LDS[m][n] (back-propagation's last product has no reader for it: the deltas of the first
+        // hidden layer are only read transposed, by the first layer's weight gradient)
+        const bool row_major = !(kDgrad && !g.out);
+        if (row_major) {
         if constexpr (EPI != LP_FP8_ACT && !kActMX)
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi)
@@ -807,6 +810,7 @@ __device__ __forceinline__ void gemm_lp_tile(const GemmLpArgs& g, int id, unsign
             if (lane % LPR == 0)
 #pragma unroll
                 for (int i = 0; i < NIT; ++i) atomicMax(&g.row_amax_bits[bm + w * (TM / 8) + i * RPI + lane / LPR], am[i] << 16);
+        }
         }
     }
     if constexpr (kDgrad) {
@@ -966,7 +970,7 @@ hipError_t ghip_gemm_lp_wgrad_group(const GemmLpArgs* a, int count, const unsign
     memset(&grp, 0, sizeof(grp));
     int total = 0;
     for (int i = 0; i < count; ++i) {
-        if (a[i].fp8 || a[i].epilogue != LP_WGRAD_SGD || !operands_ok(a[i]) || use_small_tile(a[i].M, a[i].N)) return hipErrorInvalidValue;
+        if (a[i].fp8 || a[i].epilogue != LP_WGRAD_SGD || !operands_ok(a[i]) || use_small_tile(a[i].M, a[i].N) || !a[i].out) return hipErrorInvalidValue;
         grp.p[i] = a[i];
         resolve_act(grp.p[i]);
         total += (a[i].M / 256) * (a[i].N / 256);
@@ -980,6 +984,7 @@ hipError_t ghip_gemm_lp_wgrad_group(const GemmLpArgs* a, int count, const unsign
 hipError_t ghip_gemm_lp(const GemmLpArgs& a_, hipStream_t s)
 {
     if (!operands_ok(a_)) return hipErrorInvalidValue;
+    if (!a_.out && !(a_.epilogue == LP_DGRAD && a_.outT)) return hipErrorInvalidValue;   // only back-propagation may leave the row-major copy out
     GemmLpArgs a = a_;
     resolve_act(a);
     if (!a.fp8) {

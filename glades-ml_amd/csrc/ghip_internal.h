@@ -425,7 +425,7 @@ struct GemmLpArgs {
     int n_valid;                      // LP_FWD_ACT / LP_FP8_ACT: columns from here on are padding and are stored as 0 (0: none)
     int fp8;                          // 0: bf16 operands, 1: e4m3 operands
     int epilogue;
-    void* out; void* outT;            // see LpEpilogue; outT may be NULL
+    void* out; void* outT;            // see LpEpilogue; outT may be NULL, and out for LP_DGRAD with outT (only the transposed copy is written)
     const float* bias;                // [N] or NULL
     const uint16_t* aux;              // LP_DGRAD: activations bf16 [M][N]
     // LP_FWD_ACT may leave, and LP_DGRAD take instead of aux, the signs of the stored activations (1 = positive), a bit
