@@ -162,6 +162,8 @@ struct ghip_net {
     float* logits = nullptr;
     bool shadow_dirty = true;
     // grouped weight-gradient launches: the layers of each group, its schedule (device) and number of workgroups
+    // canonical mode's dropout: which of the epochs of flags in exMasks the coming pass uses (ghip_net_set_dropout_masks)
+    int canMaskEpoch = 0;
     int wgGroups = 0;
     int wgCount[GHIP_MAX_LAYERS] = {};
     int wgLayer[GHIP_MAX_LAYERS][GHIP_GEMM_LP_GROUP_MAX] = {};
@@ -449,6 +451,7 @@ int reserve_batch(ghip_net* n, int batch)
     for (int l = 0; l <= L; ++l) if (ps[l] > maxw) maxw = ps[l];
     if (s.dtype == GHIP_F32) {
         TRY(dalloc(&n->stageX, (size_t)B * s.sizes[0]));
+        TRY(dalloc(&n->act[0], (size_t)B * s.sizes[0]));   // a batch's rows under its dropout flags
         for (int l = 1; l <= L; ++l) {
             TRY(dalloc(&n->act[l], (size_t)B * s.sizes[l]));
             TRY(dalloc(&n->dlt[l], (size_t)B * s.sizes[l]));
@@ -511,10 +514,34 @@ int out_act(const ghip_net_spec& s, int l, float* param)
 }
 
 // ---- canonical fp32 ----
-int forward_f32(ghip_net* n, const float* X, int B, int layers)
+// Dropout flags of canonical mode (fp32): per row of the table the node layers below the output side by side, 1 = dropped
+// (the layout exact mode takes).  A dropped node's activation is stored as 0, so the layer above gets nothing from it,
+// and its delta is 0 (network.cpp:476-480 carried over to batches; no rescaling, as in the reference).
+int canon_nodes(const ghip_net* n)
+{
+    int t = 0;
+    for (int l = 0; l < n->spec.n_layers; ++l) t += n->spec.sizes[l];
+    return t;
+}
+bool canon_drop_on(const ghip_net* n) { return n->spec.mode == GHIP_MODE_CANONICAL && n->canMaskEpoch < n->exMaskEpochs; }
+// the flags of table row `row0` in the epoch the coming pass uses, or NULL
+const uint8_t* canon_drop(const ghip_net* n, int64_t row0)
+{
+    if (!canon_drop_on(n)) return nullptr;
+    return n->exMasks + ((int64_t)n->canMaskEpoch * n->n_rows + row0) * canon_nodes(n);
+}
+
+// drop: the flags of the batch's first row (canon_drop) or NULL; with flags the batch's rows enter through act[0]
+int forward_f32(ghip_net* n, const float* X, int B, int layers, const uint8_t* drop = nullptr)
 {
     const ghip_net_spec& s = n->spec;
     const float* in = X;
+    const int nodes = canon_nodes(n);
+    int node0 = s.sizes[0];   // where the flags of layer l + 1's nodes start within a row's
+    if (drop) {
+        LAUNCH(n, "dropout_input", ghip_mask_rows(X, drop, nodes, B, s.sizes[0], n->act[0], n->stream));
+        in = n->act[0];
+    }
     for (int l = 0; l < layers; ++l) {
         GemmF32Args g;
         memset(&g, 0, sizeof(g));
@@ -524,6 +551,8 @@ int forward_f32(ghip_net* n, const float* X, int B, int layers)
         g.epilogue = EPI_BIAS_ACT; g.bias = n->b[l];
         g.act = out_act(s, l, &g.act_param);
         g.alpha = 1.0f;
+        const uint8_t* const drop_out = (drop && l + 1 < s.n_layers) ? drop + node0 : nullptr;   // the flags of this layer's nodes
+        node0 += s.sizes[l + 1];
         if (l == s.n_layers - 1 && ghip_narrow_out_ok(g.N, g.K) && ((uintptr_t)in % 16) == 0) {
             NarrowOutArgs a;
             memset(&a, 0, sizeof(a));
@@ -532,6 +561,8 @@ int forward_f32(ghip_net* n, const float* X, int B, int layers)
             LAUNCH(n, "narrow_out_forward", ghip_narrow_forward(a, n->stream));
         } else
             LAUNCH(n, "gemm_f32_forward", ghip_gemm_f32(g, n->stream));
+        // (a pass of its own rather than a branch in the product's epilogue, which every network without flags would carry)
+        if (drop_out) LAUNCH(n, "dropout_activations", ghip_mask_rows(n->act[l + 1], drop_out, nodes, B, s.sizes[l + 1], n->act[l + 1], n->stream));
         in = n->act[l + 1];
     }
     return 0;
@@ -572,6 +603,7 @@ int output_delta_f32(ghip_net* n, float* P, const float* Y, float* D, uint16_t* 
 // (13 us + 0.14 us per thousand of them against 50 us of launches).
 bool use_narrow(const ghip_net* n, int batch)
 {
+    if (canon_drop_on(n)) return false;   // the flags are read by the launches' epilogues
     if (!n->narrow_fit || n->canon_path == GHIP_CANON_PATH_LAUNCHES) return false;
     if (n->canon_path == GHIP_CANON_PATH_ONE_WORKGROUP) return true;
     long long macs = 0;
@@ -612,9 +644,13 @@ int step_f32(ghip_net* n, int64_t row0, int B)
     const int L = s.n_layers;
     const float* X = n->dX + row0 * s.sizes[0];
     const float* Y = n->dY + row0 * s.sizes[L];
-    // an output layer of a few units: its forward, the output delta and its backward are one launch
-    const bool narrow = n->narrowPart && ((uintptr_t)(L == 1 ? X : n->act[L - 1]) % 16) == 0;
-    TRY(forward_f32(n, X, B, narrow ? L - 1 : L));
+    const uint8_t* drop = canon_drop(n, row0);
+    const int nodes = canon_nodes(n);
+    // an output layer of a few units: its forward, the output delta and its backward are one launch (without dropout
+    // flags: that launch's backward does not read them)
+    const bool narrow = !drop && n->narrowPart && ((uintptr_t)(L == 1 ? X : n->act[L - 1]) % 16) == 0;
+    TRY(forward_f32(n, X, B, narrow ? L - 1 : L, drop));
+    if (drop) X = n->act[0];   // the rows as the first layer saw them
     if (!narrow) TRY(output_delta_f32(n, n->act[L], Y, n->dlt[L], nullptr, B));
     // The weight gradients (with their updates) only need the deltas, which the back-propagation products
     // leave layer by layer, and write what those products read (the weights): so they wait until the
@@ -652,6 +688,11 @@ int step_f32(ghip_net* n, int64_t row0, int B)
             g.epilogue = EPI_MUL_DER; g.aux = n->act[l];
             g.act = s.act[l - 1]; g.act_param = s.act_param[l - 1]; g.alpha = 1.0f;
             LAUNCH(n, "gemm_f32_dgrad", ghip_gemm_f32(g, n->stream));
+            if (drop) {
+                int node0 = 0;
+                for (int k = 0; k < l; ++k) node0 += s.sizes[k];
+                LAUNCH(n, "dropout_deltas", ghip_mask_rows(n->dlt[l], drop + node0, nodes, B, ni, n->dlt[l], n->stream));
+            }
         }
         // gradient D^T A / B and, in the same kernel's epilogue, the update of the weights (momentum,
         // both decays) and of the bias (batch mean of the delta = the row sums of the A operand)
@@ -1071,14 +1112,16 @@ int ghip_net_set_dropout_masks(ghip_net* n, const uint8_t* host_masks, int n_epo
 {
     if (!n) return fail(GHIP_EINVAL, "bad net");
     HIP_TRY(hipSetDevice(g_device));
-    if (n->spec.mode != GHIP_MODE_EXACT) return fail(GHIP_ESTATE, "dropout flags belong to exact mode");
+    if (n->spec.mode != GHIP_MODE_EXACT && n->spec.dtype != GHIP_F32)
+        return fail(GHIP_ESTATE, "dropout flags are taken in exact mode and by fp32 networks in canonical mode");
+    n->canMaskEpoch = 0;
     if (!host_masks) {
         n->exMaskEpochs = 0;
         return 0;
     }
     if (n_epochs < 1) return fail(GHIP_EINVAL, "bad arguments");
     if (!n->dX || !n->dY) return fail(GHIP_ESTATE, "no dataset (the flags are per row of the table)");
-    const int64_t len = (int64_t)n_epochs * n->n_rows * n->ex.aoff[n->L];
+    const int64_t len = (int64_t)n_epochs * n->n_rows * canon_nodes(n);
     for (int64_t k = 0; k < len; ++k)
         if (host_masks[k] > 1) return fail(GHIP_EINVAL, "flag %lld is %d, not 0 or 1", (long long)k, (int)host_masks[k]);
     // a layer with every node dropped would never finalise the next layer (Layer::lastValidPath,
@@ -1421,7 +1464,7 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
             rc = (s.dtype == GHIP_F32) ? step_f32(n, r0, b) : step_bf16(n, r0, b);
         } else {
             float* P = nullptr;
-            if (s.dtype == GHIP_F32) { rc = forward_f32(n, n->dX + r0 * s.sizes[0], b, L); P = n->act[L]; }
+            if (s.dtype == GHIP_F32) { rc = forward_f32(n, n->dX + r0 * s.sizes[0], b, L, canon_drop(n, r0)); P = n->act[L]; }
             else if (s.dtype == GHIP_BF16) { rc = forward_bf16(n, n->Xbf + r0 * n->ps[0], b); P = n->logits; }
             else { rc = forward_fp8(n, n->Xbf + r0 * n->ps[0], b, n->out8); P = n->out8; }
             if (rc == 0) rc = output_delta_f32(n, P, n->dY + r0 * s.sizes[L], nullptr, nullptr, b);
@@ -1430,6 +1473,7 @@ int ghip_net_run_epoch_canonical(ghip_net* n, int batch, int train, ghip_metrics
     }
     n->passAcc = false;
     if (rc != 0) return rc;
+    if (canon_drop_on(n)) ++n->canMaskEpoch;   // the next pass takes the next epoch's flags; past the last, none
     double acc[4];
     HIP_TRY(hipMemcpyAsync(acc, n->dAcc + 12, sizeof(acc), hipMemcpyDeviceToHost, n->stream));
     HIP_TRY(hipStreamSynchronize(n->stream));
@@ -1449,6 +1493,8 @@ int ghip_net_run_epochs_canonical(ghip_net* n, int batch, int n_epochs, int trai
     const ghip_net_spec& s = n->spec;
     const int64_t N = n->n_rows;
     if (batch > N) batch = (int)N;
+    if (canon_drop_on(n) && n_epochs > n->exMaskEpochs - n->canMaskEpoch)
+        return fail(GHIP_EINVAL, "%d epochs asked for, dropout flags for %d", n_epochs, n->exMaskEpochs - n->canMaskEpoch);
     if (s.dtype == GHIP_F32 && use_narrow(n, batch)) {
         // narrow network: the epochs are one launch, the stop condition is looked at on the device
         if (n_epochs > n->narrowEpochsCap) {
@@ -1629,7 +1675,7 @@ int ghip_net_eval_resident(ghip_net* n, int64_t row0, int batch, ghip_metrics* h
     TRY(reserve_batch(n, batch));
     const int L = s.n_layers;
     float* P = nullptr;
-    if (s.dtype == GHIP_F32) { TRY(forward_f32(n, n->dX + row0 * s.sizes[0], batch, L)); P = n->act[L]; }
+    if (s.dtype == GHIP_F32) { TRY(forward_f32(n, n->dX + row0 * s.sizes[0], batch, L, canon_drop(n, row0))); P = n->act[L]; }
     else if (s.dtype == GHIP_BF16) { TRY(refresh_shadows(n)); TRY(forward_bf16(n, n->Xbf + row0 * n->ps[0], batch)); P = n->logits; }
     else { TRY(forward_fp8(n, n->Xbf + row0 * n->ps[0], batch, n->out8)); P = n->out8; }
     TRY(output_delta_f32(n, P, n->dY + row0 * s.sizes[L], nullptr, nullptr, batch));

@@ -535,6 +535,26 @@ inline int grid_for(long long n, int cap = 65535 * 4)
 
 }  // namespace
 
+__global__ void __launch_bounds__(256) mask_rows_kernel(const float* X, const uint8_t* __restrict__ drop, int ld_drop,
+                                                        long long total, int cols, float* out)
+{
+    for (long long k = (long long)blockIdx.x * 256 + threadIdx.x; k < total; k += (long long)gridDim.x * 256) {
+        const long long r = k / cols;
+        const int c = (int)(k - r * cols);
+        out[k] = drop[r * ld_drop + c] ? 0.0f : X[k];
+    }
+}
+
+hipError_t ghip_mask_rows(const float* X, const uint8_t* drop, int ld_drop, int rows, int cols, float* out, hipStream_t s)
+{
+    const long long total = (long long)rows * cols;
+    if (total <= 0) return hipSuccess;
+    long long blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(mask_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, s, X, drop, ld_drop, total, cols, out);
+    return hipGetLastError();
+}
+
 hipError_t ghip_output_delta(const DeltaArgs& a, hipStream_t s)
 {
     const bool vec_ok = (a.n % 4) == 0 && a.n <= 2048 && (a.ldp % 4) == 0 && (!a.Y || (a.ldy % 4) == 0) &&

@@ -317,6 +317,9 @@ struct GemmF32Args {
     float* bias_w; float* bias_v;
 };
 hipError_t ghip_gemm_f32(const GemmF32Args& a, hipStream_t s);
+// out[r][c] = drop[r * ld_drop + c] ? 0 : X[r][c] (out may be X): a batch's rows, activations or deltas under its
+// dropout flags
+hipError_t ghip_mask_rows(const float* X, const uint8_t* drop, int ld_drop, int rows, int cols, float* out, hipStream_t s);
 // up to GHIP_GEMM_F32_GROUP_MAX independent products in one launch where they run the same instantiation
 // (tile height, operand orientations, alignment class), else one launch each
 #define GHIP_GEMM_F32_GROUP_MAX 8

@@ -778,7 +778,9 @@ bool NNetwork::build()
     pNode[0] = skeleton->getPInput();
     for (int h = 0; h < H; ++h) pNode[h + 1] = skeleton->getPDropout(h);
     dropoutOn = hasDropout();
-    if (dropoutOn && mode != MODE_EXACT) { lastError = "dropout follows the reference's per-row algorithm: exact mode only"; return false; }
+    // exact mode follows the reference's per-row algorithm with the flags; canonical mode in fp32 takes the same flags
+    // (a dropped node feeds nothing on and gets no delta); the low-precision kernels do not read flags
+    if (dropoutOn && mode != MODE_EXACT && dtype != DTYPE_F32) { lastError = "dropout: exact mode, or canonical mode in fp32"; return false; }
     dropFlags.clear();
     s.batch = skeleton->getBatchSize();
     s.cost = skeleton->getOutputType();
@@ -1278,9 +1280,14 @@ void NNetwork::run(DataInput* newDataInput, int runType)
             // stop conditions allow it: a narrow network then runs them as one launch, any other pass by pass with
             // every step of a pass enqueued back to back and the metrics added up on the device.
             const int mb = minibatchSize > 0 ? minibatchSize : (int)nRows;
-            const int chunk = epochChunk(terminator, epochs, runType);
+            // with dropout one epoch per call: the flags come from libc rand() as the epoch starts, as in exact mode
+            const int chunk = dropoutOn ? 1 : epochChunk(terminator, epochs, runType);
             std::vector<ghip_metrics> ms(chunk);
             int ran = 0;
+            if (dropoutOn) {
+                drawDropout();
+                if (ghip_net_set_dropout_masks(dev, dropFlags.data(), 1) != 0) { lastError = ghip_last_error(); break; }
+            }
             if (ghip_net_run_epochs_canonical(dev, mb, chunk, runType == RUN_TRAIN ? 1 : 0, terminator.getAccuracy(), ms.data(), &ran) != 0) {
                 lastError = ghip_last_error();
                 break;

@@ -151,7 +151,14 @@ int ghip_net_set_state(ghip_net* net, int layer, const float* host_a, const floa
  * ML/Networks/network.cpp:407-411) consumes them and must not ask for more epochs; later calls run
  * without dropout until flags are set again.  A row that drops every node of a layer is refused
  * (the reference redraws such a layer).  Needs the table (ghip_net_set_dataset) first.
- * NULL forgets flags that were set. */
+ * NULL forgets flags that were set.
+ * Canonical mode, fp32 networks: the same flags in the same layout.  A dropped node's activation is taken as 0 by
+ * the layer above (the reference skips every edge that leaves it, ML/Networks/network.cpp:476-480, and rescales
+ * nothing) and it gets no delta, in training and test passes alike.  Every pass of ghip_net_run_epoch_canonical /
+ * ghip_net_run_epochs_canonical uses up one epoch of flags (a call may not ask for more epochs than are left);
+ * ghip_net_train_step and ghip_net_eval_resident read the flags of their rows in the epoch that is next, without
+ * using it up; ghip_net_forward* never drop.  Past the last epoch of flags the network runs without dropout.
+ * bf16 / e4m3 networks refuse flags. */
 int ghip_net_set_dropout_masks(ghip_net* net, const uint8_t* host_masks, int n_epochs);
 /* What dropout leaves behind between rows, for checkpoints: the number of pending deltas of every
  * edge of weight layer `layer` (Edge::prevDelta.size(), ML/State/edge.cpp:64-67; sizes[layer+1] x

@@ -506,6 +506,7 @@ struct go_canon {
     float* a[GO_MAX_LAYERS + 1]; /* [B][n] activations */
     float* d[GO_MAX_LAYERS + 1]; /* [B][n] deltas (dL/dz) */
     int64_t cap;
+    const uint8_t* drop;         /* go_canon_set_drop: the coming batch's flags, or NULL */
 };
 
 go_canon* go_canon_create(const go_spec* spec)
@@ -625,14 +626,40 @@ static void canon_activate(const go_spec* s, int l, float* Z, int64_t B)
     }
 }
 
+/* Dropout in canonical mode.  The flags are the reference's: one per row and node of the input and hidden
+ * layers (Layer::generateDropout, layer.cpp:102-134), and a dropped node feeds nothing on: the reference skips
+ * every edge that leaves it (possiblePath, network.cpp:476-480), with no rescaling of the others.  Batched, that
+ * is the node's activation taken as 0 by the layer above; back-propagation through the same function gives the
+ * dropped node no delta, so the weights into it and its bias get no gradient from that row. */
+static int canon_nodes(const go_spec* s)
+{
+    int t = 0;
+    for (int l = 0; l < s->n_layers; ++l) t += s->sizes[l];
+    return t;
+}
+static void canon_drop(const go_canon* n, int l, float* A, int64_t B)
+{
+    if (!n->drop) return;
+    const go_spec* s = &n->s;
+    const int nodes = canon_nodes(s), nl = s->sizes[l];
+    int off = 0;
+    for (int k = 0; k < l; ++k) off += s->sizes[k];
+    for (int64_t b = 0; b < B; ++b)
+        for (int i = 0; i < nl; ++i)
+            if (n->drop[b * nodes + off + i]) A[b * nl + i] = 0.0f;
+}
+void go_canon_set_drop(go_canon* n, const uint8_t* flags) { n->drop = flags; }
+
 static void canon_forward_all(go_canon* n, const float* X, int64_t B)
 {
     const go_spec* s = &n->s;
     canon_reserve(n, B);
     memcpy(n->a[0], X, sizeof(float) * B * s->sizes[0]);
+    canon_drop(n, 0, n->a[0], B);
     for (int l = 0; l < s->n_layers; ++l) {
         canon_layer_forward(n->W[l], n->b[l], n->a[l], n->a[l + 1], B, s->sizes[l], s->sizes[l + 1]);
         canon_activate(s, l, n->a[l + 1], B);
+        if (l + 1 < s->n_layers) canon_drop(n, l + 1, n->a[l + 1], B);
     }
 }
 
@@ -753,6 +780,7 @@ void go_canon_step(go_canon* n, const float* X, const float* Y, int64_t B, go_me
             const float* a = n->a[l];
 #pragma omp parallel for num_threads(g_threads) schedule(static)
             for (int64_t k = 0; k < B * ni; ++k) d[k] = d[k] * canon_act_der(a[k], act, par);
+            canon_drop(n, l, d, B);
         }
         /* delta_t = lr*(g + wd1*sign(W) + wd2*W) + mom*delta_{t-1};  W -= delta_t */
         const float lr = s->lr[l], mom = s->mom[l], wd1 = s->wd1[l], wd2 = s->wd2[l];

@@ -44,7 +44,8 @@
  *   go_canon_*  no counterpart in the reference (the reference has no batched
  *       training, softmax or per-channel bias): pinned against torch autograd +
  *       torch.optim.SGD and finite differences; forward pinned against go_exact
- *       forward (bit-exact for equal parameters).
+ *       forward (bit-exact for equal parameters, with and without dropout flags);
+ *       go_canon_set_drop pinned by torch autograd through the masked network.
  *   go_cmatrix_*  ML/GMath/cmatrix.cpp needs the un-vendored shmea containers and cannot be
  *       compiled here: restated from the source text -- parity unpinned by execution; pinned
  *       by hand-computed matrices, the perfect-classifier closed form and brute force on
@@ -150,6 +151,10 @@ void  go_canon_step(go_canon* n, const float* X, const float* Y, int64_t B, go_m
 void  go_canon_get_grads(const go_canon* n, int layer, float* gW, float* gb);
 /* mean per-sample loss of a batch without touching parameters */
 double go_canon_loss(go_canon* n, const float* X, const float* Y, int64_t B);
+/* dropout flags for the rows of the calls that follow, [B][sizes[0] + ... + sizes[n_layers-1]] bytes, 1 = dropped
+   (the caller keeps them alive; NULL: none).  A dropped node's activation is taken as 0 by the layer above and
+   it gets no delta (layer.cpp:102-134, network.cpp:476-480 carried over to batches; no rescaling). */
+void  go_canon_set_drop(go_canon* n, const uint8_t* flags);
 void  go_set_threads(int t);
 /* canonical mode: 1 = every sum is walked from its far end (same mathematics, another order of fp32 addition) */
 void  go_set_sum_order(int reversed);

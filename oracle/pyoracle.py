@@ -94,6 +94,7 @@ def lib():
             "go_canon_forward": (None, [vp, f32p, C.c_int64, f32p]),
             "go_canon_step": (None, [vp, f32p, f32p, C.c_int64, C.POINTER(Metrics)]),
             "go_canon_loss": (C.c_double, [vp, f32p, f32p, C.c_int64]),
+            "go_canon_set_drop": (None, [vp, vp]),
             "go_set_threads": (None, [C.c_int]),
             "go_set_sum_order": (None, [C.c_int]),
             "go_bf16_from_f32": (C.c_uint16, [C.c_float]),
@@ -238,17 +239,33 @@ class CanonNet:
     def get_grads(self, l):
         return self._pair(lib().go_canon_get_grads, l)
 
-    def forward(self, X):
+    def _drop(self, drop, B):
+        """dropout flags [B][sum of sizes[:-1]] (1 = dropped) for the call that follows, or None"""
+        if drop is None:
+            lib().go_canon_set_drop(self.h, None)
+            return None
+        drop = np.ascontiguousarray(drop, np.uint8)
+        assert drop.shape == (B, sum(self.sizes[:-1]))
+        lib().go_canon_set_drop(self.h, drop.ctypes.data_as(C.c_void_p))
+        return drop
+
+    def forward(self, X, drop=None):
         X = np.ascontiguousarray(X, np.float32)
         out = np.empty((X.shape[0], self.sizes[-1]), np.float32)
+        keep = self._drop(drop, X.shape[0])
         lib().go_canon_forward(self.h, X, X.shape[0], out)
+        lib().go_canon_set_drop(self.h, None)
+        del keep
         return out
 
-    def step(self, X, Y):
+    def step(self, X, Y, drop=None):
         X = np.ascontiguousarray(X, np.float32)
         Y = np.ascontiguousarray(Y, np.float32)
         m = Metrics()
+        keep = self._drop(drop, X.shape[0])
         lib().go_canon_step(self.h, X, Y, X.shape[0], C.byref(m))
+        lib().go_canon_set_drop(self.h, None)
+        del keep
         return m
 
     def loss(self, X, Y):

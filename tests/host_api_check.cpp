@@ -14,6 +14,8 @@
 //   host_api_check checkpoint <case.bin> <mode> <E1> <E2> <file.ckpt> <out.bin>
 //   host_api_check meta <case.bin> <mode> <k subnets> <epochs> <out.bin>
 //   host_api_check train  <case.bin> <out.bin> <stop_epoch> <stop_accuracy> <mode>
+//   host_api_check dropout <case.bin> <seed> <E1> <E2> <file.ckpt> <out.bin> <rate of the input row> <rates of the hidden rows ...>
+//   host_api_check dropoutcanon <case.bin> <seed> <epochs> <out.bin> <rates as above>      (canonical mode)
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -413,6 +415,40 @@ static int do_dropout(const char* in, int seed, int e1, int e2, const char* ckpt
     return 0;
 }
 
+// Canonical mode with dropout rates in the table: trains `epochs` epochs and runs a test pass under srand(seed).
+// out: epochs, training loss, test accuracy, the next rand() % 65536, then every layer's weights and bias.
+static int do_dropout_canonical(const char* in, int seed, int epochs, const char* out, const std::vector<float>& pd)
+{
+    Case c;
+    int rc = read_case(in, c);
+    if (rc) return rc;
+    if ((int)pd.size() != c.nl) return 6;
+    glades::init();
+    DenseInput di(c.X.data(), c.Y.data(), c.N, c.sizes[0], c.sizes[c.nl]);
+    NNInfo* info = case_info_dropout(c, pd);
+    srand(seed);
+    NNetwork net(info);
+    seed_net(net, c, NNetwork::MODE_CANONICAL);
+    net.setVerbose(false);
+    if (!net.hasDropout()) return 7;
+    net.terminator.setEpoch(epochs);
+    net.train(&di);
+    if (!net.getLastError().empty()) { fprintf(stderr, "train: %s\n", net.getLastError().c_str()); return 5; }
+    const float train_loss = net.getLoss();
+    const int trained = net.getEpochs();
+    std::vector<std::vector<float> > w, bb;
+    for (int l = 0; l < c.nl; ++l) { w.push_back(net.getWeights(l)); bb.push_back(net.getBias(l)); }
+    net.test(&di);  // draws flags as well (network.cpp:407-411)
+    if (!net.getLastError().empty()) { fprintf(stderr, "test: %s\n", net.getLastError().c_str()); return 5; }
+    FILE* fo = fopen(out, "wb");
+    if (!fo) return 1;
+    float head[4] = {(float)trained, train_loss, net.getAccuracy(), (float)(rand() % 65536)};
+    fwrite(head, 4, 4, fo);
+    for (size_t k = 0; k < w.size(); ++k) { put(w[k], fo); put(bb[k], fo); }
+    fclose(fo);
+    return 0;
+}
+
 // A trains E1 epochs and saves; B restores and trains on to E1 + E2; C trains E1 + E2 in one go.
 // out: epochs of B and C, then every layer's weights and bias of B, then of C.
 static int do_checkpoint(const char* in, int mode, int e1, int e2, const char* ckpt, const char* out)
@@ -558,6 +594,11 @@ int main(int argc, char** argv)
         std::vector<float> pd;
         for (int k = 8; k < argc; ++k) pd.push_back((float)atof(argv[k]));
         return do_dropout(argv[2], atoi(argv[3]), atoi(argv[4]), atoi(argv[5]), argv[6], argv[7], pd);
+    }
+    if (argc >= 7 && !strcmp(argv[1], "dropoutcanon")) {
+        std::vector<float> pd;
+        for (int k = 6; k < argc; ++k) pd.push_back((float)atof(argv[k]));
+        return do_dropout_canonical(argv[2], atoi(argv[3]), atoi(argv[4]), argv[5], pd);
     }
     if (argc >= 2 && !strcmp(argv[1], "ohe")) return do_ohe();
     if (argc >= 5 && !strcmp(argv[1], "numberinput")) return do_numberinput(argv[2], argv[3], argv[4]);

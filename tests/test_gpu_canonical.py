@@ -455,3 +455,113 @@ def test_one_workgroup_small_table_in_several_batches(N, B):
         np.testing.assert_allclose(g.get_params(l)[0], o.get_params(l)[0], rtol=1e-4, atol=2e-6)
         np.testing.assert_allclose(g.get_params(l)[1], o.get_params(l)[1], rtol=1e-4, atol=2e-6)
     g.close()
+
+
+DROPOUT_CASES = [c for c in CASES if c[0] in ("relu_softmax_ragged", "cfg3_like_small", "sigmoid_bce", "cfg2_shape_tanh_mse",
+                                              "leaky_sigmoidp_kl", "narrow_16_out_chunks_of_8_rows", "mixed_weight_gradient_tiles")]
+
+
+def _flags(rng, rows, sizes, rate=0.3):
+    """per row the node layers below the output side by side, 1 = dropped; no row drops a whole layer"""
+    nodes = sum(sizes[:-1])
+    m = (rng.random((rows, nodes)) < rate).astype(np.uint8)
+    off = 0
+    for n in sizes[:-1]:
+        m[:, off] = 0
+        off += n
+    return m
+
+
+@pytest.mark.parametrize("name,sizes,acts,params,cost,B", DROPOUT_CASES, ids=[c[0] for c in DROPOUT_CASES])
+def test_dropout_steps_match_cpu(name, sizes, acts, params, cost, B):
+    """Canonical mode with the reference's dropout flags (per row and node of the input and hidden layers, a dropped
+    node feeds nothing on, no rescaling): training steps, a test pass and forward calls against the CPU restatement,
+    which torch autograd through the masked network pins (tests/test_oracle_canonical.py).  Narrow networks and
+    narrow output layers, which have kernels of their own without flags, are among the shapes."""
+    print("canonical dropout", name, flush=True)
+    o, g, rng = build_pair(sizes, acts, params, cost, 0.05, 0.9, 1e-4, 1e-3, 29, path="auto")
+    nl = len(sizes) - 1
+    steps = 5
+    N = B * steps
+    X = rng.standard_normal((N, sizes[0])).astype(np.float32)
+    if cost == po.REGRESSION:
+        Y = rng.standard_normal((N, sizes[-1])).astype(np.float32)
+    elif cost == po.KL:
+        Y = rng.random((N, sizes[-1])).astype(np.float32) * 0.8 + 0.1
+    else:
+        Y = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], N)]
+    g.set_dataset(X, Y)
+    masks = np.stack([_flags(rng, N, sizes), _flags(rng, N, sizes)])      # two epochs of flags
+    g.set_dropout_masks(masks)
+    # epoch 0 of the flags: a training pass step by step (the steps read the flags of the epoch that is next) ...
+    for s_ in range(steps):
+        r = slice(s_ * B, (s_ + 1) * B)
+        mo = o.step(X[r], Y[r], masks[0][r])
+        mg = g.train_step(s_ * B, B)
+        assert abs(mg.loss - mo.loss) <= 1e-4 * abs(mo.loss) + 1e-6, (s_, mg.loss, mo.loss)
+        assert abs(mg.correct - mo.correct) <= 1
+    for l in range(nl):
+        Wo, bo = o.get_params(l)
+        Wg, bg = g.get_params(l)
+        # (3e-5 absolute: the L1 term's sign(W) flips for the few weights that sit within rounding distance of zero)
+        np.testing.assert_allclose(Wg, Wo, rtol=1e-4, atol=3e-5, err_msg=f"layer {l}")
+        np.testing.assert_allclose(bg, bo, rtol=1e-4, atol=3e-6, err_msg=f"layer {l} bias")
+    # ... then a test pass over the table, which uses epoch 0 up ...
+    me = g.run_epoch_canonical(B, train=False)
+    # the restated pass: a step at learning rate 0 reports the forward loss under the same flags and changes nothing
+    oz = po.CanonNet(po.make_spec(sizes, acts, lr=0.0, mom=0.0, act_params=params, cost=cost))
+    for l in range(nl):
+        oz.set_params(l, *o.get_params(l))
+    tot = 0.0
+    cor = 0
+    for s_ in range(steps):
+        r = slice(s_ * B, (s_ + 1) * B)
+        mz = oz.step(X[r], Y[r], masks[0][r])
+        tot += mz.loss * B
+        cor += mz.correct
+    assert abs(me.loss - tot / N) <= 1e-4 * abs(tot / N) + 1e-6, (me.loss, tot / N)
+    assert abs(me.correct - cor) <= 2
+    # ... so the next pass trains under epoch 1's flags, and the one after that without any
+    m1 = g.run_epoch_canonical(B, train=True)
+    tot = 0.0
+    for s_ in range(steps):
+        r = slice(s_ * B, (s_ + 1) * B)
+        tot += o.step(X[r], Y[r], masks[1][r]).loss * B
+    assert abs(m1.loss - tot / N) <= 1e-4 * abs(tot / N) + 1e-6, (m1.loss, tot / N)
+    m2 = g.run_epoch_canonical(B, train=True)
+    tot = 0.0
+    for s_ in range(steps):
+        r = slice(s_ * B, (s_ + 1) * B)
+        tot += o.step(X[r], Y[r]).loss * B
+    assert abs(m2.loss - tot / N) <= 1e-4 * abs(tot / N) + 1e-6, (m2.loss, tot / N)
+    for l in range(nl):
+        Wo, bo = o.get_params(l)
+        Wg, bg = g.get_params(l)
+        np.testing.assert_allclose(Wg, Wo, rtol=2e-4, atol=1e-4, err_msg=f"layer {l} after three passes")
+    # forward calls never drop
+    np.testing.assert_allclose(g.forward(X[:B]), o.forward(X[:B]), rtol=1e-4, atol=1e-5)
+    g.close()
+
+
+def test_dropout_flags_error_paths():
+    import pyglades as pg
+    rng = np.random.default_rng(3)
+    sizes, acts = [8, 12, 4], [po.TANH, po.SOFTMAX]
+    X = rng.standard_normal((40, 8)).astype(np.float32)
+    Y = np.eye(4, dtype=np.float32)[rng.integers(0, 4, 40)]
+    g = pg.Net(pg.make_spec(sizes, acts, lr=0.1, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=pg.F32))
+    g.set_dataset(X, Y)
+    g.set_dropout_masks(_flags(rng, 40, sizes)[None])
+    with pytest.raises(pg.GladesHipError):
+        g.run_epochs_canonical(10, 2)                      # two epochs asked for, flags for one
+    assert len(g.run_epochs_canonical(10, 1)) == 1
+    bad = _flags(rng, 40, sizes)[None].copy()
+    bad[0, 3, :8] = 1                                      # a row that drops the whole input layer
+    with pytest.raises(pg.GladesHipError):
+        g.set_dropout_masks(bad)
+    g.close()
+    h = pg.Net(pg.make_spec([256, 256, 256], acts, lr=0.1, cost=pg.CLASSIFICATION, mode=pg.MODE_CANONICAL, dtype=pg.BF16))
+    h.set_dataset(rng.standard_normal((256, 256)).astype(np.float32), np.eye(256, dtype=np.float32))
+    with pytest.raises(pg.GladesHipError):
+        h.set_dropout_masks(np.zeros((1, 256, 512), np.uint8))
+    h.close()

@@ -476,6 +476,52 @@ def test_dropout_through_the_class_api_follows_the_rand_stream():
 
 
 @needs_bin
+@pytest.mark.gpu
+def test_dropout_in_canonical_mode_through_the_class_api():
+    """NNInfo rows with dropout rates in canonical mode (fp32): the class draws an epoch's flags from libc rand() in
+    the reference's order as the epoch starts, exactly as in exact mode, hands them to the library and runs the epoch's
+    batches; the test pass draws flags too.  Against the CPU restatement fed from the same srand(seed) stream:
+    weights, biases, loss, the test pass's accuracy, and where rand() stands afterwards."""
+    c = load_case("batch1_5_7_6_4", "dropout")
+    seed, epochs = 5, 4
+    rows = [0.2, 0.3, 0.9]                      # input row, hidden row 0, hidden row 1 (never used)
+    resolved = np.array([0.2, 0.2, 0.3], np.float32)   # node layers 0, 1, 2
+    mb = c["mb"]
+    with tempfile.TemporaryDirectory() as td:
+        cin, cout = os.path.join(td, "c.bin"), os.path.join(td, "o.bin")
+        write_case(cin, c)
+        subprocess.check_call([BIN, "dropoutcanon", cin, str(seed), str(epochs), cout] + [str(p) for p in rows], stdout=subprocess.DEVNULL)
+        raw = np.fromfile(cout, np.float32)
+    assert raw[0] == epochs
+    c["spec"].wd2[0] = c["spec"].wd1[0]   # NNInfo::getWeightDecay2(0) returns the input row's weightDecay1 (nninfo.cpp:305-306)
+    o = po.CanonNet(c["spec"])
+    for l in range(c["nl"]):
+        o.set_params(l, c["W0"][l])         # the driver injects the weights; canonical biases start at zero
+    po.libc_srand(seed)
+    N, dropped = c["N"], 0
+    for _ in range(epochs):
+        masks = po.dropout_draw(c["spec"], resolved, N)
+        dropped += int(masks.sum())
+        tot = 0.0
+        for r0 in range(0, N, mb):
+            r = slice(r0, min(r0 + mb, N))
+            tot += o.step(c["X"][r], c["Y"][r], masks[r]).loss * (r.stop - r.start)
+    assert dropped > 0
+    np.testing.assert_allclose(raw[1], tot / N, rtol=1e-4)
+    masks = po.dropout_draw(c["spec"], resolved, N)      # the test pass
+    assert int(raw[3]) == po.libc_rand() % 65536         # both sides consumed the same number of draws
+    pos = 4
+    for l in range(c["nl"]):
+        n = c["sizes"][l] * c["sizes"][l + 1]
+        W = raw[pos:pos + n].reshape(c["sizes"][l + 1], c["sizes"][l])
+        b = raw[pos + n:pos + n + c["sizes"][l + 1]]
+        pos += n + c["sizes"][l + 1]
+        Wo, bo = o.get_params(l)
+        np.testing.assert_allclose(W, Wo, rtol=1e-4, atol=2e-6, err_msg=f"layer {l}")
+        np.testing.assert_allclose(b, bo, rtol=1e-4, atol=2e-6, err_msg=f"layer {l} bias")
+
+
+@needs_bin
 def test_whole_network_initialisation_follows_the_reference_order():
     """NNetwork::build's sampling (sampleInitialWeights) against sequences of the reference's compiled
     Layer::initWeights under one srand: the order of LayerBuilder::buildHiddenLayers / buildOutputLayer

@@ -12,9 +12,12 @@ def torch_mlp(sizes, acts, params, Ws, bs):
     Wt = [torch.tensor(w, dtype=torch.float64, requires_grad=True) for w in Ws]
     bt = [torch.tensor(b, dtype=torch.float64, requires_grad=True) for b in bs]
 
-    def fwd(x):
-        a = x
+    def fwd(x, keep=None):
+        """keep: per node layer below the output a [B][n] array of 1 (kept) / 0 (dropped), or None"""
+        a = x if keep is None else x * keep[0]
         for l, (W, b) in enumerate(zip(Wt, bt)):
+            if keep is not None and 0 < l:
+                a = a * keep[l]
             z = a @ W.T + b
             k = acts[l]
             if k == po.RELU:
@@ -85,6 +88,64 @@ def test_steps_match_torch_sgd(name, sizes, acts, params, cost):
         np.testing.assert_allclose(b, bt[l].detach().numpy(), rtol=5e-4, atol=5e-6)
 
 
+@pytest.mark.parametrize("name,sizes,acts,params,cost", CASES)
+def test_dropout_steps_match_torch_autograd_through_the_masked_network(name, sizes, acts, params, cost):
+    """Dropout in canonical mode = the reference's per-row, per-node flags (input and hidden layers, no rescaling)
+    with a dropped node's activation taken as 0 by the layer above.  Stated independently: the torch network
+    multiplies each node layer below the output by its 0/1 keep array, autograd differentiates through that, and
+    torch.optim.SGD steps.  Gradients after the first step, losses of every step and the parameters after six
+    steps agree; so a delta that leaks through a dropped node, a dropped input that still feeds the first layer,
+    or a mask applied to the output layer fails."""
+    rng = np.random.default_rng(11)
+    nl = len(sizes) - 1
+    lr, mom, wd2 = 0.05, 0.9, 1e-3
+    Ws = [(rng.standard_normal((sizes[l + 1], sizes[l])) * (1.5 / np.sqrt(sizes[l]))).astype(np.float32) for l in range(nl)]
+    bs = [(rng.standard_normal(sizes[l + 1]) * 0.1).astype(np.float32) for l in range(nl)]
+    B, steps = 29, 6
+    Xs = rng.standard_normal((steps, B, sizes[0])).astype(np.float32)
+    if cost == po.CLASSIFICATION:
+        Ys = np.eye(sizes[-1], dtype=np.float32)[rng.integers(0, sizes[-1], (steps, B))]
+    else:
+        Ys = rng.standard_normal((steps, B, sizes[-1])).astype(np.float32)
+    nodes = sum(sizes[:-1])
+    drops = (rng.random((steps, B, nodes)) < 0.3).astype(np.uint8)
+    net = po.CanonNet(po.make_spec(sizes, acts, lr=lr, mom=mom, wd2=wd2, act_params=params, batch=B, cost=cost))
+    for l in range(nl):
+        net.set_params(l, Ws[l], bs[l])
+    Wt, bt, fwd = torch_mlp(sizes, acts, params, Ws, bs)
+    opt = torch.optim.SGD([{"params": Wt, "weight_decay": wd2}, {"params": bt, "weight_decay": 0.0}], lr=lr, momentum=mom)
+    offs = np.concatenate([[0], np.cumsum(sizes[:-1])])
+    for s in range(steps):
+        keep = [torch.tensor(1.0 - drops[s][:, offs[l]:offs[l + 1]], dtype=torch.float64) for l in range(nl)]
+        x = torch.tensor(Xs[s], dtype=torch.float64)
+        y = torch.tensor(Ys[s], dtype=torch.float64)
+        p = fwd(x, keep)
+        if acts[-1] == po.SOFTMAX:
+            loss = -(y * torch.log(p)).sum(1).mean()
+        elif cost == po.CLASSIFICATION:
+            loss = -(y * torch.log(p) + (1 - y) * torch.log(1 - p)).sum(1).mean()
+        else:
+            loss = ((p - y) ** 2).sum(1).mean()
+        opt.zero_grad()
+        loss.backward()
+        if s == 0:
+            np.testing.assert_allclose(net.forward(Xs[s], drops[s]), p.detach().numpy(), rtol=2e-5, atol=2e-6)
+        m = net.step(Xs[s], Ys[s], drops[s])
+        if s == 0:
+            for l in range(nl):
+                gW, gb = net.get_grads(l)
+                np.testing.assert_allclose(gW, Wt[l].grad.numpy(), rtol=2e-4, atol=2e-6)
+                np.testing.assert_allclose(gb, bt[l].grad.numpy(), rtol=2e-4, atol=2e-6)
+        opt.step()
+        np.testing.assert_allclose(m.loss, loss.item(), rtol=1e-4)
+    for l in range(nl):
+        W, b = net.get_params(l)
+        np.testing.assert_allclose(W, Wt[l].detach().numpy(), rtol=5e-4, atol=5e-6)
+        np.testing.assert_allclose(b, bt[l].detach().numpy(), rtol=5e-4, atol=5e-6)
+    # and the flags are not ignored: the same batch without them gives another output
+    assert np.abs(net.forward(Xs[0], drops[0]) - net.forward(Xs[0])).max() > 1e-3
+
+
 def test_l1_term_and_ragged_batch():
     """wd1 adds wd1*sign(W) to the gradient; a batch of 1 and a batch that is not a multiple
     of the internal row block give the same per-row forward."""
@@ -121,6 +182,15 @@ def test_forward_equals_exact_mode_forward():
         ca.set_params(l, Ws[l], np.full(sizes[l + 1], sb[l], np.float32))
     _, preds = ex.epoch(X, Y, train=False)
     assert bits_equal(ca.forward(X), preds)
+    # with the reference's dropout flags (pinned on the exact side against the reference's compiled Layer methods): a
+    # dropped node feeds nothing on in either statement, so the outputs are the same bits.  Summation order differs
+    # where an input is skipped rather than multiplied by 0: adding +-0 changes no float, so neither do the sums.
+    masks = (rng.random((21, sum(sizes[:-1]))) < 0.35).astype(np.uint8)
+    for l0, n in zip(np.concatenate([[0], np.cumsum(sizes[:-2])]), sizes[:-1]):
+        masks[:, l0] = 0                                   # no row drops a whole layer (the reference redraws those)
+    _, preds = ex.epoch(X, Y, train=False, masks=masks)
+    assert bits_equal(ca.forward(X, masks), preds)
+    assert not bits_equal(ca.forward(X), preds)
 
 
 def test_cfg3_schedule_two_summation_orders_part_ways():
